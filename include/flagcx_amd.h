@@ -1,0 +1,287 @@
+/*
+ * flagcx_amd.h - C ABI of the MI355X (gfx950) local reduce / chunk copy library.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers and sizes, allocates
+ * nothing, never calls hipSetDevice, and enqueues its work asynchronously on the
+ * caller's stream.  Return values are flagcxResult_t numbers.
+ *
+ * Conventions shared by all entry points
+ *   - "sendbuffs" is a HOST array of `nranks` DEVICE pointers: buffer j holds what
+ *     simulated rank j contributes.  The array is read during the call only.
+ *   - stream is the reference's opaque handle (flagcx/include/flagcx.h:112); on AMD
+ *     it points at a struct whose first member is the hipStream_t
+ *     (flagcx/adaptor/include/amd_adaptor.h:14-16).  NULL selects the legacy default
+ *     stream and the call blocks until the work has finished, like the reference's
+ *     hipAdaptorDeviceMemcpy / Memset (flagcx/adaptor/device/hip_adaptor.cc:16-41).
+ *   - recvbuff may be the same address as one sendbuff (element i is read before
+ *     element i is written); any other overlap is flagcxInvalidArgument.
+ *   - buffers need only be aligned to the element size (byte aligned for copies).
+ *   - count == 0 / size == 0 is flagcxSuccess and launches nothing.
+ */
+#ifndef FLAGCX_AMD_H_
+#define FLAGCX_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------- */
+/* Enums: numeric values are ABI and equal flagcx/include/flagcx.h:12-57,78-88 */
+/* If the reference's own flagcx.h was included first, its definitions are    */
+/* used and these are skipped.                                                */
+/* ------------------------------------------------------------------------- */
+#ifndef FLAGCX_H_
+
+typedef enum {
+  flagcxSuccess = 0,
+  flagcxUnhandledDeviceError = 1,
+  flagcxSystemError = 2,
+  flagcxInternalError = 3,
+  flagcxInvalidArgument = 4,
+  flagcxInvalidUsage = 5,
+  flagcxRemoteError = 6,
+  flagcxInProgress = 7,
+  flagcxUnhandledCCLError = 8,
+  flagcxNotSupported = 9,
+  flagcxNumResults = 10
+} flagcxResult_t;
+
+typedef enum {
+  flagcxInt8 = 0, flagcxChar = 0,
+  flagcxUint8 = 1,
+  flagcxInt32 = 2, flagcxInt = 2,
+  flagcxUint32 = 3,
+  flagcxInt64 = 4,
+  flagcxUint64 = 5,
+  flagcxFloat16 = 6, flagcxHalf = 6,
+  flagcxFloat32 = 7, flagcxFloat = 7,
+  flagcxFloat64 = 8, flagcxDouble = 8,
+  flagcxBfloat16 = 9,
+  flagcxNumTypes = 10
+} flagcxDataType_t;
+
+typedef enum {
+  flagcxSum = 0,
+  flagcxProd = 1,
+  flagcxMax = 2,
+  flagcxMin = 3,
+  flagcxAvg = 4,
+  flagcxRedNoOp = 5,
+  flagcxNumRedOps = 5
+} flagcxRedOp_t;
+
+typedef enum {
+  flagcxCommOpSend = 0,
+  flagcxCommOpRecv = 1,
+  flagcxCommOpBroadcast = 2,
+  flagcxCommOpGather = 3,
+  flagcxCommOpScatter = 4,
+  flagcxCommOpReduce = 5,
+  flagcxCommOpAllReduce = 6,
+  flagcxCommOpAllGather = 7,
+  flagcxCommOpReduceScatter = 8,
+  flagcxCommOpAlltoAll = 9,
+  flagcxCommOpAlltoAllv = 10,
+  flagcxCommNoOp = 11,
+  flagcxNumCommOps = 12
+} flagcxCommOp_t;
+
+typedef enum {
+  flagcxMemcpyHostToDevice = 0,
+  flagcxMemcpyDeviceToHost = 1,
+  flagcxMemcpyDeviceToDevice = 2
+} flagcxMemcpyType_t;
+
+/* Opaque in the reference (flagcx.h:112); layout fixed by amd_adaptor.h:14-16. */
+typedef struct flagcxStream *flagcxStream_t;
+
+#endif /* FLAGCX_H_ */
+
+/* Bytes per element, 0 for an unknown enum value: the table of
+ * getFlagcxDataTypeSize (flagcx/flagcx.cc:30-61) under a name that does not clash
+ * with the reference's own export when both libraries are loaded. */
+size_t flagcxLocalGetDataTypeSize(flagcxDataType_t dtype);
+
+/* Largest number of simulated ranks (input buffers) one call accepts. */
+#define FLAGCX_LOCAL_MAX_RANKS 64
+
+/* Pipeline constants of the reference's staging rings:
+ * flagcx/core/p2p.h:11-15 and flagcx/core/net.h:19-22. */
+#define FLAGCX_LOCAL_CHUNKSIZE (4ULL * 1024 * 1024)
+#define FLAGCX_LOCAL_STEPS 16
+
+/* ------------------------------------------------------------------------- */
+/* Library                                                                    */
+/* ------------------------------------------------------------------------- */
+
+/* Caches the properties of the current device (CU count).  Optional: every
+ * entry point does this on first use.  Thread-safe. */
+flagcxResult_t flagcxLocalInit(void);
+
+/* Static string for a result code (never NULL). */
+const char *flagcxLocalGetErrorString(flagcxResult_t result);
+
+/* Text of the last failure seen by the calling thread ("" if none). */
+const char *flagcxLocalGetLastError(void);
+
+/* ------------------------------------------------------------------------- */
+/* N-way elementwise reduction                                                */
+/* ------------------------------------------------------------------------- */
+
+/* recvbuff[i] = fold over j of sendbuffs[j][i], i in [0,count).
+ *
+ * The fold is the one the reference's host ring performs: acc = sendbuffs[0][i];
+ * then for j = 1..nranks-1: acc = OP(sendbuffs[j][i], acc), where OP(a,b) is
+ *   sum  a + b            (flagcx/service/utils.h:681-689)
+ *   min  (b < a) ? b : a  (std::min(a,b), utils.h:691-699)
+ *   max  (a < b) ? b : a  (std::max(a,b), utils.h:701-709)
+ *   prod a * b, avg = sum then one division by nranks (the reference's host path
+ *        rejects both, flagcx/service/bootstrap.cc:668-670; they exist here because
+ *        the reduce-op enum carries them).
+ * The call site replaced is `GENERATE_ALL_TYPES(datatype, sum, data_for_recv,
+ * sendbuff + offset, data_for_recv, n)` (bootstrap.cc:649-671), i.e. op1 = the new
+ * local input, op2 = the running partial, and on the device the vendor-CCL reduce
+ * of flagcxC2cHomoFunc::run (flagcx/core/c2c_algo.cc:310-336).
+ *
+ * Integer sum/prod wrap modulo 2^bits.  fp16/bf16 sum, prod and avg accumulate in
+ * fp32 and round to nearest even once; their min/max compare the widened values
+ * and return the selected input bit pattern unchanged.  fp32/fp64 use their own
+ * precision with no contraction or reassociation.  nranks == 1 is a copy
+ * (bootstrap.cc:816-821).
+ *
+ * Errors: flagcxInvalidArgument for a NULL pointer, nranks outside
+ * [1, FLAGCX_LOCAL_MAX_RANKS], an unknown datatype or op, a misaligned pointer or a
+ * partial overlap; flagcxUnhandledDeviceError if the launch fails. */
+flagcxResult_t flagcxLocalReduce(const void *const *sendbuffs, int nranks,
+                                 void *recvbuff, size_t count,
+                                 flagcxDataType_t datatype, flagcxRedOp_t op,
+                                 flagcxStream_t stream);
+
+/* What simulated rank `rank` ends with after the reference's ring reduce-scatter
+ * with equal blocks (ReduceScatterBootstrap, flagcx/service/bootstrap.cc:848-874;
+ * adaptor slot flagcxCCLAdaptor::reduceScatter, flagcx/adaptor/include/adaptor.h:118-121):
+ * recvbuff[i] = fold of sendbuffs[r][rank*recvcount + i] taken in the ring's order
+ * r = rank+1, rank+2, ..., rank (mod nranks) (bootstrap.cc:597-598,651-653).
+ * recvbuff may equal sendbuffs[rank] + rank*recvcount (in place, flagcx.h:356). */
+flagcxResult_t flagcxLocalReduceScatter(const void *const *sendbuffs, int nranks,
+                                        int rank, void *recvbuff,
+                                        size_t recvcount,
+                                        flagcxDataType_t datatype,
+                                        flagcxRedOp_t op, flagcxStream_t stream);
+
+/* The same result produced chunk by chunk, the way the staging ring hands data
+ * over (4 MiB steps, flagcx/core/p2p.cc:81-94): one launch per `chunkbytes` of
+ * output.  chunkbytes == 0 selects FLAGCX_LOCAL_CHUNKSIZE; it must be a multiple of
+ * the element size. */
+flagcxResult_t flagcxLocalReduceScatterChunked(const void *const *sendbuffs,
+                                               int nranks, int rank,
+                                               void *recvbuff, size_t recvcount,
+                                               flagcxDataType_t datatype,
+                                               flagcxRedOp_t op,
+                                               size_t chunkbytes,
+                                               flagcxStream_t stream);
+
+/* What every rank ends with after the reference's host ring all-reduce
+ * (AllReduceBootstrap, flagcx/service/bootstrap.cc:810-827): the buffer is cut by
+ * the chunk table of bootstrapRingAllReduce (bootstrap.cc:692-738) and chunk c is
+ * folded in the order c+1, ..., c (mod nranks).  One recvbuff, since all ranks hold
+ * the same bytes after the all-gather half.  recvbuff may equal one sendbuff. */
+flagcxResult_t flagcxLocalAllReduce(const void *const *sendbuffs, int nranks,
+                                    void *recvbuff, size_t count,
+                                    flagcxDataType_t datatype, flagcxRedOp_t op,
+                                    flagcxStream_t stream);
+
+/* The chunk table itself (bootstrap.cc:692-738): offsets[i], lengths[i] in bytes
+ * for i in [0,nranks).  Host-only. */
+flagcxResult_t flagcxLocalRingChunkTable(size_t count, flagcxDataType_t datatype,
+                                         int nranks, size_t *offsets,
+                                         size_t *lengths);
+
+/* ------------------------------------------------------------------------- */
+/* Chunk copy / zero-fill / pack / unpack                                      */
+/* ------------------------------------------------------------------------- */
+
+/* Device-to-device byte copy on the stream; replaces the deviceMemcpy(D2D) of
+ * the staging loops (flagcx/core/p2p.cc:86-89,182-185,245-247;
+ * flagcx/core/net.cc:153-161,298-306; hip_adaptor.cc:16-29).  Buffers must not
+ * overlap unless dst == src. */
+flagcxResult_t flagcxLocalMemcpy(void *dst, const void *src, size_t size,
+                                 flagcxStream_t stream);
+
+/* Byte fill; replaces deviceMemset (hip_adaptor.cc:31-41). */
+flagcxResult_t flagcxLocalMemset(void *ptr, int value, size_t size,
+                                 flagcxStream_t stream);
+
+/* flagcxC2cRefreshFunc::run (flagcx/core/c2c_algo.cc:586-608) in one launch: when
+ * op == flagcxSum, zero elements [start, start+offset) and
+ * [start+offset+count, start+totalcount) of buff and leave [start+offset,
+ * start+offset+count) alone; any other op does nothing.  offset+count >
+ * totalcount is flagcxInvalidArgument. */
+flagcxResult_t flagcxLocalRefresh(void *buff, size_t start, size_t offset,
+                                  size_t count, size_t totalcount,
+                                  flagcxDataType_t datatype, flagcxRedOp_t op,
+                                  flagcxStream_t stream);
+
+/* Strided gather: dst[c*chunkbytes + b] = src[c*srcstride + b] for c in
+ * [0,nchunks), b in [0,chunkbytes); srcstride >= chunkbytes.  Rank r's chunk at
+ * buffer + r*stride is the addressing of flagcx/adaptor/ccl/rccl_adaptor.cc:103-159. */
+flagcxResult_t flagcxLocalPack(void *dst, const void *src, size_t nchunks,
+                               size_t chunkbytes, size_t srcstride,
+                               flagcxStream_t stream);
+
+/* Strided scatter, the inverse: dst[c*dststride + b] = src[c*chunkbytes + b].
+ * Bytes of dst between chunks are not written. */
+flagcxResult_t flagcxLocalUnpack(void *dst, const void *src, size_t nchunks,
+                                 size_t chunkbytes, size_t dststride,
+                                 flagcxStream_t stream);
+
+/* Flatten n separate device buffers of `bytes` each into one contiguous buffer
+ * (dst + j*bytes), one launch instead of the per-tensor copy_ loop of
+ * plugin/torch/flagcx/src/backend_flagcx.cpp:831-840,942-951.  srcs is a host
+ * array, n <= FLAGCX_LOCAL_MAX_RANKS. */
+flagcxResult_t flagcxLocalPackList(void *dst, const void *const *srcs, int n,
+                                   size_t bytes, flagcxStream_t stream);
+
+/* The inverse (backend_flagcx.cpp:429-445,753-769). */
+flagcxResult_t flagcxLocalUnpackList(void *const *dsts, const void *src, int n,
+                                     size_t bytes, flagcxStream_t stream);
+
+/* ------------------------------------------------------------------------- */
+/* Launcher-convention symbols                                                */
+/* ------------------------------------------------------------------------- */
+/* These have the reference's device-function shape
+ *   typedef void (*flagcxLaunchFunc_t)(flagcxStream_t, void *)
+ * (flagcx/adaptor/include/adaptor.h:15) so that loadKernelSymbol
+ * (flagcx/core/launch_kernel.cc:11-29) can dlsym them from the library named by
+ * FLAGCX_DEVICE_FUNC_PATH (flagcx/flagcx.cc:552-562) and launchDeviceFunc
+ * (hip_adaptor.cc:263-269) can call them.  They return nothing, so the result
+ * code is written into the argument block. */
+
+typedef struct {
+  const void *const *sendbuffs; /* host array of nranks device pointers */
+  void *recvbuff;
+  uint64_t count;
+  int32_t nranks;
+  int32_t datatype; /* flagcxDataType_t */
+  int32_t op;       /* flagcxRedOp_t */
+  int32_t result;   /* out: flagcxResult_t */
+} flagcxLocalReduceArgs;
+
+typedef struct {
+  void *dst;
+  const void *src;
+  uint64_t size;
+  int32_t result; /* out */
+  int32_t reserved;
+} flagcxLocalCopyArgs;
+
+void flagcxLocalReduceFunc(flagcxStream_t stream, void *args /* flagcxLocalReduceArgs* */);
+void flagcxLocalCopyFunc(flagcxStream_t stream, void *args /* flagcxLocalCopyArgs* */);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLAGCX_AMD_H_ */
