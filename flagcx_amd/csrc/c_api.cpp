@@ -1,0 +1,415 @@
+// c_api.cpp - the extern "C" boundary of libflagcx_amd.so.
+//
+// Thin by design: validate on the host exactly what the kernels and their grids
+// assume (pointers, alignment, overlap, enum ranges), resolve the stream handle,
+// launch.  No allocation, no hipSetDevice, no global mutable state beyond the
+// immutable device-property cache and the launch-shape table.
+#include "../../include/flagcx_amd.h"
+#include "launch.h"
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+namespace flagcx_amd {
+
+// ---------------------------------------------------------------- errors
+static thread_local char tlsLastError[256] = "";
+
+static flagcxResult_t fail(flagcxResult_t code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(tlsLastError, sizeof(tlsLastError), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static flagcxResult_t fromHip(int err, const char *what) {
+  if (err == (int)hipSuccess) return flagcxSuccess;
+  // any runtime error maps to one code, like DEVCHECK
+  // (flagcx/adaptor/include/amd_adaptor.h:26-31)
+  return fail(flagcxUnhandledDeviceError, "%s: %s", what, hipGetErrorString((hipError_t)err));
+}
+
+// ----------------------------------------------------------- device facts
+static DeviceInfo gInfo{256, 160 * 1024};
+static std::once_flag gInfoOnce;
+static int gInfoErr = 0;
+
+const DeviceInfo &deviceInfo() {
+  std::call_once(gInfoOnce, [] {
+    int dev = 0, cus = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess && cus > 0) gInfo.numCU = cus; else gInfoErr = (int)e;
+    gInfo.ldsPerCU = 160 * 1024; // gfx950: 160 KiB of LDS per CU
+  });
+  return gInfo;
+}
+
+// Resident one-wave workgroups per CU by number of inputs (index 0: copies).
+// Measured on MI355X with 256 MiB buffers; see the kernel header for why fewer
+// resident wavefronts stream faster.
+static std::atomic<int> gWaves[9] = {{12}, {12}, {8}, {12}, {12}, {10}, {8}, {8}, {8}};
+
+int wavesPerCUFor(int k) {
+  if (k < 0) k = 0;
+  if (k > 8) k = 8;
+  return gWaves[k].load(std::memory_order_relaxed);
+}
+void setWavesPerCU(int k, int waves) {
+  if (k >= 0 && k <= 8) gWaves[k].store(waves, std::memory_order_relaxed);
+}
+int ldsReservation(int waves) {
+  if (waves <= 0 || waves >= 32) return 0;
+  int bytes = (deviceInfo().ldsPerCU / waves) & ~511;
+  if (bytes > 64 * 1024) bytes = 64 * 1024;
+  return bytes;
+}
+
+// ------------------------------------------------------- typed launchers
+int launchReduce_0(const ReduceCall &);
+int launchReduce_1(const ReduceCall &);
+int launchReduce_2(const ReduceCall &);
+int launchReduce_3(const ReduceCall &);
+int launchReduce_4(const ReduceCall &);
+int launchReduce_5(const ReduceCall &);
+int launchReduce_6(const ReduceCall &);
+int launchReduce_7(const ReduceCall &);
+int launchReduce_8(const ReduceCall &);
+int launchReduce_9(const ReduceCall &);
+
+ReduceLauncher reduceLauncherFor(int dtype) {
+  static const ReduceLauncher table[10] = {launchReduce_0, launchReduce_1, launchReduce_2,
+                                           launchReduce_3, launchReduce_4, launchReduce_5,
+                                           launchReduce_6, launchReduce_7, launchReduce_8,
+                                           launchReduce_9};
+  return (dtype >= 0 && dtype < 10) ? table[dtype] : nullptr;
+}
+
+// ----------------------------------------------------------------- helpers
+// First member of the AMD stream wrapper is the hipStream_t
+// (flagcx/adaptor/include/amd_adaptor.h:14-16).
+static inline hipStream_t hipStreamOf(flagcxStream_t s) {
+  return s ? *reinterpret_cast<hipStream_t *>(s) : nullptr;
+}
+
+// NULL stream: blocking semantics (flagcx/adaptor/device/hip_adaptor.cc:19-20,34-35).
+static flagcxResult_t finish(flagcxStream_t s, int err, const char *what) {
+  flagcxResult_t r = fromHip(err, what);
+  if (r != flagcxSuccess) return r;
+  if (!s) return fromHip((int)hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+  return flagcxSuccess;
+}
+
+static inline bool overlaps(const void *a, const void *b, uint64_t bytes) {
+  const uintptr_t x = (uintptr_t)a, y = (uintptr_t)b;
+  return x < y + bytes && y < x + bytes;
+}
+
+// Validation + launch shared by every reduce-type entry point.  `srcs` are the
+// inputs already in fold order.
+static flagcxResult_t reduceOrdered(const void *const *srcs, int k, void *dst, uint64_t count,
+                                    int dtype, int op, hipStream_t stream, const char *who) {
+  const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
+  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, dtype);
+  if (op < 0 || op >= (int)flagcxNumRedOps)
+    return fail(flagcxInvalidArgument, "%s: unsupported reduction operation %d", who, op);
+  if (k < 1 || k > FLAGCX_LOCAL_MAX_RANKS)
+    return fail(flagcxInvalidArgument, "%s: nranks %d outside [1, %d]", who, k, FLAGCX_LOCAL_MAX_RANKS);
+  if (count == 0) return flagcxSuccess;
+  if (!dst) return fail(flagcxInvalidArgument, "%s: recvbuff is NULL", who);
+  if ((uintptr_t)dst % ts) return fail(flagcxInvalidArgument, "%s: recvbuff not aligned to %zu", who, ts);
+  if (count > (UINT64_MAX / ts)) return fail(flagcxInvalidArgument, "%s: count overflows", who);
+  const uint64_t bytes = count * ts;
+  ReduceCall c;
+  for (int j = 0; j < k; j++) {
+    const void *s = srcs[j];
+    if (!s) return fail(flagcxInvalidArgument, "%s: sendbuffs[%d] is NULL", who, j);
+    if ((uintptr_t)s % ts) return fail(flagcxInvalidArgument, "%s: sendbuffs[%d] not aligned to %zu", who, j, ts);
+    if (s != dst && overlaps(s, dst, bytes))
+      return fail(flagcxInvalidArgument, "%s: recvbuff partially overlaps sendbuffs[%d]", who, j);
+    c.src[j] = s;
+  }
+  c.dst = dst;
+  c.count = count;
+  c.k = k;
+  c.op = op;
+  c.stream = stream;
+  (void)deviceInfo();
+  return fromHip(reduceLauncherFor(dtype)(c), who);
+}
+
+static void ringChunkTable(uint64_t size, uint64_t ts, int nranks, size_t *offset, size_t *length) {
+  // flagcx/service/bootstrap.cc:692 (4 MiB floor), :719-722, :727-738
+  const uint64_t minChunk = 4ull * 1024 * 1024;
+  uint64_t chunk = (size + (uint64_t)nranks - 1) / (uint64_t)nranks;
+  if (chunk < minChunk) chunk = minChunk;
+  if (chunk % ts) chunk += ts - chunk % ts;
+  for (int i = 0; i < nranks; i++) {
+    if (chunk * (uint64_t)i >= size) {
+      offset[i] = size;
+      length[i] = 0;
+      continue;
+    }
+    offset[i] = chunk * (uint64_t)i;
+    length[i] = chunk * (uint64_t)(i + 1) >= size ? size - chunk * (uint64_t)i : chunk;
+  }
+}
+
+} // namespace flagcx_amd
+
+using namespace flagcx_amd;
+
+// Only the C ABI leaves the library; everything else is built hidden.
+#pragma GCC visibility push(default)
+extern "C" {
+
+size_t flagcxLocalGetDataTypeSize(flagcxDataType_t dtype) {
+  switch ((int)dtype) {
+    case flagcxInt8: case flagcxUint8: return 1;
+    case flagcxFloat16: case flagcxBfloat16: return 2;
+    case flagcxInt32: case flagcxUint32: case flagcxFloat: return 4;
+    case flagcxInt64: case flagcxUint64: case flagcxFloat64: return 8;
+    default: return 0;
+  }
+}
+
+flagcxResult_t flagcxLocalInit(void) {
+  (void)deviceInfo();
+  if (gInfoErr) return fromHip(gInfoErr, "flagcxLocalInit");
+  return flagcxSuccess;
+}
+
+const char *flagcxLocalGetErrorString(flagcxResult_t result) {
+  switch ((int)result) {
+    case flagcxSuccess: return "no error";
+    case flagcxUnhandledDeviceError: return "unhandled device error";
+    case flagcxSystemError: return "unhandled system error";
+    case flagcxInternalError: return "internal error";
+    case flagcxInvalidArgument: return "invalid argument";
+    case flagcxInvalidUsage: return "invalid usage";
+    case flagcxRemoteError: return "remote process exited or there was a network error";
+    case flagcxInProgress: return "operation in progress";
+    case flagcxUnhandledCCLError: return "unhandled ccl error";
+    case flagcxNotSupported: return "not supported";
+    default: return "unknown result code";
+  }
+}
+
+const char *flagcxLocalGetLastError(void) { return tlsLastError; }
+
+flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU) {
+  if (nranks < 0 || nranks > 8 || wavesPerCU < 0 || wavesPerCU > 64)
+    return fail(flagcxInvalidArgument, "flagcxLocalTune: nranks %d / wavesPerCU %d out of range", nranks, wavesPerCU);
+  setWavesPerCU(nranks, wavesPerCU);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduce(const void *const *sendbuffs, int nranks, void *recvbuff,
+                                 size_t count, flagcxDataType_t datatype, flagcxRedOp_t op,
+                                 flagcxStream_t stream) {
+  if (!sendbuffs) return fail(flagcxInvalidArgument, "flagcxLocalReduce: sendbuffs is NULL");
+  flagcxResult_t r = reduceOrdered(sendbuffs, nranks, recvbuff, count, (int)datatype, (int)op,
+                                   hipStreamOf(stream), "flagcxLocalReduce");
+  if (r != flagcxSuccess) return r;
+  return finish(stream, 0, "flagcxLocalReduce");
+}
+
+flagcxResult_t flagcxLocalReduceScatterChunked(const void *const *sendbuffs, int nranks, int rank,
+                                               void *recvbuff, size_t recvcount,
+                                               flagcxDataType_t datatype, flagcxRedOp_t op,
+                                               size_t chunkbytes, flagcxStream_t stream) {
+  const char *who = "flagcxLocalReduceScatter";
+  if (!sendbuffs) return fail(flagcxInvalidArgument, "%s: sendbuffs is NULL", who);
+  if (nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS)
+    return fail(flagcxInvalidArgument, "%s: nranks %d outside [1, %d]", who, nranks, FLAGCX_LOCAL_MAX_RANKS);
+  if (rank < 0 || rank >= nranks) return fail(flagcxInvalidArgument, "%s: rank %d outside [0, %d)", who, rank, nranks);
+  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, (int)datatype);
+  if (chunkbytes == 0) chunkbytes = recvcount * ts ? recvcount * ts : ts; // one launch
+  if (chunkbytes % ts) return fail(flagcxInvalidArgument, "%s: chunkbytes %zu not a multiple of %zu", who, chunkbytes, ts);
+  for (int j = 0; j < nranks; j++)
+    if (!sendbuffs[j]) return fail(flagcxInvalidArgument, "%s: sendbuffs[%d] is NULL", who, j);
+  // ring order: rank+1, rank+2, ..., rank (flagcx/service/bootstrap.cc:597-598,651-653)
+  const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
+  const size_t chunkElems = chunkbytes / ts;
+  hipStream_t hs = hipStreamOf(stream);
+  size_t done = 0;
+  do {
+    const size_t n = recvcount - done < chunkElems ? recvcount - done : chunkElems;
+    for (int j = 0; j < nranks; j++) {
+      const int r = (rank + 1 + j) % nranks;
+      ordered[j] = (const char *)sendbuffs[r] + ((size_t)rank * recvcount + done) * ts;
+    }
+    flagcxResult_t res = reduceOrdered(ordered, nranks, (char *)recvbuff + done * ts, n, (int)datatype,
+                                       (int)op, hs, who);
+    if (res != flagcxSuccess) return res;
+    done += n;
+  } while (done < recvcount);
+  return finish(stream, 0, who);
+}
+
+flagcxResult_t flagcxLocalReduceScatter(const void *const *sendbuffs, int nranks, int rank,
+                                        void *recvbuff, size_t recvcount, flagcxDataType_t datatype,
+                                        flagcxRedOp_t op, flagcxStream_t stream) {
+  return flagcxLocalReduceScatterChunked(sendbuffs, nranks, rank, recvbuff, recvcount, datatype, op, 0,
+                                         stream);
+}
+
+flagcxResult_t flagcxLocalRingChunkTable(size_t count, flagcxDataType_t datatype, int nranks,
+                                         size_t *offsets, size_t *lengths) {
+  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  if (!ts || nranks < 1 || !offsets || !lengths)
+    return fail(flagcxInvalidArgument, "flagcxLocalRingChunkTable: bad argument");
+  ringChunkTable((uint64_t)count * ts, ts, nranks, offsets, lengths);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalAllReduce(const void *const *sendbuffs, int nranks, void *recvbuff,
+                                    size_t count, flagcxDataType_t datatype, flagcxRedOp_t op,
+                                    flagcxStream_t stream) {
+  const char *who = "flagcxLocalAllReduce";
+  if (!sendbuffs) return fail(flagcxInvalidArgument, "%s: sendbuffs is NULL", who);
+  if (nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS)
+    return fail(flagcxInvalidArgument, "%s: nranks %d outside [1, %d]", who, nranks, FLAGCX_LOCAL_MAX_RANKS);
+  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, (int)datatype);
+  for (int j = 0; j < nranks; j++)
+    if (!sendbuffs[j]) return fail(flagcxInvalidArgument, "%s: sendbuffs[%d] is NULL", who, j);
+  size_t offset[FLAGCX_LOCAL_MAX_RANKS], length[FLAGCX_LOCAL_MAX_RANKS];
+  ringChunkTable((uint64_t)count * ts, ts, nranks, offset, length);
+  hipStream_t hs = hipStreamOf(stream);
+  const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
+  // The validation of op has to happen even when every chunk is empty.
+  if ((int)op < 0 || (int)op >= (int)flagcxNumRedOps)
+    return fail(flagcxInvalidArgument, "%s: unsupported reduction operation %d", who, (int)op);
+  for (int c = 0; c < nranks; c++) {
+    if (length[c] == 0) continue; // zero-length chunks are skipped (bootstrap.cc:599-610)
+    for (int j = 0; j < nranks; j++)
+      ordered[j] = (const char *)sendbuffs[(c + 1 + j) % nranks] + offset[c];
+    flagcxResult_t res = reduceOrdered(ordered, nranks, (char *)recvbuff + offset[c], length[c] / ts,
+                                       (int)datatype, (int)op, hs, who);
+    if (res != flagcxSuccess) return res;
+  }
+  return finish(stream, 0, who);
+}
+
+// ------------------------------------------------------------ byte movers
+
+static flagcxResult_t copy2d(const Copy2D &c, flagcxStream_t stream, const char *who) {
+  (void)deviceInfo();
+  return finish(stream, launchCopy2D(c), who);
+}
+
+flagcxResult_t flagcxLocalMemcpy(void *dst, const void *src, size_t size, flagcxStream_t stream) {
+  const char *who = "flagcxLocalMemcpy";
+  if (size == 0) return flagcxSuccess;
+  if (!dst || !src) return fail(flagcxInvalidArgument, "%s: NULL pointer", who);
+  if (dst == src) return stream ? flagcxSuccess : finish(stream, 0, who);
+  if (overlaps(dst, src, size)) return fail(flagcxInvalidArgument, "%s: buffers overlap", who);
+  Copy2D c{dst, src, 1, size, size, size, nullptr, nullptr, hipStreamOf(stream)};
+  return copy2d(c, stream, who);
+}
+
+flagcxResult_t flagcxLocalMemset(void *ptr, int value, size_t size, flagcxStream_t stream) {
+  if (size == 0) return flagcxSuccess;
+  if (!ptr) return fail(flagcxInvalidArgument, "flagcxLocalMemset: NULL pointer");
+  (void)deviceInfo();
+  return finish(stream, launchFill(ptr, size, nullptr, 0, value, hipStreamOf(stream)), "flagcxLocalMemset");
+}
+
+flagcxResult_t flagcxLocalRefresh(void *buff, size_t start, size_t offset, size_t count,
+                                  size_t totalcount, flagcxDataType_t datatype, flagcxRedOp_t op,
+                                  flagcxStream_t stream) {
+  const char *who = "flagcxLocalRefresh";
+  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, (int)datatype);
+  if (offset + count > totalcount || offset + count < offset)
+    return fail(flagcxInvalidArgument, "%s: offset %zu + count %zu exceeds totalcount %zu", who, offset, count, totalcount);
+  if (op != flagcxSum) return flagcxSuccess; // flagcx/core/c2c_algo.cc:596
+  if (totalcount == count) return flagcxSuccess;
+  if (!buff) return fail(flagcxInvalidArgument, "%s: NULL pointer", who);
+  char *base = (char *)buff + start * ts;
+  (void)deviceInfo();
+  return finish(stream,
+                launchFill(base, offset * ts, base + (offset + count) * ts,
+                           (totalcount - offset - count) * ts, 0, hipStreamOf(stream)),
+                who);
+}
+
+flagcxResult_t flagcxLocalPack(void *dst, const void *src, size_t nchunks, size_t chunkbytes,
+                               size_t srcstride, flagcxStream_t stream) {
+  const char *who = "flagcxLocalPack";
+  if (nchunks == 0 || chunkbytes == 0) return flagcxSuccess;
+  if (!dst || !src) return fail(flagcxInvalidArgument, "%s: NULL pointer", who);
+  if (srcstride < chunkbytes) return fail(flagcxInvalidArgument, "%s: srcstride %zu < chunkbytes %zu", who, srcstride, chunkbytes);
+  const size_t span = (nchunks - 1) * srcstride + chunkbytes;
+  if ((uintptr_t)dst < (uintptr_t)src + span && (uintptr_t)src < (uintptr_t)dst + nchunks * chunkbytes)
+    return fail(flagcxInvalidArgument, "%s: buffers overlap", who);
+  Copy2D c{dst, src, nchunks, chunkbytes, srcstride, chunkbytes, nullptr, nullptr, hipStreamOf(stream)};
+  return copy2d(c, stream, who);
+}
+
+flagcxResult_t flagcxLocalUnpack(void *dst, const void *src, size_t nchunks, size_t chunkbytes,
+                                 size_t dststride, flagcxStream_t stream) {
+  const char *who = "flagcxLocalUnpack";
+  if (nchunks == 0 || chunkbytes == 0) return flagcxSuccess;
+  if (!dst || !src) return fail(flagcxInvalidArgument, "%s: NULL pointer", who);
+  if (dststride < chunkbytes) return fail(flagcxInvalidArgument, "%s: dststride %zu < chunkbytes %zu", who, dststride, chunkbytes);
+  const size_t span = (nchunks - 1) * dststride + chunkbytes;
+  if ((uintptr_t)src < (uintptr_t)dst + span && (uintptr_t)dst < (uintptr_t)src + nchunks * chunkbytes)
+    return fail(flagcxInvalidArgument, "%s: buffers overlap", who);
+  Copy2D c{dst, src, nchunks, chunkbytes, chunkbytes, dststride, nullptr, nullptr, hipStreamOf(stream)};
+  return copy2d(c, stream, who);
+}
+
+flagcxResult_t flagcxLocalPackList(void *dst, const void *const *srcs, int n, size_t bytes,
+                                   flagcxStream_t stream) {
+  const char *who = "flagcxLocalPackList";
+  if (n == 0 || bytes == 0) return flagcxSuccess;
+  if (!dst || !srcs) return fail(flagcxInvalidArgument, "%s: NULL pointer", who);
+  if (n < 0 || n > FLAGCX_LOCAL_MAX_RANKS) return fail(flagcxInvalidArgument, "%s: n %d outside [0, %d]", who, n, FLAGCX_LOCAL_MAX_RANKS);
+  for (int j = 0; j < n; j++) {
+    if (!srcs[j]) return fail(flagcxInvalidArgument, "%s: srcs[%d] is NULL", who, j);
+    if ((uintptr_t)srcs[j] < (uintptr_t)dst + (size_t)n * bytes && (uintptr_t)dst < (uintptr_t)srcs[j] + bytes)
+      return fail(flagcxInvalidArgument, "%s: srcs[%d] overlaps dst", who, j);
+  }
+  Copy2D c{dst, nullptr, (uint64_t)n, bytes, 0, bytes, srcs, nullptr, hipStreamOf(stream)};
+  return copy2d(c, stream, who);
+}
+
+flagcxResult_t flagcxLocalUnpackList(void *const *dsts, const void *src, int n, size_t bytes,
+                                     flagcxStream_t stream) {
+  const char *who = "flagcxLocalUnpackList";
+  if (n == 0 || bytes == 0) return flagcxSuccess;
+  if (!dsts || !src) return fail(flagcxInvalidArgument, "%s: NULL pointer", who);
+  if (n < 0 || n > FLAGCX_LOCAL_MAX_RANKS) return fail(flagcxInvalidArgument, "%s: n %d outside [0, %d]", who, n, FLAGCX_LOCAL_MAX_RANKS);
+  for (int j = 0; j < n; j++) {
+    if (!dsts[j]) return fail(flagcxInvalidArgument, "%s: dsts[%d] is NULL", who, j);
+    if ((uintptr_t)dsts[j] < (uintptr_t)src + (size_t)n * bytes && (uintptr_t)src < (uintptr_t)dsts[j] + bytes)
+      return fail(flagcxInvalidArgument, "%s: dsts[%d] overlaps src", who, j);
+  }
+  Copy2D c{nullptr, src, (uint64_t)n, bytes, bytes, 0, nullptr, dsts, hipStreamOf(stream)};
+  return copy2d(c, stream, who);
+}
+
+// ---------------------------------------------------- launcher convention
+
+void flagcxLocalReduceFunc(flagcxStream_t stream, void *args) {
+  flagcxLocalReduceArgs *a = static_cast<flagcxLocalReduceArgs *>(args);
+  if (!a) return;
+  a->result = (int32_t)flagcxLocalReduce(a->sendbuffs, a->nranks, a->recvbuff, (size_t)a->count,
+                                         (flagcxDataType_t)a->datatype, (flagcxRedOp_t)a->op, stream);
+}
+
+void flagcxLocalCopyFunc(flagcxStream_t stream, void *args) {
+  flagcxLocalCopyArgs *a = static_cast<flagcxLocalCopyArgs *>(args);
+  if (!a) return;
+  a->result = (int32_t)flagcxLocalMemcpy(a->dst, a->src, (size_t)a->size, stream);
+}
+
+} // extern "C"
+#pragma GCC visibility pop

@@ -1,0 +1,234 @@
+// copy_kernels.hip - chunk copy, strided pack / unpack, pointer-list flatten /
+// unflatten and zero-fill kernels for gfx950.
+//
+// All movers share one shape: a workgroup is one wavefront; a lane moves one
+// 16-byte vector per instruction, so each wavefront-wide access is a coalesced
+// 1 KiB request and a tile is U consecutive KiB of one chunk.  blockIdx.y walks
+// chunks (or list entries), blockIdx.x walks tiles inside a chunk.  Buffer
+// descriptors are clipped to the tile, so ragged chunk ends need no branches.
+// Bytes that cannot be moved as 16-byte vectors (different address modulo 16 on
+// the two sides, chunk sizes or strides that are not multiples of 16) go through
+// an element path at the widest width every address shares.
+// HBM bound: 2 bytes of traffic per payload byte (1 for fills); no LDS, no MFMA.
+#include "launch.h"
+#include "reduce_device.h"
+
+namespace flagcx_amd {
+
+constexpr int kCopyUnroll = 4;
+constexpr uint64_t kMaxGridX = 1u << 24;
+constexpr uint64_t kMaxGridY = 65535;
+
+struct CopyParams {
+  const char *src;
+  char *dst;
+  uint64_t nchunks, chunkBytes, srcStride, dstStride;
+  uint64_t head; // bytes before the 16-byte body (single-chunk case only)
+  uint64_t body; // bytes in the body of each chunk
+  uint64_t tail; // bytes after the body (single-chunk case only)
+};
+
+struct ListParams {
+  const char *src[FLAGCX_MAX_RANKS];
+  char *dst[FLAGCX_MAX_RANKS];
+};
+
+// LIST: 0 both sides strided, 1 sources from a pointer list, 2 destinations from one
+template <int U, int LIST>
+__global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p, ListParams l) {
+  constexpr uint32_t kTileBytes = 64u * U * 16u;
+  const uint64_t ntiles = (p.body + kTileBytes - 1) / kTileBytes;
+  const uint32_t voff = threadIdx.x * 16u;
+  for (uint64_t c = blockIdx.y; c < p.nchunks; c += gridDim.y) {
+    const char *s = (LIST == 1 ? l.src[c] : p.src + c * p.srcStride) + p.head;
+    char *d = (LIST == 2 ? l.dst[c] : p.dst + c * p.dstStride) + p.head;
+    for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+      const uint64_t off = t * kTileBytes;
+      const uint64_t left = p.body - off;
+      const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
+      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(s + off), 0, span, kRsrcFlags);
+      __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void *)(d + off), 0, span, kRsrcFlags);
+      u32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + u * 1024u, 0, kLoadAux);
+#pragma unroll
+      for (int u = 0; u < U; u++) __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, voff + u * 1024u, 0, kStoreAux);
+    }
+  }
+  // head / tail bytes of an unaligned single chunk: fewer than 32, one lane each
+  if (blockIdx.x == gridDim.x - 1 && blockIdx.y == 0) {
+    const uint64_t edge = p.head + p.tail;
+    if (threadIdx.x < edge) {
+      const uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.body + (threadIdx.x - p.head);
+      const char *s = (LIST == 1 ? l.src[0] : p.src);
+      char *d = (LIST == 2 ? l.dst[0] : p.dst);
+      d[i] = s[i];
+    }
+  }
+}
+
+// Element path: W-byte units, chunk by chunk.
+template <typename W, int LIST>
+__global__ void __launch_bounds__(256) copyElemKernel(CopyParams p, ListParams l) {
+  const uint64_t n = p.chunkBytes / sizeof(W);
+  const uint64_t stride = (uint64_t)gridDim.x * 256;
+  for (uint64_t c = blockIdx.y; c < p.nchunks; c += gridDim.y) {
+    const W *s = (const W *)(LIST == 1 ? l.src[c] : p.src + c * p.srcStride);
+    W *d = (W *)(LIST == 2 ? l.dst[c] : p.dst + c * p.dstStride);
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) d[i] = s[i];
+  }
+}
+
+template <int LIST>
+static int launchCopyT(const CopyParams &p, const ListParams &l, bool vector, unsigned width,
+                       hipStream_t stream) {
+  const uint64_t gy = p.nchunks < kMaxGridY ? p.nchunks : kMaxGridY;
+  if (vector) {
+    constexpr uint64_t tileBytes = 64ull * kCopyUnroll * 16ull;
+    uint64_t gx = (p.body + tileBytes - 1) / tileBytes;
+    if (gx < 1) gx = 1;
+    if (gx > kMaxGridX) gx = kMaxGridX;
+    const int lds = ldsReservation(wavesPerCUFor(0));
+    copyWaveKernel<kCopyUnroll, LIST><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), lds, stream>>>(p, l);
+    return (int)hipGetLastError();
+  }
+  uint64_t gx = (p.chunkBytes / width + 255) / 256;
+  const uint64_t cap = (uint64_t)deviceInfo().numCU * 16;
+  if (gx > cap) gx = cap;
+  if (gx < 1) gx = 1;
+  const dim3 grid((unsigned)gx, (unsigned)gy);
+  switch (width) {
+    case 8: copyElemKernel<uint64_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
+    case 4: copyElemKernel<uint32_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
+    case 2: copyElemKernel<uint16_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
+    default: copyElemKernel<uint8_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
+  }
+  return (int)hipGetLastError();
+}
+
+static unsigned lowBits(uint64_t x) { return (unsigned)(x & 15u); }
+
+int launchCopy2D(const Copy2D &c) {
+  CopyParams p{};
+  ListParams l{};
+  p.src = (const char *)c.src;
+  p.dst = (char *)c.dst;
+  p.nchunks = c.nchunks;
+  p.chunkBytes = c.chunkBytes;
+  p.srcStride = c.srcStride;
+  p.dstStride = c.dstStride;
+  const int list = c.srcList ? 1 : (c.dstList ? 2 : 0);
+
+  // Collect every chunk base address modulo 16 on both sides.
+  unsigned orBits = 0;       // union of differing low bits -> common alignment
+  bool sameMis = true;       // src and dst of each chunk share (addr % 16)
+  bool allAligned = true;    // every chunk base is 16-byte aligned
+  if (list) {
+    for (uint64_t j = 0; j < c.nchunks; j++) {
+      const uint64_t s = list == 1 ? (uint64_t)c.srcList[j] : (uint64_t)c.src + j * c.srcStride;
+      const uint64_t d = list == 2 ? (uint64_t)c.dstList[j] : (uint64_t)c.dst + j * c.dstStride;
+      if (list == 1) l.src[j] = (const char *)c.srcList[j]; else l.dst[j] = (char *)c.dstList[j];
+      orBits |= lowBits(s) | lowBits(d);
+      if (lowBits(s) != lowBits(d)) sameMis = false;
+      if (lowBits(s) || lowBits(d)) allAligned = false;
+    }
+  } else {
+    const uint64_t s = (uint64_t)c.src, d = (uint64_t)c.dst;
+    orBits = lowBits(s) | lowBits(d);
+    if (c.nchunks > 1) orBits |= lowBits(c.srcStride) | lowBits(c.dstStride);
+    sameMis = lowBits(s) == lowBits(d);
+    allAligned = (orBits == 0);
+  }
+
+  bool vector;
+  if (c.nchunks == 1) {
+    // one contiguous run: peel bytes up to the next 16-byte line, then vectors
+    vector = sameMis;
+    if (vector) {
+      uint64_t head = (16u - lowBits((uint64_t)(list == 2 ? (uint64_t)l.dst[0] : (uint64_t)c.dst))) & 15u;
+      if (head > c.chunkBytes) head = c.chunkBytes;
+      p.head = head;
+      p.body = (c.chunkBytes - head) & ~15ull;
+      p.tail = c.chunkBytes - head - p.body;
+    }
+  } else {
+    vector = allAligned && (c.chunkBytes & 15u) == 0;
+    p.body = c.chunkBytes;
+  }
+  unsigned width = 1;
+  if (!vector) {
+    const unsigned bits = orBits | lowBits(c.chunkBytes);
+    width = (bits & 1u) ? 1 : (bits & 2u) ? 2 : (bits & 4u) ? 4 : 8;
+  }
+  switch (list) {
+    case 1: return launchCopyT<1>(p, l, vector, width, c.stream);
+    case 2: return launchCopyT<2>(p, l, vector, width, c.stream);
+    default: return launchCopyT<0>(p, l, vector, width, c.stream);
+  }
+}
+
+// ------------------------------------------------------------------- fills
+
+struct FillParams {
+  char *ptr[2];
+  uint64_t head[2], body[2], tail[2];
+  uint32_t pattern;
+};
+
+// Up to two byte ranges in one launch (blockIdx.y picks the range).
+template <int U>
+__global__ void __launch_bounds__(64) fillWaveKernel(FillParams p) {
+  constexpr uint32_t kTileBytes = 64u * U * 16u;
+  const int r = blockIdx.y;
+  char *base = p.ptr[r] + p.head[r];
+  const uint64_t body = p.body[r];
+  const uint64_t ntiles = (body + kTileBytes - 1) / kTileBytes;
+  const uint32_t voff = threadIdx.x * 16u;
+  const u32x4 v = {p.pattern, p.pattern, p.pattern, p.pattern};
+  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const uint64_t off = t * kTileBytes;
+    const uint64_t left = body - off;
+    const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
+    __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void *)(base + off), 0, span, kRsrcFlags);
+#pragma unroll
+    for (int u = 0; u < U; u++) __builtin_amdgcn_raw_buffer_store_b128(v, rd, voff + u * 1024u, 0, kStoreAux);
+  }
+  if (blockIdx.x == gridDim.x - 1) {
+    const uint64_t edge = p.head[r] + p.tail[r];
+    if (threadIdx.x < edge) {
+      const uint64_t i = threadIdx.x < p.head[r] ? threadIdx.x : p.head[r] + body + (threadIdx.x - p.head[r]);
+      p.ptr[r][i] = (char)(p.pattern & 0xffu);
+    }
+  }
+}
+
+int launchFill(void *p0, uint64_t n0, void *p1, uint64_t n1, int value, hipStream_t stream) {
+  FillParams p{};
+  void *ptrs[2] = {p0, p1};
+  uint64_t lens[2] = {n0, n1};
+  int nr = 0;
+  uint64_t maxBody = 0;
+  for (int r = 0; r < 2; r++) {
+    if (lens[r] == 0) continue;
+    uint64_t head = (16u - lowBits((uint64_t)ptrs[r])) & 15u;
+    if (head > lens[r]) head = lens[r];
+    p.ptr[nr] = (char *)ptrs[r];
+    p.head[nr] = head;
+    p.body[nr] = (lens[r] - head) & ~15ull;
+    p.tail[nr] = lens[r] - head - p.body[nr];
+    if (p.body[nr] > maxBody) maxBody = p.body[nr];
+    nr++;
+  }
+  if (nr == 0) return (int)hipSuccess;
+  const uint32_t b = (uint32_t)(value & 0xff);
+  p.pattern = b | (b << 8) | (b << 16) | (b << 24);
+  constexpr int U = 4;
+  constexpr uint64_t tileBytes = 64ull * U * 16ull;
+  uint64_t gx = (maxBody + tileBytes - 1) / tileBytes;
+  if (gx < 1) gx = 1;
+  if (gx > kMaxGridX) gx = kMaxGridX;
+  fillWaveKernel<U><<<dim3((unsigned)gx, (unsigned)nr), dim3(64), 0, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+} // namespace flagcx_amd

@@ -1,0 +1,287 @@
+// reduce_device.h - gfx950 device code of the N-way elementwise reduction.
+//
+// One launch folds K input buffers into one output buffer:
+//   acc = in[0][i]; for j = 1..K-1: acc = OP(in[j][i], acc); out[i] = finish(acc)
+// which is the order and the operand placement (op1 = new input, op2 = partial)
+// of the reference's host ring (flagcx/service/bootstrap.cc:651-653) over its
+// binary templates (flagcx/service/utils.h:681-709).
+//
+// Streaming layout: a workgroup is ONE wavefront (64 lanes).  A lane owns one
+// 16-byte vector per load, so a wavefront-wide load is one coalesced 1 KiB
+// request; the wavefront's tile is U consecutive KiB of every input, and all K*U
+// loads are issued, input by input, before the first use.  Loads carry the `nt`
+// cache hint (streamed once), stores go out with `sc1`.  The launch reserves LDS
+// it never touches, only to cap how many wavefronts share a CU: with K = 8 inputs
+// about 8 resident wavefronts per CU (128 KiB of loads in flight) keep HBM busy
+// while staying out of each other's DRAM pages, and measured faster than a full
+// CU or a persistent grid.  No MFMA: (K+1)*16 bytes move per lane per step against
+// a handful of VALU ops.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace flagcx_amd {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+enum : int { kSum = 0, kProd = 1, kMax = 2, kMin = 3, kAvg = 4 };
+
+// Element tags for the two 16-bit float formats (raw bit carriers).
+struct f16 { uint16_t bits; };
+struct bf16 { uint16_t bits; };
+
+#define FLAGCX_MAX_RANKS 64
+
+template <int K>
+struct ReduceParams {
+  const void *src[K];
+  void *dst;
+  uint64_t nvec;   // 16-byte vectors in the aligned body
+  uint64_t head;   // elements before the body
+  uint64_t tail;   // elements after the body
+  int32_t k;       // number of inputs actually used (== K except generic)
+};
+
+// ------------------------------------------------------------------ widen
+__device__ __forceinline__ float widen(f16 h) {
+  _Float16 v;
+  __builtin_memcpy(&v, &h.bits, 2);
+  return (float)v; // v_cvt_f32_f16: exact, subnormals kept
+}
+__device__ __forceinline__ float widen(bf16 b) {
+  return __builtin_bit_cast(float, (uint32_t)b.bits << 16);
+}
+__device__ __forceinline__ void narrow(float f, f16 &out) {
+  _Float16 v = (_Float16)f; // v_cvt_f16_f32: round to nearest even
+  __builtin_memcpy(&out.bits, &v, 2);
+}
+__device__ __forceinline__ void narrow(float f, bf16 &out) {
+  uint32_t x = __builtin_bit_cast(uint32_t, f);
+  uint32_t r = x + 0x7fffu + ((x >> 16) & 1u); // round to nearest even
+  uint32_t q = (x >> 16) | 0x40u;              // quiet NaN keeps sign and top payload
+  out.bits = (uint16_t)(((x & 0x7fffffffu) > 0x7f800000u) ? q : (r >> 16));
+}
+
+// ---------------------------------------------------------- accumulators
+// Acc<T,OP>::type is what the fold carries: fp32 for half-type arithmetic, the
+// unsigned twin for integer arithmetic (wraps instead of overflowing), T itself
+// for min/max (the selected input is returned bit for bit).
+template <typename T> struct Unsigned { typedef T type; };
+template <> struct Unsigned<int8_t> { typedef uint8_t type; };
+template <> struct Unsigned<int32_t> { typedef uint32_t type; };
+template <> struct Unsigned<int64_t> { typedef uint64_t type; };
+
+template <typename T> struct IsHalf { static constexpr bool value = false; };
+template <> struct IsHalf<f16> { static constexpr bool value = true; };
+template <> struct IsHalf<bf16> { static constexpr bool value = true; };
+
+template <typename T, int OP, bool HALF = IsHalf<T>::value, bool SEL = (OP == kMax || OP == kMin)>
+struct Fold;
+
+// min / max on ordinary types
+template <typename T, int OP>
+struct Fold<T, OP, false, true> {
+  typedef T acc_t;
+  static __device__ __forceinline__ acc_t init(T x) { return x; }
+  static __device__ __forceinline__ acc_t step(T a, acc_t b) {
+    // std::max(a,b) = (a<b)?b:a ; std::min(a,b) = (b<a)?b:a
+    return (OP == kMax) ? ((a < b) ? b : a) : ((b < a) ? b : a);
+  }
+  static __device__ __forceinline__ T fin(acc_t acc, int) { return acc; }
+};
+
+// min / max on fp16 / bf16: compare widened, keep the chosen bits
+template <typename T, int OP>
+struct Fold<T, OP, true, true> {
+  struct acc_t { T bits; float val; };
+  static __device__ __forceinline__ acc_t init(T x) { return {x, widen(x)}; }
+  static __device__ __forceinline__ acc_t step(T a, acc_t b) {
+    float av = widen(a);
+    bool take_b = (OP == kMax) ? (av < b.val) : (b.val < av);
+    return take_b ? b : acc_t{a, av};
+  }
+  static __device__ __forceinline__ T fin(acc_t acc, int) { return acc.bits; }
+};
+
+// sum / prod / avg on ordinary types
+template <typename T, int OP>
+struct Fold<T, OP, false, false> {
+  typedef typename Unsigned<T>::type acc_t;
+  static __device__ __forceinline__ acc_t init(T x) { return (acc_t)x; }
+  static __device__ __forceinline__ acc_t step(T a, acc_t b) {
+    return (OP == kProd) ? (acc_t)((acc_t)a * b) : (acc_t)((acc_t)a + b);
+  }
+  static __device__ __forceinline__ T fin(acc_t acc, int k) {
+    return (OP == kAvg) ? (T)((T)acc / (T)k) : (T)acc;
+  }
+};
+
+// sum / prod / avg on fp16 / bf16: fp32 accumulator, one rounding
+template <typename T, int OP>
+struct Fold<T, OP, true, false> {
+  typedef float acc_t;
+  static __device__ __forceinline__ acc_t init(T x) { return widen(x); }
+  static __device__ __forceinline__ acc_t step(T a, acc_t b) {
+    return (OP == kProd) ? widen(a) * b : widen(a) + b;
+  }
+  static __device__ __forceinline__ T fin(acc_t acc, int k) {
+    if (OP == kAvg) acc = acc / (float)k;
+    T out;
+    narrow(acc, out);
+    return out;
+  }
+};
+
+// --------------------------------------------------------- vector plumbing
+template <typename T>
+union Vec16 {
+  u32x4 v;
+  T e[16 / sizeof(T)];
+};
+
+template <bool NT>
+__device__ __forceinline__ u32x4 loadVec(const u32x4 *p) {
+  return NT ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool NT>
+__device__ __forceinline__ void storeVec(u32x4 *p, u32x4 v) {
+  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+}
+
+// Fold one 16-byte vector position across K registers.
+template <typename T, int OP, int K>
+__device__ __forceinline__ u32x4 foldVec(const u32x4 (&in)[K], int k) {
+  typedef Fold<T, OP> F;
+  constexpr int N = 16 / sizeof(T);
+  Vec16<T> r;
+#pragma unroll
+  for (int e = 0; e < N; e++) {
+    Vec16<T> x;
+    x.v = in[0];
+    typename F::acc_t acc = F::init(x.e[e]);
+#pragma unroll
+    for (int j = 1; j < K; j++) {
+      x.v = in[j];
+      acc = F::step(x.e[e], acc);
+    }
+    r.e[e] = F::fin(acc, k);
+  }
+  return r.v;
+}
+
+// One element, inputs addressed individually (head/tail and unaligned path).
+template <typename T, int OP>
+__device__ __forceinline__ void foldScalar(const void *const *src, int k, void *dst, uint64_t i) {
+  typedef Fold<T, OP> F;
+  typename F::acc_t acc = F::init(((const T *)src[0])[i]);
+  for (int j = 1; j < k; j++) acc = F::step(((const T *)src[j])[i], acc);
+  ((T *)dst)[i] = F::fin(acc, k);
+}
+
+// ------------------------------------------------------------------ kernels
+
+// Cache-policy bits of the buffer instructions on gfx950.
+enum : int { kAuxSc0 = 1, kAuxNt = 2, kAuxSc1 = 16 };
+constexpr int kLoadAux = kAuxNt;
+constexpr int kStoreAux = kAuxSc1;
+// Raw buffer descriptor word 3 for gfx9-family: 32-bit data format, no swizzle.
+constexpr int kRsrcFlags = 0x00020000;
+
+// Aligned body with K known at compile time; one wavefront per workgroup.
+// All pointers share the same address modulo 16; p.head elements precede the
+// first vector and p.tail follow the last.  Each tile builds buffer descriptors
+// that span exactly its own bytes, so the ragged last tile needs no branches:
+// out-of-range lanes load zeros and their stores are dropped by the hardware.
+// dst may be one of the inputs: a lane reads its positions before it writes
+// them, and no other lane touches them.
+template <typename T, int OP, int K, int U>
+__global__ void __launch_bounds__(64) reduceWaveKernel(ReduceParams<K> p) {
+  constexpr int N = 16 / sizeof(T);
+  constexpr uint32_t kTileBytes = 64u * U * 16u;
+  const uint64_t bodyBytes = p.nvec * 16;
+  const uint64_t ntiles = (bodyBytes + kTileBytes - 1) / kTileBytes;
+  const uint64_t headBytes = p.head * sizeof(T);
+  const uint32_t voff = threadIdx.x * 16u;
+
+  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const uint64_t off = t * kTileBytes;
+    const uint64_t left = bodyBytes - off;
+    const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
+    u32x4 in[U][K];
+#pragma unroll
+    for (int j = 0; j < K; j++) {
+      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+          (void *)((const char *)p.src[j] + headBytes + off), 0, span, kRsrcFlags);
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        in[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + u * 1024u, 0, kLoadAux);
+    }
+    __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((char *)p.dst + headBytes + off), 0, span, kRsrcFlags);
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in[u], K), rd, voff + u * 1024u, 0,
+                                             kStoreAux);
+  }
+  // head and tail elements (fewer than 2*N <= 32): last workgroup, one lane each
+  if (blockIdx.x == gridDim.x - 1) {
+    const uint64_t edge = p.head + p.tail;
+    if (threadIdx.x < edge) {
+      uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
+      foldScalar<T, OP>(p.src, K, p.dst, i);
+    }
+  }
+}
+
+// Aligned body, any k up to FLAGCX_MAX_RANKS: inputs are consumed in batches of
+// eight loads so that the memory pipeline stays full without k-specific code.
+template <typename T, int OP, int BLOCK, bool NT>
+__global__ void __launch_bounds__(BLOCK) reduceVecAnyKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
+  typedef Fold<T, OP> F;
+  constexpr int N = 16 / sizeof(T);
+  constexpr int B = 8;
+  const int k = p.k;
+  const uint64_t stride = (uint64_t)gridDim.x * BLOCK;
+  for (uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x; i < p.nvec; i += stride) {
+    typename F::acc_t acc[N];
+    Vec16<T> x;
+    x.v = loadVec<NT>((const u32x4 *)((const T *)p.src[0] + p.head) + i);
+#pragma unroll
+    for (int e = 0; e < N; e++) acc[e] = F::init(x.e[e]);
+    for (int j0 = 1; j0 < k; j0 += B) {
+      u32x4 in[B];
+#pragma unroll
+      for (int b = 0; b < B; b++)
+        if (j0 + b < k) in[b] = loadVec<NT>((const u32x4 *)((const T *)p.src[j0 + b] + p.head) + i);
+#pragma unroll
+      for (int b = 0; b < B; b++)
+        if (j0 + b < k) {
+          x.v = in[b];
+#pragma unroll
+          for (int e = 0; e < N; e++) acc[e] = F::step(x.e[e], acc[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < N; e++) x.e[e] = F::fin(acc[e], k);
+    storeVec<NT>((u32x4 *)((T *)p.dst + p.head) + i, x.v);
+  }
+  if (blockIdx.x == gridDim.x - 1) {
+    const uint64_t edge = p.head + p.tail;
+    if (threadIdx.x < edge) {
+      uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
+      foldScalar<T, OP>(p.src, k, p.dst, i);
+    }
+  }
+}
+
+// Pointers that do not share an address modulo 16: one element per lane per step
+// (still coalesced).  p.tail carries the element count.
+template <typename T, int OP, int BLOCK>
+__global__ void __launch_bounds__(BLOCK) reduceElemKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
+  const uint64_t stride = (uint64_t)gridDim.x * BLOCK;
+  for (uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x; i < p.tail; i += stride)
+    foldScalar<T, OP>(p.src, p.k, p.dst, i);
+}
+
+} // namespace flagcx_amd

@@ -1,0 +1,139 @@
+// reduce_kernels.hip - instantiates the N-way reduce kernels for ONE element type
+// and provides its launcher.  Compiled once per type with -DFLAGCX_DT=<enum value>
+// so the ten types build in parallel.
+#include "launch.h"
+#include "reduce_device.h"
+
+#ifndef FLAGCX_DT
+#error "compile with -DFLAGCX_DT=<flagcxDataType_t value>"
+#endif
+
+namespace flagcx_amd {
+
+#if FLAGCX_DT == 0
+typedef int8_t elem_t;
+#elif FLAGCX_DT == 1
+typedef uint8_t elem_t;
+#elif FLAGCX_DT == 2
+typedef int32_t elem_t;
+#elif FLAGCX_DT == 3
+typedef uint32_t elem_t;
+#elif FLAGCX_DT == 4
+typedef int64_t elem_t;
+#elif FLAGCX_DT == 5
+typedef uint64_t elem_t;
+#elif FLAGCX_DT == 6
+typedef f16 elem_t;
+#elif FLAGCX_DT == 7
+typedef float elem_t;
+#elif FLAGCX_DT == 8
+typedef double elem_t;
+#elif FLAGCX_DT == 9
+typedef bf16 elem_t;
+#else
+#error "unknown FLAGCX_DT"
+#endif
+
+#define FLAGCX_CAT2(a, b) a##b
+#define FLAGCX_CAT(a, b) FLAGCX_CAT2(a, b)
+
+// Unroll (KiB of each input per wavefront): measured best on MI355X.
+constexpr int unrollFor(int K) { return K <= 2 ? 4 : 2; }
+
+constexpr uint64_t kMaxGrid = 1u << 24;
+
+struct Split {
+  uint64_t head, nvec, tail;
+  bool vector;
+};
+
+// Decide between the 16-byte path and the element path.  The 16-byte path needs
+// every pointer at the same offset inside a 16-byte line.
+static Split splitFor(const ReduceCall &c) {
+  constexpr uint64_t N = 16 / sizeof(elem_t);
+  Split s{0, 0, 0, true};
+  const uintptr_t mis = (uintptr_t)c.dst & 15u;
+  for (int j = 0; j < c.k; j++)
+    if (((uintptr_t)c.src[j] & 15u) != mis) s.vector = false;
+  if (!s.vector) {
+    s.tail = c.count;
+    return s;
+  }
+  uint64_t head = ((16u - mis) & 15u) / sizeof(elem_t);
+  if (head > c.count) head = c.count;
+  s.head = head;
+  s.nvec = (c.count - head) / N;
+  s.tail = c.count - head - s.nvec * N;
+  return s;
+}
+
+template <int OP, int K>
+static int launchFixed(const ReduceCall &c, const Split &s) {
+  constexpr int U = unrollFor(K);
+  ReduceParams<K> p;
+  for (int j = 0; j < K; j++) p.src[j] = c.src[j];
+  p.dst = c.dst;
+  p.nvec = s.nvec;
+  p.head = s.head;
+  p.tail = s.tail;
+  p.k = K;
+  const uint64_t tileBytes = 64ull * U * 16ull;
+  uint64_t tiles = (s.nvec * 16 + tileBytes - 1) / tileBytes;
+  if (tiles < 1) tiles = 1;
+  if (tiles > kMaxGrid) tiles = kMaxGrid;
+  const int lds = ldsReservation(wavesPerCUFor(K));
+  reduceWaveKernel<elem_t, OP, K, U><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+template <int OP>
+static int launchAny(const ReduceCall &c, const Split &s) {
+  ReduceParams<FLAGCX_MAX_RANKS> p;
+  for (int j = 0; j < c.k; j++) p.src[j] = c.src[j];
+  for (int j = c.k; j < FLAGCX_MAX_RANKS; j++) p.src[j] = nullptr;
+  p.dst = c.dst;
+  p.nvec = s.nvec;
+  p.head = s.head;
+  p.tail = s.tail;
+  p.k = c.k;
+  constexpr int BLOCK = 256;
+  const uint64_t work = s.vector ? s.nvec : s.tail;
+  uint64_t blocks = (work + BLOCK - 1) / BLOCK;
+  const uint64_t cap = (uint64_t)deviceInfo().numCU * 32;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  if (s.vector)
+    reduceVecAnyKernel<elem_t, OP, BLOCK, true><<<dim3((unsigned)blocks), dim3(BLOCK), 0, c.stream>>>(p);
+  else
+    reduceElemKernel<elem_t, OP, BLOCK><<<dim3((unsigned)blocks), dim3(BLOCK), 0, c.stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+template <int OP>
+static int launchOp(const ReduceCall &c) {
+  const Split s = splitFor(c);
+  if (!s.vector || c.k > 8) return launchAny<OP>(c, s);
+  switch (c.k) {
+    case 1: return launchFixed<OP, 1>(c, s);
+    case 2: return launchFixed<OP, 2>(c, s);
+    case 3: return launchFixed<OP, 3>(c, s);
+    case 4: return launchFixed<OP, 4>(c, s);
+    case 5: return launchFixed<OP, 5>(c, s);
+    case 6: return launchFixed<OP, 6>(c, s);
+    case 7: return launchFixed<OP, 7>(c, s);
+    default: return launchFixed<OP, 8>(c, s);
+  }
+}
+
+int FLAGCX_CAT(launchReduce_, FLAGCX_DT)(const ReduceCall &c) {
+  switch (c.op) {
+    case kSum: return launchOp<kSum>(c);
+    case kProd: return launchOp<kProd>(c);
+    case kMax: return launchOp<kMax>(c);
+    case kMin: return launchOp<kMin>(c);
+    case kAvg: return launchOp<kAvg>(c);
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
+} // namespace flagcx_amd

@@ -1,0 +1,237 @@
+"""ctypes binding of libflagcx_amd.so (include/flagcx_amd.h).
+
+Device memory and streams come from torch; nothing here computes.  Every call
+goes through the C ABI, and a missing library is an error (ImportError-like
+RuntimeError), never a silent fallback.
+"""
+import ctypes as C
+import enum
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(HERE, "lib", "libflagcx_amd.so")
+_lib = None
+
+MAX_RANKS = 64
+CHUNKSIZE = 4 * 1024 * 1024
+
+
+class Result(enum.IntEnum):          # flagcx/include/flagcx.h:12-24
+    Success = 0
+    UnhandledDeviceError = 1
+    SystemError = 2
+    InternalError = 3
+    InvalidArgument = 4
+    InvalidUsage = 5
+    RemoteError = 6
+    InProgress = 7
+    UnhandledCCLError = 8
+    NotSupported = 9
+
+
+class DataType(enum.IntEnum):        # flagcx/include/flagcx.h:27-44
+    Int8 = 0
+    Uint8 = 1
+    Int32 = 2
+    Uint32 = 3
+    Int64 = 4
+    Uint64 = 5
+    Float16 = 6
+    Float32 = 7
+    Float64 = 8
+    Bfloat16 = 9
+
+
+class RedOp(enum.IntEnum):           # flagcx/include/flagcx.h:47-57
+    Sum = 0
+    Prod = 1
+    Max = 2
+    Min = 3
+    Avg = 4
+
+
+class FlagcxError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("flagcx result %d (%s): %s" % (code, Result(code).name if 0 <= code < 10 else "?", msg))
+        self.code = code
+
+
+class Stream(C.Structure):
+    """struct flagcxStream { hipStream_t base; } (flagcx/adaptor/include/amd_adaptor.h:14-16)"""
+    _fields_ = [("base", C.c_void_p)]
+
+
+class ReduceArgs(C.Structure):       # flagcxLocalReduceArgs
+    _fields_ = [("sendbuffs", C.POINTER(C.c_void_p)), ("recvbuff", C.c_void_p), ("count", C.c_uint64),
+                ("nranks", C.c_int32), ("datatype", C.c_int32), ("op", C.c_int32), ("result", C.c_int32)]
+
+
+class CopyArgs(C.Structure):         # flagcxLocalCopyArgs
+    _fields_ = [("dst", C.c_void_p), ("src", C.c_void_p), ("size", C.c_uint64), ("result", C.c_int32),
+                ("reserved", C.c_int32)]
+
+
+EXPORTS = [
+    "flagcxLocalGetDataTypeSize", "flagcxLocalInit", "flagcxLocalGetErrorString", "flagcxLocalGetLastError",
+    "flagcxLocalTune", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
+    "flagcxLocalAllReduce", "flagcxLocalRingChunkTable", "flagcxLocalMemcpy", "flagcxLocalMemset",
+    "flagcxLocalRefresh", "flagcxLocalPack", "flagcxLocalUnpack", "flagcxLocalPackList",
+    "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
+]
+
+
+def lib_path():
+    return _LIB_PATH
+
+
+def lib():
+    """The loaded C library; raises if it was not built (python -m flagcx_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError("%s is missing: build it with `python -m flagcx_amd.build` "
+                               "(there is no fallback implementation)" % _LIB_PATH)
+        L = C.CDLL(_LIB_PATH)
+        vp, sz, i, pp = C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)
+        sp = C.POINTER(Stream)
+        L.flagcxLocalGetDataTypeSize.restype = sz
+        L.flagcxLocalGetDataTypeSize.argtypes = [i]
+        L.flagcxLocalInit.argtypes = []
+        L.flagcxLocalGetErrorString.restype = C.c_char_p
+        L.flagcxLocalGetErrorString.argtypes = [i]
+        L.flagcxLocalGetLastError.restype = C.c_char_p
+        L.flagcxLocalTune.argtypes = [i, i]
+        L.flagcxLocalReduce.argtypes = [pp, i, vp, sz, i, i, sp]
+        L.flagcxLocalReduceScatter.argtypes = [pp, i, i, vp, sz, i, i, sp]
+        L.flagcxLocalReduceScatterChunked.argtypes = [pp, i, i, vp, sz, i, i, sz, sp]
+        L.flagcxLocalAllReduce.argtypes = [pp, i, vp, sz, i, i, sp]
+        L.flagcxLocalRingChunkTable.argtypes = [sz, i, i, C.POINTER(sz), C.POINTER(sz)]
+        L.flagcxLocalMemcpy.argtypes = [vp, vp, sz, sp]
+        L.flagcxLocalMemset.argtypes = [vp, i, sz, sp]
+        L.flagcxLocalRefresh.argtypes = [vp, sz, sz, sz, sz, i, i, sp]
+        L.flagcxLocalPack.argtypes = [vp, vp, sz, sz, sz, sp]
+        L.flagcxLocalUnpack.argtypes = [vp, vp, sz, sz, sz, sp]
+        L.flagcxLocalPackList.argtypes = [vp, pp, i, sz, sp]
+        L.flagcxLocalUnpackList.argtypes = [pp, vp, i, sz, sp]
+        L.flagcxLocalReduceFunc.restype = None
+        L.flagcxLocalReduceFunc.argtypes = [sp, C.POINTER(ReduceArgs)]
+        L.flagcxLocalCopyFunc.restype = None
+        L.flagcxLocalCopyFunc.argtypes = [sp, C.POINTER(CopyArgs)]
+        _lib = L
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        raise FlagcxError(code, lib().flagcxLocalGetLastError().decode())
+
+
+def type_size(dtype):
+    return lib().flagcxLocalGetDataTypeSize(int(dtype))
+
+
+# ---------------------------------------------------------------- torch side
+
+def _torch():
+    import torch
+    return torch
+
+
+def dtype_of(t, bits_as=None):
+    """flagcx enum for a torch tensor's dtype (uint16/uint32/uint64 carried as the
+    signed tensor type of the same width unless bits_as names the enum)."""
+    torch = _torch()
+    if bits_as is not None:
+        return DataType(bits_as)
+    m = {torch.int8: DataType.Int8, torch.uint8: DataType.Uint8, torch.int32: DataType.Int32,
+         torch.int64: DataType.Int64, torch.float16: DataType.Float16, torch.float32: DataType.Float32,
+         torch.float64: DataType.Float64, torch.bfloat16: DataType.Bfloat16}
+    return m[t.dtype]
+
+
+def current_stream():
+    """A flagcxStream wrapper around torch's current HIP stream (not owned)."""
+    torch = _torch()
+    return Stream(torch.cuda.current_stream().cuda_stream)
+
+
+def _sref(stream):
+    return C.byref(stream) if stream is not None else None
+
+
+def _ptr_array(ptrs):
+    return (C.c_void_p * len(ptrs))(*ptrs)
+
+
+def reduce(srcs, dst, op, dtype=None, count=None, stream="current"):
+    """dst = fold of srcs (torch device tensors) through flagcxLocalReduce."""
+    st = current_stream() if stream == "current" else stream
+    dt = dtype_of(dst, dtype)
+    n = dst.numel() if count is None else count
+    check(lib().flagcxLocalReduce(_ptr_array([s.data_ptr() for s in srcs]), len(srcs), dst.data_ptr(), n,
+                                  int(dt), int(op), _sref(st)))
+    return dst
+
+
+def reduce_scatter(sendbuffs, rank, recv, op, dtype=None, chunkbytes=None, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    dt = dtype_of(recv, dtype)
+    ptrs = _ptr_array([s.data_ptr() for s in sendbuffs])
+    if chunkbytes is None:
+        check(lib().flagcxLocalReduceScatter(ptrs, len(sendbuffs), rank, recv.data_ptr(), recv.numel(),
+                                             int(dt), int(op), _sref(st)))
+    else:
+        check(lib().flagcxLocalReduceScatterChunked(ptrs, len(sendbuffs), rank, recv.data_ptr(), recv.numel(),
+                                                    int(dt), int(op), chunkbytes, _sref(st)))
+    return recv
+
+
+def all_reduce(sendbuffs, recv, op, dtype=None, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    dt = dtype_of(recv, dtype)
+    check(lib().flagcxLocalAllReduce(_ptr_array([s.data_ptr() for s in sendbuffs]), len(sendbuffs),
+                                     recv.data_ptr(), recv.numel(), int(dt), int(op), _sref(st)))
+    return recv
+
+
+def ring_chunk_table(count, dtype, nranks):
+    off = (C.c_size_t * nranks)()
+    ln = (C.c_size_t * nranks)()
+    check(lib().flagcxLocalRingChunkTable(count, int(dtype), nranks, off, ln))
+    return list(off), list(ln)
+
+
+def memcpy(dst_ptr, src_ptr, size, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    check(lib().flagcxLocalMemcpy(dst_ptr, src_ptr, size, _sref(st)))
+
+
+def memset(ptr, value, size, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    check(lib().flagcxLocalMemset(ptr, value, size, _sref(st)))
+
+
+def refresh(buff, start, offset, count, totalcount, op, dtype=None, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    dt = dtype_of(buff, dtype)
+    check(lib().flagcxLocalRefresh(buff.data_ptr(), start, offset, count, totalcount, int(dt), int(op), _sref(st)))
+
+
+def pack(dst_ptr, src_ptr, nchunks, chunkbytes, srcstride, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    check(lib().flagcxLocalPack(dst_ptr, src_ptr, nchunks, chunkbytes, srcstride, _sref(st)))
+
+
+def unpack(dst_ptr, src_ptr, nchunks, chunkbytes, dststride, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    check(lib().flagcxLocalUnpack(dst_ptr, src_ptr, nchunks, chunkbytes, dststride, _sref(st)))
+
+
+def pack_list(dst_ptr, src_ptrs, nbytes, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    check(lib().flagcxLocalPackList(dst_ptr, _ptr_array(src_ptrs), len(src_ptrs), nbytes, _sref(st)))
+
+
+def unpack_list(dst_ptrs, src_ptr, nbytes, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    check(lib().flagcxLocalUnpackList(_ptr_array(dst_ptrs), src_ptr, len(dst_ptrs), nbytes, _sref(st)))

@@ -127,6 +127,12 @@ const char *flagcxLocalGetErrorString(flagcxResult_t result);
 /* Text of the last failure seen by the calling thread ("" if none). */
 const char *flagcxLocalGetLastError(void);
 
+/* Launch-shape knob, in the spirit of the reference's FLAGCX_* tuning variables:
+ * how many one-wavefront workgroups may share a CU for a reduce of `nranks`
+ * inputs (1..8; 0 selects the copy kernels).  wavesPerCU == 0 removes the cap.
+ * Process-wide; the defaults are the measured optimum on MI355X. */
+flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU);
+
 /* ------------------------------------------------------------------------- */
 /* N-way elementwise reduction                                                */
 /* ------------------------------------------------------------------------- */

@@ -1,0 +1,131 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol the
+header declares, and rejects bad arguments before touching a device."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from flagcx_amd import local
+from oracle import cpu_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "flagcx_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(flagcxLocal\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = local.lib()
+    names = declared_symbols()
+    assert len(names) >= 19
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(local.EXPORTS) == names
+
+
+def test_header_enum_values_are_the_reference_abi():
+    text = open(os.path.join(ROOT, "include", "flagcx_amd.h")).read()
+    for name, val in dict(flagcxSuccess=0, flagcxInvalidArgument=4, flagcxNotSupported=9, flagcxInt8=0,
+                          flagcxUint8=1, flagcxInt32=2, flagcxUint32=3, flagcxInt64=4, flagcxUint64=5,
+                          flagcxFloat16=6, flagcxFloat32=7, flagcxFloat64=8, flagcxBfloat16=9, flagcxSum=0,
+                          flagcxProd=1, flagcxMax=2, flagcxMin=3, flagcxAvg=4).items():
+        assert re.search(r"\b%s\s*=\s*%d\b" % (name, val), text), name
+    assert [int(d) for d in local.DataType] == list(range(10))
+    assert [int(o) for o in local.RedOp] == list(range(5))
+
+
+def test_type_sizes_match_oracle():
+    for d in range(-1, 12):
+        assert local.type_size(d) == O.type_size(d)
+
+
+def test_ring_chunk_table_matches_oracle():
+    M = 1 << 20
+    for count in (0, 1, 1000, M, 4 * M + 3, 16 * M, 33 * M + 5):
+        for dt in (O.INT8, O.FP16, O.FP32, O.FP64):
+            for n in (1, 2, 3, 8, 64):
+                ts = O.type_size(dt)
+                assert local.ring_chunk_table(count, dt, n) == tuple(O.ring_chunk_table(count * ts, ts, n))
+
+
+def _call_reduce(ptrs, n, dst, count, dt, op):
+    arr = (C.c_void_p * max(len(ptrs), 1))(*ptrs)
+    st = local.Stream(None)
+    return local.lib().flagcxLocalReduce(arr, n, dst, count, dt, op, C.byref(st))
+
+
+def test_reduce_rejects_bad_arguments_without_a_device():
+    L = local.lib()
+    a, b = 0x10000, 0x20000   # never dereferenced: validation fails first
+    inv = int(local.Result.InvalidArgument)
+    assert _call_reduce([a, a], 2, b, 16, 10, 0) == inv          # unknown dtype
+    assert b"data type" in L.flagcxLocalGetLastError()
+    assert _call_reduce([a, a], 2, b, 16, -1, 0) == inv
+    assert _call_reduce([a, a], 2, b, 16, 7, 5) == inv           # flagcxRedNoOp
+    assert b"reduction operation" in L.flagcxLocalGetLastError()
+    assert _call_reduce([a, a], 2, b, 16, 7, -1) == inv
+    assert _call_reduce([a, a], 0, b, 16, 7, 0) == inv           # nranks
+    assert _call_reduce([a] * 65, 65, b, 16, 7, 0) == inv
+    assert _call_reduce([a, 0], 2, b, 16, 7, 0) == inv           # NULL input
+    assert _call_reduce([a, a], 2, 0, 16, 7, 0) == inv           # NULL output
+    assert _call_reduce([a, a + 2], 2, b, 16, 7, 0) == inv       # misaligned for fp32
+    assert _call_reduce([a, a], 2, b + 1, 16, 4, 0) == inv       # misaligned for int64
+    assert _call_reduce([a, b - 8], 2, b, 16, 7, 0) == inv       # partial overlap
+    assert b"overlaps" in L.flagcxLocalGetLastError()
+    assert _call_reduce([a, a], 2, b, 0, 7, 0) == 0              # empty: success, nothing launched
+    st = local.Stream(None)
+    assert L.flagcxLocalReduce(None, 2, b, 16, 7, 0, C.byref(st)) == inv
+
+
+def test_other_entry_points_reject_bad_arguments():
+    L = local.lib()
+    st = C.byref(local.Stream(None))
+    inv = int(local.Result.InvalidArgument)
+    a, b = 0x10000, 0x90000
+    ptrs = (C.c_void_p * 2)(a, a + 0x1000)
+    assert L.flagcxLocalReduceScatter(ptrs, 2, 2, b, 16, 7, 0, st) == inv       # rank out of range
+    assert L.flagcxLocalReduceScatter(ptrs, 2, -1, b, 16, 7, 0, st) == inv
+    assert L.flagcxLocalReduceScatterChunked(ptrs, 2, 0, b, 16, 7, 0, 6, st) == inv  # chunk not multiple of 4
+    assert L.flagcxLocalAllReduce(ptrs, 2, b, 16, 6, 9, st) == inv
+    assert L.flagcxLocalAllReduce(ptrs, 0, b, 16, 7, 0, st) == inv
+    assert L.flagcxLocalMemcpy(a, a + 8, 16, st) == inv                         # overlap
+    assert L.flagcxLocalMemcpy(None, a, 16, st) == inv
+    assert L.flagcxLocalMemcpy(a, a, 16, st) == 0                               # same buffer: no-op
+    assert L.flagcxLocalMemset(None, 0, 16, st) == inv
+    assert L.flagcxLocalRefresh(a, 0, 8, 9, 16, 7, 0, st) == inv                # offset+count > total
+    assert L.flagcxLocalRefresh(a, 0, 0, 16, 16, 7, 0, st) == 0                 # nothing to clear
+    assert L.flagcxLocalRefresh(a, 0, 4, 4, 16, 7, 2, st) == 0                  # max: no-op (c2c_algo.cc:596)
+    assert L.flagcxLocalPack(b, a, 4, 64, 32, st) == inv                        # stride < chunk
+    assert L.flagcxLocalUnpack(b, a, 4, 64, 32, st) == inv
+    assert L.flagcxLocalPack(a + 64, a, 4, 64, 128, st) == inv                  # overlap
+    assert L.flagcxLocalPackList(b, ptrs, 65, 16, st) == inv
+    assert L.flagcxLocalPackList(a, ptrs, 2, 16, st) == inv                     # dst overlaps a source
+    assert L.flagcxLocalTune(9, 8) == inv
+    assert L.flagcxLocalTune(8, 8) == 0
+    # zero sizes succeed without a launch
+    assert L.flagcxLocalMemcpy(b, a, 0, st) == 0
+    assert L.flagcxLocalPack(b, a, 0, 64, 64, st) == 0
+
+
+def test_launcher_convention_reports_through_the_argument_block():
+    L = local.lib()
+    arr = (C.c_void_p * 2)(0x10000, 0x20000)
+    args = local.ReduceArgs(arr, 0x30000, 16, 2, 10, 0, -1)   # unknown dtype
+    st = local.Stream(None)
+    L.flagcxLocalReduceFunc(C.byref(st), C.byref(args))
+    assert args.result == int(local.Result.InvalidArgument)
+    cargs = local.CopyArgs(None, 0x10000, 16, -1, 0)
+    L.flagcxLocalCopyFunc(C.byref(st), C.byref(cargs))
+    assert cargs.result == int(local.Result.InvalidArgument)
+
+
+def test_error_strings():
+    L = local.lib()
+    for code in range(0, 11):
+        s = L.flagcxLocalGetErrorString(code)
+        assert s and isinstance(s, bytes)

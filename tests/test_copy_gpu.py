@@ -1,0 +1,128 @@
+"""GPU parity of the chunk copy / pack / unpack / fill kernels: byte-exact against
+the oracle's memcpy loops, round trips, and untouched guard bytes."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from tests.util import from_dev, same, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def L():
+    import torch
+    assert torch.cuda.is_available()
+    from flagcx_amd import local
+    assert local.lib().flagcxLocalInit() == 0
+    return local
+
+
+def rand_bytes(n, seed):
+    return np.random.default_rng(seed).integers(0, 256, n, dtype=np.uint8)
+
+
+@pytest.mark.parametrize("size", [1, 15, 16, 17, 1000, 4096, 65536 + 5, (4 << 20), (4 << 20) + 123])
+def test_memcpy_sizes_and_offsets(L, size):
+    import torch
+    src_h = rand_bytes(size + 64, size)
+    src = to_dev(src_h)
+    for so, do in ((0, 0), (1, 1), (3, 3), (0, 5), (7, 2), (4, 8), (2, 4)):
+        dst = torch.full((size + 64,), 0xAB, dtype=torch.uint8, device="cuda")
+        L.memcpy(dst.data_ptr() + do, src.data_ptr() + so, size)
+        torch.cuda.synchronize()
+        got = from_dev(dst, np.uint8)
+        assert same(got[do:do + size], src_h[so:so + size]), (so, do)
+        assert (got[:do] == 0xAB).all() and (got[do + size:] == 0xAB).all(), (so, do)
+
+
+def test_self_copy_reference_pattern(L):
+    # test/perf/test_core_sendrecv.cpp:80-94: 0xAA x 100 then 0xBB x 200, self send/recv
+    import torch
+    h = np.concatenate([np.full(100, 0xAA, np.uint8), np.full(200, 0xBB, np.uint8)])
+    src = to_dev(h)
+    dst = torch.zeros(300, dtype=torch.uint8, device="cuda")
+    args = L.CopyArgs(dst.data_ptr(), src.data_ptr(), 300, -1, 0)
+    st = L.current_stream()
+    L.lib().flagcxLocalCopyFunc(C.byref(st), C.byref(args))
+    torch.cuda.synchronize()
+    assert args.result == 0 and same(from_dev(dst, np.uint8), h)
+
+
+@pytest.mark.parametrize("size", [1, 31, 4096, 100003])
+def test_memset(L, size):
+    import torch
+    for off, val in ((0, 0), (1, 0x5A), (9, 0xFF), (16, 7)):
+        buf = torch.full((size + 64,), 0xCD, dtype=torch.uint8, device="cuda")
+        L.memset(buf.data_ptr() + off, val, size)
+        torch.cuda.synchronize()
+        got = from_dev(buf, np.uint8)
+        assert (got[off:off + size] == val).all()
+        assert (got[:off] == 0xCD).all() and (got[off + size:] == 0xCD).all()
+
+
+@pytest.mark.parametrize("tsz,dt", [(4, O.FP32), (2, O.BF16), (1, O.INT8), (8, O.FP64)])
+def test_refresh_matches_oracle(L, tsz, dt):
+    import torch
+    carrier = {1: np.uint8, 2: np.uint16, 4: np.float32, 8: np.float64}[tsz]
+    for start, offset, count, total in ((0, 0, 10, 100), (3, 20, 30, 80), (0, 90, 10, 100), (5, 0, 0, 50),
+                                        (1, 1000, 3000, 100001), (0, 7, 1, 9)):
+        n = start + total + 13
+        h = rand_bytes(n * tsz, total).view(carrier).copy()
+        for op in (O.SUM, O.MAX, O.MIN, O.PROD):
+            want = h.copy()
+            O.refresh(want, start, offset, count, total, op)
+            d = to_dev(h)
+            L.refresh(d, start, offset, count, total, op, dtype=dt)
+            torch.cuda.synchronize()
+            assert same(from_dev(d, carrier), want), (start, offset, count, total, op)
+
+
+@pytest.mark.parametrize("chunk,stride", [(64, 512), (4096, 32768), (100, 800), (48, 48), (17, 33),
+                                          (1 << 20, 8 << 20), (6, 64)])
+def test_pack_unpack_round_trip(L, chunk, stride):
+    import torch
+    nch = 8
+    span = (nch - 1) * stride + chunk
+    h = rand_bytes(span + 32, chunk + stride)
+    for base in (0, 4, 1):
+        src = to_dev(h)
+        staged = torch.full((nch * chunk + 32,), 0x77, dtype=torch.uint8, device="cuda")
+        L.pack(staged.data_ptr() + base, src.data_ptr() + base, nch, chunk, stride)
+        torch.cuda.synchronize()
+        want = O.pack(np.ascontiguousarray(h[base:]), nch, chunk, stride)
+        got = from_dev(staged, np.uint8)
+        assert same(got[base:base + nch * chunk], want), (chunk, stride, base)
+        assert (got[:base] == 0x77).all() and (got[base + nch * chunk:] == 0x77).all()
+        # scatter back into a fresh sparse buffer: chunks restored, gaps untouched
+        back = torch.full((span + 32,), 0xEE, dtype=torch.uint8, device="cuda")
+        L.unpack(back.data_ptr() + base, staged.data_ptr() + base, nch, chunk, stride)
+        torch.cuda.synchronize()
+        wantb = np.full(span + 32, 0xEE, np.uint8)
+        O.unpack(wantb[base:], want, nch, chunk, stride)
+        assert same(from_dev(back, np.uint8), wantb), (chunk, stride, base)
+
+
+@pytest.mark.parametrize("nbytes", [16, 1000, 4096, 65536 + 16, 333])
+def test_pack_list_and_unpack_list(L, nbytes):
+    import torch
+    n = 8
+    hs = [rand_bytes(nbytes + 16, 100 + j) for j in range(n)]
+    for off in (0, 3):
+        devs = [to_dev(h) for h in hs]
+        flat = torch.full((n * nbytes + 16,), 0x11, dtype=torch.uint8, device="cuda")
+        L.pack_list(flat.data_ptr() + off, [d.data_ptr() + off for d in devs], nbytes)
+        torch.cuda.synchronize()
+        got = from_dev(flat, np.uint8)
+        want = np.concatenate([h[off:off + nbytes] for h in hs])
+        assert same(got[off:off + n * nbytes], want), (nbytes, off)
+        assert (got[:off] == 0x11).all() and (got[off + n * nbytes:] == 0x11).all()
+        outs = [torch.full((nbytes + 16,), 0x22, dtype=torch.uint8, device="cuda") for _ in range(n)]
+        L.unpack_list([o.data_ptr() + off for o in outs], flat.data_ptr() + off, nbytes)
+        torch.cuda.synchronize()
+        for j in range(n):
+            g = from_dev(outs[j], np.uint8)
+            assert same(g[off:off + nbytes], hs[j][off:off + nbytes]), (nbytes, off, j)
+            assert (g[:off] == 0x22).all() and (g[off + nbytes:] == 0x22).all()

@@ -1,0 +1,243 @@
+"""GPU parity of the N-way reduce (through the C ABI) against the CPU oracle and
+the golden vectors made with the reference's own templates.
+
+Bar: bit-exact for integers, min/max and fp32/fp64 arithmetic in the stated fold
+order; for fp16/bf16 sum/prod/avg and for avg the stated tolerance is 1 ulp of the
+output type - the tests below demand equality with the oracle, which is stricter.
+The only relaxation: where an arithmetic result is NaN, any NaN payload is accepted.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from tests.util import (ALL_DTYPES, ALL_OPS, DT_NAME, OP_NAME, dev_empty, from_dev, is_float,
+                        make_inputs, same, to_dev)
+
+pytestmark = pytest.mark.gpu
+
+GOLD_NAMES = {O.INT8: "i8", O.UINT8: "u8", O.INT32: "i32", O.UINT32: "u32", O.INT64: "i64",
+              O.UINT64: "u64", O.FP32: "f32", O.FP64: "f64"}
+GOLD_OPS = {O.SUM: "sum", O.MAX: "max", O.MIN: "min"}
+
+
+@pytest.fixture(scope="module")
+def L():
+    import torch
+    assert torch.cuda.is_available()
+    from flagcx_amd import local
+    assert local.lib().flagcxLocalInit() == 0
+    return local
+
+
+def gpu_reduce(L, srcs_np, dtype, op, dst_fill=None):
+    import torch
+    devs = [to_dev(s) for s in srcs_np]
+    out = dev_empty(srcs_np[0].size, srcs_np[0].dtype.itemsize, fill=dst_fill)
+    L.reduce(devs, out, op, dtype=dtype)
+    torch.cuda.synchronize()
+    return from_dev(out, srcs_np[0].dtype)
+
+
+def arith_nan_ok(dtype, op):
+    return is_float(dtype) and op in (O.SUM, O.PROD, O.AVG)
+
+
+# ------------------------------------------------------------------ golden
+
+@pytest.mark.parametrize("dt", list(GOLD_NAMES), ids=lambda d: DT_NAME[d])
+@pytest.mark.parametrize("op", list(GOLD_OPS), ids=lambda o: OP_NAME[o])
+def test_reduce_matches_reference_golden(L, golden, dt, op):
+    nm, on = GOLD_NAMES[dt], GOLD_OPS[op]
+    signed = np.dtype(O.NP_OF[dt]).kind == "i"
+    src = golden[f"in_safe_{nm}"] if (signed and op == O.SUM) else golden[f"in_full_{nm}"]
+    for k in (2, 3, 8):
+        got = gpu_reduce(L, [np.ascontiguousarray(src[j]) for j in range(k)], dt, op)
+        assert same(got, golden[f"fold_{nm}_{on}_k{k}"], nan_class=arith_nan_ok(dt, op), dtype=dt), (nm, on, k)
+
+
+@pytest.mark.parametrize("dt", list(GOLD_NAMES), ids=lambda d: DT_NAME[d])
+@pytest.mark.parametrize("op", list(GOLD_OPS), ids=lambda o: OP_NAME[o])
+def test_reduce_scatter_matches_reference_golden(L, golden, dt, op):
+    import torch
+    nm, on = GOLD_NAMES[dt], GOLD_OPS[op]
+    signed = np.dtype(O.NP_OF[dt]).kind == "i"
+    src = golden[f"in_safe_{nm}"] if (signed and op == O.SUM) else golden[f"in_full_{nm}"]
+    nr, rcount = 4, 129
+    send = [to_dev(np.ascontiguousarray(src[r, :nr * rcount])) for r in range(nr)]
+    for rank in range(nr):
+        out = dev_empty(rcount, src.dtype.itemsize)
+        L.reduce_scatter(send, rank, out, op, dtype=dt)
+        torch.cuda.synchronize()
+        assert same(from_dev(out, src.dtype), golden[f"ringrs_{nm}_{on}_r{rank}"],
+                    nan_class=arith_nan_ok(dt, op), dtype=dt), (nm, on, rank)
+
+
+# ------------------------------------------------------- oracle, all types
+
+@pytest.mark.parametrize("dt", ALL_DTYPES, ids=lambda d: DT_NAME[d])
+@pytest.mark.parametrize("op", ALL_OPS, ids=lambda o: OP_NAME[o])
+def test_reduce_matches_oracle_all_types(L, dt, op):
+    # sizes straddle the vector width, one wavefront tile and several tiles
+    for k, n in ((1, 5), (2, 1), (2, 4096 + 3), (3, 1000), (4, 70001), (5, 33), (8, 262144 + 17),
+                 (9, 5000), (16, 12345), (64, 777)):
+        srcs = make_inputs(dt, k, n, seed=1000 * dt + 10 * op + k, op=op)
+        rc, want = O.reduce(srcs, dt, op)
+        assert rc == 0
+        got = gpu_reduce(L, srcs, dt, op)
+        assert same(got, want, nan_class=arith_nan_ok(dt, op), dtype=dt), (DT_NAME[dt], OP_NAME[op], k, n)
+
+
+@pytest.mark.parametrize("dt", [O.FP16, O.BF16, O.FP32], ids=lambda d: DT_NAME[d])
+def test_float_special_values(L, dt):
+    # every ordered pair of specials, folded with k = 2 and k = 3
+    if dt == O.FP32:
+        sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.17549435e-38, 3.4028235e38,
+                       -3.4028235e38, 1.0, -1.0, 1.0000001, 3.0, 1e-40, 16777216.0], dtype=np.float32)
+    elif dt == O.FP16:
+        sp = np.array([0x0000, 0x8000, 0x7c00, 0xfc00, 0x7e00, 0x0001, 0x8001, 0x0400, 0x7bff, 0xfbff,
+                       0x3c00, 0xbc00, 0x3c01, 0x4200, 0x03ff, 0x6800], dtype=np.uint16).view(np.float16)
+    else:
+        sp = np.array([0x0000, 0x8000, 0x7f80, 0xff80, 0x7fc0, 0x0001, 0x8001, 0x0080, 0x7f7f, 0xff7f,
+                       0x3f80, 0xbf80, 0x3f81, 0x4040, 0x007f, 0x4b80], dtype=np.uint16)
+    m = len(sp)
+    a = np.repeat(sp, m)
+    b = np.tile(sp, m)
+    c = np.roll(b, 5)
+    for op in ALL_OPS:
+        for srcs in ([a, b], [a, b, c], [c, a, b, a]):
+            srcs = [np.ascontiguousarray(s) for s in srcs]
+            rc, want = O.reduce(srcs, dt, op)
+            got = gpu_reduce(L, srcs, dt, op)
+            assert same(got, want, nan_class=arith_nan_ok(dt, op), dtype=dt), (DT_NAME[dt], OP_NAME[op], len(srcs))
+
+
+def test_reference_pattern_i_mod_10(L):
+    # test/unittest/main.cpp:23-48: every rank holds i % 10, sum = nranks * (i % 10)
+    n, k = 1 << 20, 8
+    x = (np.arange(n) % 10).astype(np.float32)
+    got = gpu_reduce(L, [x] * k, O.FP32, O.SUM)
+    assert np.array_equal(got, k * x)
+    got = gpu_reduce(L, [x] * k, O.FP32, O.AVG)
+    assert np.array_equal(got, x)
+
+
+# ------------------------------------------------------ alignment, aliasing
+
+@pytest.mark.parametrize("dt", [O.INT8, O.BF16, O.FP32, O.FP64], ids=lambda d: DT_NAME[d])
+def test_unaligned_and_mixed_offsets(L, dt):
+    import torch
+    ts = O.type_size(dt)
+    n, k = 10007, 3
+    srcs = make_inputs(dt, k, n + 64, seed=77 + dt)
+    devs = [to_dev(s) for s in srcs]
+    for offs, doff in (((1, 1, 1), 1), ((3, 3, 3), 3), ((0, 1, 2), 0), ((5, 5, 5), 2), ((0, 0, 0), 7)):
+        out = dev_empty(n + 64, ts, fill=0x55 if ts == 1 else 0x5555)
+        guard = from_dev(out, srcs[0].dtype).copy()
+        views = [d[o:o + n] for d, o in zip(devs, offs)]
+        L.reduce(views, out[doff:doff + n], O.SUM, dtype=dt)
+        torch.cuda.synchronize()
+        rc, want = O.reduce([np.ascontiguousarray(s[o:o + n]) for s, o in zip(srcs, offs)], dt, O.SUM)
+        got = from_dev(out, srcs[0].dtype)
+        assert same(got[doff:doff + n], want, nan_class=is_float(dt), dtype=dt), (offs, doff)
+        # nothing outside the destination range was written
+        assert same(got[:doff], guard[:doff]) and same(got[doff + n:], guard[doff + n:]), (offs, doff)
+
+
+@pytest.mark.parametrize("dt", [O.FP32, O.BF16, O.INT32], ids=lambda d: DT_NAME[d])
+def test_in_place_on_any_input(L, dt):
+    import torch
+    k, n = 4, 50001
+    srcs = make_inputs(dt, k, n, seed=5 + dt)
+    rc, want = O.reduce(srcs, dt, O.SUM)
+    for j in range(k):
+        devs = [to_dev(s) for s in srcs]
+        L.reduce(devs, devs[j], O.SUM, dtype=dt)
+        torch.cuda.synchronize()
+        assert same(from_dev(devs[j], srcs[0].dtype), want, nan_class=is_float(dt), dtype=dt), j
+
+
+def test_null_stream_blocks_and_launcher_symbol(L):
+    import torch
+    srcs = make_inputs(O.FP32, 2, 4097, seed=3)
+    rc, want = O.reduce(srcs, O.FP32, O.SUM)
+    devs = [to_dev(s) for s in srcs]
+    out = dev_empty(4097, 4)
+    torch.cuda.synchronize()
+    L.reduce(devs, out, O.SUM, dtype=O.FP32, stream=None)  # NULL: returns after completion
+    assert same(from_dev(out, np.float32), want)
+    # the launcher-convention entry: void fn(flagcxStream_t, void *args)
+    out2 = dev_empty(4097, 4)
+    arr = (C.c_void_p * 2)(devs[0].data_ptr(), devs[1].data_ptr())
+    args = L.ReduceArgs(arr, out2.data_ptr(), 4097, 2, O.FP32, O.SUM, -1)
+    st = L.current_stream()
+    L.lib().flagcxLocalReduceFunc(C.byref(st), C.byref(args))
+    torch.cuda.synchronize()
+    assert args.result == 0 and same(from_dev(out2, np.float32), want)
+
+
+# --------------------------------------------------------------- ring forms
+
+@pytest.mark.parametrize("dt,op", [(O.FP32, O.SUM), (O.INT32, O.MAX), (O.FP64, O.MIN), (O.BF16, O.SUM),
+                                   (O.FP16, O.AVG), (O.FP32, O.PROD)],
+                         ids=lambda v: str(v))
+def test_all_reduce_matches_ring_oracle(L, dt, op):
+    import torch
+    strict = dt in O.REF_DTYPES and op in O.REF_OPS
+    ts = O.type_size(dt)
+    for nranks, n in ((2, 1000), (3, (9 << 20) // ts + 5), (8, (5 << 20) // ts + 1), (1, 333)):
+        send = make_inputs(dt, nranks, n, seed=nranks * 7 + dt, op=op)
+        rc, want = O.ring_allreduce(send, dt, op, strict=strict)
+        assert rc == 0
+        devs = [to_dev(s) for s in send]
+        out = dev_empty(n, ts)
+        L.all_reduce(devs, out, op, dtype=dt)
+        torch.cuda.synchronize()
+        assert same(from_dev(out, send[0].dtype), want, nan_class=arith_nan_ok(dt, op), dtype=dt), (nranks, n)
+    # in place on rank 1's buffer
+    send = make_inputs(dt, 3, 4099, seed=1, op=op)
+    rc, want = O.ring_allreduce(send, dt, op, strict=strict)
+    devs = [to_dev(s) for s in send]
+    L.all_reduce(devs, devs[1], op, dtype=dt)
+    torch.cuda.synchronize()
+    assert same(from_dev(devs[1], send[0].dtype), want, nan_class=arith_nan_ok(dt, op), dtype=dt)
+
+
+@pytest.mark.parametrize("dt,op", [(O.FP32, O.SUM), (O.FP16, O.AVG), (O.INT64, O.MIN)], ids=lambda v: str(v))
+def test_reduce_scatter_and_chunked_match_oracle(L, dt, op):
+    import torch
+    strict = dt in O.REF_DTYPES and op in O.REF_OPS
+    ts = O.type_size(dt)
+    nranks, rcount = 8, 30011
+    send = make_inputs(dt, nranks, nranks * rcount, seed=21 + dt, op=op)
+    devs = [to_dev(s) for s in send]
+    for rank in (0, 3, 7):
+        rc, want = O.reduce_scatter_rank(send, rank, rcount, dt, op, strict=strict)
+        assert rc == 0
+        out = dev_empty(rcount, ts)
+        L.reduce_scatter(devs, rank, out, op, dtype=dt)
+        out2 = dev_empty(rcount, ts)
+        L.reduce_scatter(devs, rank, out2, op, dtype=dt, chunkbytes=4096 * ts)
+        torch.cuda.synchronize()
+        assert same(from_dev(out, send[0].dtype), want, nan_class=arith_nan_ok(dt, op), dtype=dt), rank
+        assert same(from_dev(out2, send[0].dtype), want, nan_class=arith_nan_ok(dt, op), dtype=dt), rank
+    # in place: recvbuff == sendbuffs[rank] + rank*recvcount (flagcx.h:356)
+    rank = 2
+    rc, want = O.reduce_scatter_rank(send, rank, rcount, dt, op, strict=strict)
+    L.reduce_scatter(devs, rank, devs[rank][rank * rcount:(rank + 1) * rcount], op, dtype=dt)
+    torch.cuda.synchronize()
+    got = from_dev(devs[rank], send[0].dtype)[rank * rcount:(rank + 1) * rcount]
+    assert same(got, want, nan_class=arith_nan_ok(dt, op), dtype=dt)
+
+
+def test_reduce_scatter_reference_pattern(L):
+    # test/perf/test_reducescatter.cpp:86-97: value floor(i / recvcount) -> shard r = nranks * r
+    import torch
+    k, rcount = 8, 4096
+    x = to_dev((np.arange(k * rcount) // rcount).astype(np.float32))
+    for rank in range(k):
+        out = dev_empty(rcount, 4)
+        L.reduce_scatter([x] * k, rank, out, O.SUM, dtype=O.FP32)
+        torch.cuda.synchronize()
+        assert np.array_equal(from_dev(out, np.float32), np.full(rcount, k * rank, np.float32))
