@@ -49,10 +49,10 @@ const DeviceInfo &deviceInfo() {
   return gInfo;
 }
 
-// Resident one-wave workgroups per CU by number of inputs (index 0: copies).
-// Measured on MI355X with 256 MiB buffers; see the kernel header for why fewer
-// resident wavefronts stream faster.
-static std::atomic<int> gWaves[9] = {{12}, {12}, {8}, {12}, {12}, {10}, {8}, {8}, {8}};
+// Resident one-wave workgroups per CU by number of inputs (index 0: copies;
+// 0 = no cap).  Measured on MI355X with HBM-resident buffers; see the kernel
+// header for why fewer resident wavefronts stream faster as inputs multiply.
+static std::atomic<int> gWaves[9] = {{0}, {0}, {24}, {24}, {16}, {10}, {8}, {8}, {8}};
 
 int wavesPerCUFor(int k) {
   if (k < 0) k = 0;

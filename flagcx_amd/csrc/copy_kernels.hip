@@ -15,7 +15,7 @@
 
 namespace flagcx_amd {
 
-constexpr int kCopyUnroll = 4;
+constexpr int kCopyUnroll = 1;
 constexpr uint64_t kMaxGridX = 1u << 24;
 constexpr uint64_t kMaxGridY = 65535;
 

@@ -14,8 +14,8 @@
 // it never touches, only to cap how many wavefronts share a CU: with K = 8 inputs
 // about 8 resident wavefronts per CU (128 KiB of loads in flight) keep HBM busy
 // while staying out of each other's DRAM pages, and measured faster than a full
-// CU or a persistent grid.  No MFMA: (K+1)*16 bytes move per lane per step against
-// a handful of VALU ops.
+// CU or a persistent grid; with one or two inputs no cap is needed.  No MFMA:
+// (K+1)*16 bytes move per lane per step against a handful of VALU ops.
 #pragma once
 
 #include <hip/hip_runtime.h>

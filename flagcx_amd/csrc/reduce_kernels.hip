@@ -37,8 +37,9 @@ typedef bf16 elem_t;
 #define FLAGCX_CAT2(a, b) a##b
 #define FLAGCX_CAT(a, b) FLAGCX_CAT2(a, b)
 
-// Unroll (KiB of each input per wavefront): measured best on MI355X.
-constexpr int unrollFor(int K) { return K <= 2 ? 4 : 2; }
+// Unroll (KiB of each input per wavefront): measured best on MI355X with buffers
+// large enough to stream from HBM (1 GiB for K <= 4, 256 MiB for K = 8).
+constexpr int unrollFor(int K) { return K <= 4 ? 1 : 2; }
 
 constexpr uint64_t kMaxGrid = 1u << 24;
 

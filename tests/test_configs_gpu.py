@@ -1,0 +1,167 @@
+"""The benchmark configurations at their full sizes (BASELINE.json configs 1-5),
+checked against the oracle where it finishes in seconds and through
+size-independent properties elsewhere.  All GPU work goes through the C ABI."""
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from tests.util import same
+
+pytestmark = pytest.mark.gpu
+
+MiB = 1 << 20
+
+
+@pytest.fixture(scope="module")
+def L():
+    import torch
+    assert torch.cuda.is_available()
+    from flagcx_amd import local
+    assert local.lib().flagcxLocalInit() == 0
+    return local
+
+
+def test_c1_two_input_fp32_sum_64MiB(L):
+    """2 x fp32, 16 Mi elements, uniform[-1,1) seed 0; bit-exact, and the same
+    through the host-ring restatement (2 ranks -> two 32 MiB chunks)."""
+    import torch
+    n = 16 * MiB
+    rng = np.random.default_rng(0)
+    a = rng.uniform(-1, 1, n).astype(np.float32)
+    b = rng.uniform(-1, 1, n).astype(np.float32)
+    da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    out = torch.empty(n, device="cuda")
+    L.reduce([da, db], out, L.RedOp.Sum)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert same(got, a + b)                       # numpy's IEEE add, in0 + in1
+    rc, want = O.reduce([a, b], O.FP32, O.SUM)    # the reference loop's restatement
+    assert rc == 0 and same(got, want)
+    assert L.ring_chunk_table(n, L.DataType.Float32, 2) == ([0, 32 * MiB], [32 * MiB, 32 * MiB])
+    rc, ring = O.ring_allreduce([a, b], O.FP32, O.SUM, strict=True)
+    out2 = torch.empty(n, device="cuda")
+    L.all_reduce([da, db], out2, L.RedOp.Sum)
+    torch.cuda.synchronize()
+    assert rc == 0 and same(out2.cpu().numpy(), ring)
+
+
+def test_c2_eight_input_bf16_sum_256MiB(L):
+    """8 x bf16, 128 Mi elements, N(0,1) seeds 0..7, fp32 accumulation in rank
+    order: the whole output against the oracle, bit for bit."""
+    import torch
+    n = 128 * MiB
+    ins = []
+    for seed in range(8):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        ins.append(torch.randn(n, generator=g, device="cuda").to(torch.bfloat16))
+    out = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    L.reduce(ins, out, L.RedOp.Sum)
+    torch.cuda.synchronize()
+    hosts = [t.view(torch.int16).cpu().numpy().view(np.uint16) for t in ins]
+    rc, want = O.reduce(hosts, O.BF16, O.SUM)
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert rc == 0 and same(got, want)
+    # within 1 ulp (here: exactly) of a float64 evaluation wherever that is unambiguous
+    idx = np.random.default_rng(1).integers(0, n, 200000)
+    f = lambda bits: (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    exact = sum(f(h[idx]) for h in hosts)
+    err = np.abs(f(got[idx]) - exact)
+    ulp = np.maximum(np.abs(exact), 2.0 ** -126) * 2.0 ** -7
+    assert (err <= ulp).all()
+    # linearity on integer-valued data: k * (i % 10) exactly (the reference's pattern)
+    pat = (torch.arange(n, device="cuda", dtype=torch.int32) % 10).to(torch.bfloat16)
+    L.reduce([pat] * 8, out, L.RedOp.Sum)
+    torch.cuda.synchronize()
+    assert torch.equal(out.float(), pat.float() * 8)
+
+
+def test_c3_reduce_scatter_chunk_pipeline_fp16_avg(L):
+    """8 ranks x 1 GiB fp16, N(0, sigma=0.01); rank 3's shard (128 MiB) as 32
+    launches of 4 MiB and as one launch: identical, and equal to the oracle."""
+    import torch
+    nranks, per_rank = 8, 512 * MiB            # elements: 1 GiB of fp16
+    shard = per_rank // nranks                 # 64 Mi elements = 128 MiB
+    send = []
+    for r in range(nranks):
+        g = torch.Generator(device="cuda").manual_seed(100 + r)
+        buf = torch.empty(per_rank, dtype=torch.float16, device="cuda")
+        for s in range(nranks):
+            buf[s * shard:(s + 1) * shard] = (torch.randn(shard, generator=g, device="cuda") * 0.01).to(torch.float16)
+        send.append(buf)
+    rank = 3
+    fused = torch.empty(shard, dtype=torch.float16, device="cuda")
+    piped = torch.empty(shard, dtype=torch.float16, device="cuda")
+    L.reduce_scatter(send, rank, fused, L.RedOp.Avg)
+    L.reduce_scatter(send, rank, piped, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE)
+    torch.cuda.synchronize()
+    assert torch.equal(fused.view(torch.int16), piped.view(torch.int16))
+    hosts = [s[rank * shard:(rank + 1) * shard].cpu().numpy() for s in send]
+    order = [hosts[(rank + 1 + j) % nranks] for j in range(nranks)]   # ring order
+    rc, want = O.reduce(order, O.FP16, O.AVG)
+    assert rc == 0 and same(fused.cpu().numpy(), want)
+    # other shards: pipeline == fused, and a window against the oracle
+    for rk in (0, 7):
+        L.reduce_scatter(send, rk, fused, L.RedOp.Avg)
+        L.reduce_scatter(send, rk, piped, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE)
+        torch.cuda.synchronize()
+        assert torch.equal(fused.view(torch.int16), piped.view(torch.int16))
+        w0, w1 = 5 * MiB + 3, 6 * MiB + 3
+        win = [send[(rk + 1 + j) % nranks][rk * shard + w0:rk * shard + w1].cpu().numpy() for j in range(nranks)]
+        rc, want = O.reduce(win, O.FP16, O.AVG)
+        assert same(fused[w0:w1].cpu().numpy(), want)
+
+
+def test_c4_four_input_int32_max_min_512MiB(L):
+    """4 x int32, 128 Mi elements, uniform over the full range, seed 3: bit-exact."""
+    import torch
+    n = 128 * MiB
+    rng = np.random.default_rng(3)
+    hosts = [rng.integers(-2**31, 2**31 - 1, n, dtype=np.int32, endpoint=True) for _ in range(4)]
+    devs = [torch.from_numpy(h).cuda() for h in hosts]
+    out = torch.empty(n, dtype=torch.int32, device="cuda")
+    for op, npf in ((L.RedOp.Max, np.maximum), (L.RedOp.Min, np.minimum)):
+        L.reduce(devs, out, op)
+        torch.cuda.synchronize()
+        want = npf(npf(hosts[0], hosts[1]), npf(hosts[2], hosts[3]))
+        assert same(out.cpu().numpy(), want)
+    rc, want = O.reduce([h[:4 * MiB] for h in hosts], O.INT32, O.MAX)
+    L.reduce(devs, out, L.RedOp.Max)
+    torch.cuda.synchronize()
+    assert same(out[:4 * MiB].cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("log2", list(range(10, 31)))
+def test_c5_sweep_reduce2_and_strided_pack_unpack(L, log2):
+    """Sizes 1 KiB .. 1 GiB: 2-input fp32 sum; gather of 8 chunks (stride = 8 x
+    chunk) into a staging buffer and the scatter back: chunks restored exactly,
+    gaps untouched."""
+    import torch
+    size = 1 << log2
+    n = size // 4
+    g = torch.Generator(device="cuda").manual_seed(log2)
+    a = torch.rand(n, generator=g, device="cuda") * 2 - 1
+    b = torch.rand(n, generator=g, device="cuda") * 2 - 1
+    out = torch.empty(n, device="cuda")
+    L.reduce([a, b], out, L.RedOp.Sum)
+    torch.cuda.synchronize()
+    assert torch.equal(out, a + b)              # torch's elementwise IEEE add
+    if size <= 16 * MiB:
+        rc, want = O.reduce([a.cpu().numpy(), b.cpu().numpy()], O.FP32, O.SUM)
+        assert same(out.cpu().numpy(), want)
+    del a, b, out
+    chunk = size // 8                            # bytes
+    ce = chunk // 4                              # fp32 elements per chunk
+    sparse = torch.rand(8 * n, generator=g, device="cuda") * 2 - 1   # 8 chunks at stride `size`
+    staged = torch.full((n,), -7.0, device="cuda")
+    L.pack(staged.data_ptr(), sparse.data_ptr(), 8, chunk, size)
+    torch.cuda.synchronize()
+    assert torch.equal(staged.view(8, ce), sparse.view(8, n)[:, :ce])
+    if size <= 16 * MiB:
+        want = O.pack(sparse.cpu().numpy().view(np.uint8), 8, chunk, size)
+        assert same(staged.cpu().numpy().view(np.uint8), want)
+    back = torch.full((8 * n,), -3.0, device="cuda")
+    L.unpack(back.data_ptr(), staged.data_ptr(), 8, chunk, size)
+    torch.cuda.synchronize()
+    bv = back.view(8, n)
+    assert torch.equal(bv[:, :ce], sparse.view(8, n)[:, :ce])
+    assert bool((bv[:, ce:] == -3.0).all())
