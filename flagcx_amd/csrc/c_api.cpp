@@ -81,6 +81,19 @@ int launchReduce_7(const ReduceCall &);
 int launchReduce_8(const ReduceCall &);
 int launchReduce_9(const ReduceCall &);
 
+#define FLAGCX_DECL_BATCH(n) int launchReduceBatch_##n(const ReduceCall *, int);
+FLAGCX_DECL_BATCH(0) FLAGCX_DECL_BATCH(1) FLAGCX_DECL_BATCH(2) FLAGCX_DECL_BATCH(3) FLAGCX_DECL_BATCH(4)
+FLAGCX_DECL_BATCH(5) FLAGCX_DECL_BATCH(6) FLAGCX_DECL_BATCH(7) FLAGCX_DECL_BATCH(8) FLAGCX_DECL_BATCH(9)
+#undef FLAGCX_DECL_BATCH
+
+ReduceBatchLauncher reduceBatchLauncherFor(int dtype) {
+  static const ReduceBatchLauncher table[10] = {
+      launchReduceBatch_0, launchReduceBatch_1, launchReduceBatch_2, launchReduceBatch_3,
+      launchReduceBatch_4, launchReduceBatch_5, launchReduceBatch_6, launchReduceBatch_7,
+      launchReduceBatch_8, launchReduceBatch_9};
+  return (dtype >= 0 && dtype < 10) ? table[dtype] : nullptr;
+}
+
 ReduceLauncher reduceLauncherFor(int dtype) {
   static const ReduceLauncher table[10] = {launchReduce_0, launchReduce_1, launchReduce_2,
                                            launchReduce_3, launchReduce_4, launchReduce_5,
@@ -109,10 +122,12 @@ static inline bool overlaps(const void *a, const void *b, uint64_t bytes) {
   return x < y + bytes && y < x + bytes;
 }
 
-// Validation + launch shared by every reduce-type entry point.  `srcs` are the
-// inputs already in fold order.
-static flagcxResult_t reduceOrdered(const void *const *srcs, int k, void *dst, uint64_t count,
-                                    int dtype, int op, hipStream_t stream, const char *who) {
+// Validation shared by every reduce-type entry point.  `srcs` are the inputs
+// already in fold order.  Fills `c`; *empty is set when there is nothing to do.
+static flagcxResult_t prepareReduce(const void *const *srcs, int k, void *dst, uint64_t count,
+                                    int dtype, int op, hipStream_t stream, const char *who,
+                                    ReduceCall &c, bool *empty) {
+  *empty = true;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
   if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, dtype);
   if (op < 0 || op >= (int)flagcxNumRedOps)
@@ -124,7 +139,6 @@ static flagcxResult_t reduceOrdered(const void *const *srcs, int k, void *dst, u
   if ((uintptr_t)dst % ts) return fail(flagcxInvalidArgument, "%s: recvbuff not aligned to %zu", who, ts);
   if (count > (UINT64_MAX / ts)) return fail(flagcxInvalidArgument, "%s: count overflows", who);
   const uint64_t bytes = count * ts;
-  ReduceCall c;
   for (int j = 0; j < k; j++) {
     const void *s = srcs[j];
     if (!s) return fail(flagcxInvalidArgument, "%s: sendbuffs[%d] is NULL", who, j);
@@ -138,6 +152,16 @@ static flagcxResult_t reduceOrdered(const void *const *srcs, int k, void *dst, u
   c.k = k;
   c.op = op;
   c.stream = stream;
+  *empty = false;
+  return flagcxSuccess;
+}
+
+static flagcxResult_t reduceOrdered(const void *const *srcs, int k, void *dst, uint64_t count,
+                                    int dtype, int op, hipStream_t stream, const char *who) {
+  ReduceCall c;
+  bool empty;
+  flagcxResult_t r = prepareReduce(srcs, k, dst, count, dtype, op, stream, who, c, &empty);
+  if (r != flagcxSuccess || empty) return r;
   (void)deviceInfo();
   return fromHip(reduceLauncherFor(dtype)(c), who);
 }
@@ -218,6 +242,98 @@ flagcxResult_t flagcxLocalReduce(const void *const *sendbuffs, int nranks, void 
   return finish(stream, 0, "flagcxLocalReduce");
 }
 
+static flagcxResult_t launchBatch(ReduceCall *calls, int n, int dtype, const char *who) {
+  if (n == 0) return flagcxSuccess;
+  (void)deviceInfo();
+  return fromHip(reduceBatchLauncherFor(dtype)(calls, n), who);
+}
+
+flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int ndescs, int nranks,
+                                      flagcxDataType_t datatype, flagcxRedOp_t op,
+                                      flagcxStream_t stream) {
+  const char *who = "flagcxLocalReduceBatch";
+  if (ndescs < 0) return fail(flagcxInvalidArgument, "%s: ndescs %d is negative", who, ndescs);
+  if (ndescs == 0) return flagcxSuccess;
+  if (!descs) return fail(flagcxInvalidArgument, "%s: descs is NULL", who);
+  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  hipStream_t hs = hipStreamOf(stream);
+  constexpr int kGroup = 64;
+  ReduceCall calls[kGroup];
+  for (int base = 0; base < ndescs; base += kGroup) {
+    const int m = ndescs - base < kGroup ? ndescs - base : kGroup;
+    int ncalls = 0;
+    for (int i = 0; i < m; i++) {
+      const flagcxLocalReduceDesc &d = descs[base + i];
+      if (!d.sendbuffs) return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs is NULL", who, base + i);
+      bool empty;
+      flagcxResult_t r = prepareReduce(d.sendbuffs, nranks, d.recvbuff, d.count, (int)datatype, (int)op,
+                                       hs, who, calls[ncalls], &empty);
+      if (r != flagcxSuccess) return r;
+      if (empty) continue;
+      for (int e = 0; e < ncalls; e++)
+        if ((uintptr_t)calls[e].dst < (uintptr_t)d.recvbuff + d.count * ts &&
+            (uintptr_t)d.recvbuff < (uintptr_t)calls[e].dst + calls[e].count * ts)
+          return fail(flagcxInvalidArgument, "%s: recvbuff of descs[%d] overlaps an earlier one", who, base + i);
+      ncalls++;
+    }
+    flagcxResult_t r = launchBatch(calls, ncalls, (int)datatype, who);
+    if (r != flagcxSuccess) return r;
+  }
+  return finish(stream, 0, who);
+}
+
+flagcxResult_t flagcxLocalReduceTriggers(const flagcxLocalReduceTrigger *triggers, int ntriggers,
+                                         flagcxStream_t stream) {
+  const char *who = "flagcxLocalReduceTriggers";
+  if (ntriggers < 0) return fail(flagcxInvalidArgument, "%s: ntriggers %d is negative", who, ntriggers);
+  if (ntriggers == 0) return flagcxSuccess;
+  if (!triggers) return fail(flagcxInvalidArgument, "%s: triggers is NULL", who);
+  hipStream_t hs = hipStreamOf(stream);
+  constexpr int kGroup = 64;
+  ReduceCall calls[kGroup];
+  int ncalls = 0, gdt = -1, gop = -1;
+  for (int i = 0; i < ntriggers; i++) {
+    const uint64_t *v = triggers[i].value;
+    const void *op1 = (const void *)(uintptr_t)v[0];
+    const void *op2 = (const void *)(uintptr_t)v[1];
+    void *res = (void *)(uintptr_t)v[2];
+    const uint64_t count = v[3] & 0xffffffffull;
+    const int dt = (int)((v[3] >> 48) & 0xf), op = (int)((v[3] >> 52) & 0xf);
+    const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dt);
+    const uint64_t bytes = count * ts;
+    // a trigger that touches what an earlier trigger of the group writes, or
+    // writes what one reads, must wait for it: close the group first
+    bool flush = ncalls == kGroup || (ncalls > 0 && (dt != gdt || op != gop));
+    for (int e = 0; !flush && e < ncalls; e++) {
+      const uint64_t eb = calls[e].count * ts;
+      auto hit = [](const void *a, uint64_t an, const void *b, uint64_t bn) {
+        return (uintptr_t)a < (uintptr_t)b + bn && (uintptr_t)b < (uintptr_t)a + an;
+      };
+      if (hit(calls[e].dst, eb, op1, bytes) || hit(calls[e].dst, eb, op2, bytes) ||
+          hit(calls[e].dst, eb, res, bytes) || hit(res, bytes, calls[e].src[0], eb) ||
+          hit(res, bytes, calls[e].src[1], eb))
+        flush = true;
+    }
+    if (flush) {
+      flagcxResult_t r = launchBatch(calls, ncalls, gdt, who);
+      if (r != flagcxSuccess) return r;
+      ncalls = 0;
+    }
+    // fold order: acc = op2; acc = OP(op1, acc)  ==  OP(op1, op2)
+    const void *srcs[2] = {op2, op1};
+    bool empty;
+    flagcxResult_t r = prepareReduce(srcs, 2, res, count, dt, op, hs, who, calls[ncalls], &empty);
+    if (r != flagcxSuccess) return r;
+    if (empty) continue;
+    gdt = dt;
+    gop = op;
+    ncalls++;
+  }
+  flagcxResult_t r = launchBatch(calls, ncalls, gdt, who);
+  if (r != flagcxSuccess) return r;
+  return finish(stream, 0, who);
+}
+
 flagcxResult_t flagcxLocalReduceScatterChunked(const void *const *sendbuffs, int nranks, int rank,
                                                void *recvbuff, size_t recvcount,
                                                flagcxDataType_t datatype, flagcxRedOp_t op,
@@ -286,15 +402,22 @@ flagcxResult_t flagcxLocalAllReduce(const void *const *sendbuffs, int nranks, vo
   // The validation of op has to happen even when every chunk is empty.
   if ((int)op < 0 || (int)op >= (int)flagcxNumRedOps)
     return fail(flagcxInvalidArgument, "%s: unsupported reduction operation %d", who, (int)op);
+  ReduceCall calls[FLAGCX_LOCAL_MAX_RANKS];
+  int ncalls = 0;
   for (int c = 0; c < nranks; c++) {
     if (length[c] == 0) continue; // zero-length chunks are skipped (bootstrap.cc:599-610)
     for (int j = 0; j < nranks; j++)
       ordered[j] = (const char *)sendbuffs[(c + 1 + j) % nranks] + offset[c];
-    flagcxResult_t res = reduceOrdered(ordered, nranks, (char *)recvbuff + offset[c], length[c] / ts,
-                                       (int)datatype, (int)op, hs, who);
+    bool empty;
+    flagcxResult_t res = prepareReduce(ordered, nranks, (char *)recvbuff + offset[c], length[c] / ts,
+                                       (int)datatype, (int)op, hs, who, calls[ncalls], &empty);
     if (res != flagcxSuccess) return res;
+    if (!empty) ncalls++;
   }
-  return finish(stream, 0, who);
+  if (ncalls == 0) return flagcxSuccess;
+  (void)deviceInfo();
+  // all chunks in one launch; each chunk keeps its own fold order
+  return finish(stream, reduceBatchLauncherFor((int)datatype)(calls, ncalls), who);
 }
 
 // ------------------------------------------------------------ byte movers

@@ -37,6 +37,9 @@ int ldsReservation(int waves);
 // One launcher per element type; returns a hipError_t value.
 typedef int (*ReduceLauncher)(const ReduceCall &);
 ReduceLauncher reduceLauncherFor(int dtype);
+// n reductions sharing k, op and stream, in as few launches as possible.
+typedef int (*ReduceBatchLauncher)(const ReduceCall *, int);
+ReduceBatchLauncher reduceBatchLauncherFor(int dtype);
 
 // Byte movers (copy_kernels.hip); all return a hipError_t value.
 struct Copy2D {

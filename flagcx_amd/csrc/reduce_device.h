@@ -196,7 +196,7 @@ constexpr int kRsrcFlags = 0x00020000;
 // dst may be one of the inputs: a lane reads its positions before it writes
 // them, and no other lane touches them.
 template <typename T, int OP, int K, int U>
-__global__ void __launch_bounds__(64) reduceWaveKernel(ReduceParams<K> p) {
+__device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
   constexpr int N = 16 / sizeof(T);
   constexpr uint32_t kTileBytes = 64u * U * 16u;
   const uint64_t bodyBytes = p.nvec * 16;
@@ -232,6 +232,26 @@ __global__ void __launch_bounds__(64) reduceWaveKernel(ReduceParams<K> p) {
       foldScalar<T, OP>(p.src, K, p.dst, i);
     }
   }
+}
+
+template <typename T, int OP, int K, int U>
+__global__ void __launch_bounds__(64) reduceWaveKernel(ReduceParams<K> p) {
+  reduceWaveBody<T, OP, K, U>(p);
+}
+
+// Several independent reductions of the same type, op and K in one launch:
+// blockIdx.y picks the segment, blockIdx.x walks its tiles.  Used where a
+// collective is cut into chunks that each have their own pointers or fold order
+// (ring all-reduce chunks, pipeline chunks, reduce triggers).
+#define FLAGCX_BATCH_MAX 32
+template <int K>
+struct ReduceBatchParams {
+  ReduceParams<K> seg[FLAGCX_BATCH_MAX];
+};
+
+template <typename T, int OP, int K, int U>
+__global__ void __launch_bounds__(64) reduceBatchKernel(ReduceBatchParams<K> bp) {
+  reduceWaveBody<T, OP, K, U>(bp.seg[blockIdx.y]);
 }
 
 // Aligned body, any k up to FLAGCX_MAX_RANKS: inputs are consumed in batches of

@@ -126,6 +126,81 @@ static int launchOp(const ReduceCall &c) {
   }
 }
 
+template <int OP, int K>
+static int launchBatchFixed(const ReduceCall *calls, const Split *splits, int n) {
+  constexpr int U = unrollFor(K);
+  const uint64_t tileBytes = 64ull * U * 16ull;
+  for (int base = 0; base < n; base += FLAGCX_BATCH_MAX) {
+    const int m = n - base < FLAGCX_BATCH_MAX ? n - base : FLAGCX_BATCH_MAX;
+    ReduceBatchParams<K> bp;
+    uint64_t maxTiles = 1;
+    for (int i = 0; i < m; i++) {
+      const ReduceCall &c = calls[base + i];
+      const Split &s = splits[base + i];
+      ReduceParams<K> &p = bp.seg[i];
+      for (int j = 0; j < K; j++) p.src[j] = c.src[j];
+      p.dst = c.dst;
+      p.nvec = s.nvec;
+      p.head = s.head;
+      p.tail = s.tail;
+      p.k = K;
+      const uint64_t tiles = (s.nvec * 16 + tileBytes - 1) / tileBytes;
+      if (tiles > maxTiles) maxTiles = tiles;
+    }
+    if (maxTiles > kMaxGrid) maxTiles = kMaxGrid;
+    const int lds = ldsReservation(wavesPerCUFor(K));
+    reduceBatchKernel<elem_t, OP, K, U>
+        <<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, calls[0].stream>>>(bp);
+    const int err = (int)hipGetLastError();
+    if (err) return err;
+  }
+  return 0;
+}
+
+template <int OP>
+static int launchBatchOp(const ReduceCall *calls, int n) {
+  // One launch per 32 segments when every segment can take the 16-byte path with
+  // the same compile-time K; otherwise segment by segment.
+  const int k = calls[0].k;
+  bool fast = k <= 8 && n > 1;
+  Split splits[256];
+  if (n > 256) fast = false;
+  for (int i = 0; fast && i < n; i++) {
+    splits[i] = splitFor(calls[i]);
+    if (!splits[i].vector || calls[i].k != k) fast = false;
+  }
+  if (!fast) {
+    for (int i = 0; i < n; i++) {
+      const int err = launchOp<OP>(calls[i]);
+      if (err) return err;
+    }
+    return 0;
+  }
+  switch (k) {
+    case 1: return launchBatchFixed<OP, 1>(calls, splits, n);
+    case 2: return launchBatchFixed<OP, 2>(calls, splits, n);
+    case 3: return launchBatchFixed<OP, 3>(calls, splits, n);
+    case 4: return launchBatchFixed<OP, 4>(calls, splits, n);
+    case 5: return launchBatchFixed<OP, 5>(calls, splits, n);
+    case 6: return launchBatchFixed<OP, 6>(calls, splits, n);
+    case 7: return launchBatchFixed<OP, 7>(calls, splits, n);
+    default: return launchBatchFixed<OP, 8>(calls, splits, n);
+  }
+}
+
+// n reductions that share k, op and stream.
+int FLAGCX_CAT(launchReduceBatch_, FLAGCX_DT)(const ReduceCall *calls, int n) {
+  if (n <= 0) return 0;
+  switch (calls[0].op) {
+    case kSum: return launchBatchOp<kSum>(calls, n);
+    case kProd: return launchBatchOp<kProd>(calls, n);
+    case kMax: return launchBatchOp<kMax>(calls, n);
+    case kMin: return launchBatchOp<kMin>(calls, n);
+    case kAvg: return launchBatchOp<kAvg>(calls, n);
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
 int FLAGCX_CAT(launchReduce_, FLAGCX_DT)(const ReduceCall &c) {
   switch (c.op) {
     case kSum: return launchOp<kSum>(c);

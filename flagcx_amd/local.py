@@ -66,6 +66,23 @@ class ReduceArgs(C.Structure):       # flagcxLocalReduceArgs
                 ("nranks", C.c_int32), ("datatype", C.c_int32), ("op", C.c_int32), ("result", C.c_int32)]
 
 
+class ReduceDesc(C.Structure):       # flagcxLocalReduceDesc
+    _fields_ = [("sendbuffs", C.POINTER(C.c_void_p)), ("recvbuff", C.c_void_p), ("count", C.c_size_t)]
+
+
+class ReduceTrigger(C.Structure):    # flagcxLocalReduceTrigger, 16-byte aligned
+    _fields_ = [("value", C.c_uint64 * 4)]
+    _pack_ = 16
+
+    @classmethod
+    def make(cls, addr1, addr2, addr3, count, datatype, redop, nthreads=0):
+        t = cls()
+        t.value[0], t.value[1], t.value[2] = addr1, addr2, addr3
+        t.value[3] = (count & 0xffffffff) | ((nthreads & 0xffff) << 32) | ((int(datatype) & 0xf) << 48) | \
+                     ((int(redop) & 0xf) << 52)
+        return t
+
+
 class CopyArgs(C.Structure):         # flagcxLocalCopyArgs
     _fields_ = [("dst", C.c_void_p), ("src", C.c_void_p), ("size", C.c_uint64), ("result", C.c_int32),
                 ("reserved", C.c_int32)]
@@ -77,6 +94,8 @@ EXPORTS = [
     "flagcxLocalAllReduce", "flagcxLocalRingChunkTable", "flagcxLocalMemcpy", "flagcxLocalMemset",
     "flagcxLocalRefresh", "flagcxLocalPack", "flagcxLocalUnpack", "flagcxLocalPackList",
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
+    "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
+    "flagcxLocalReduceBatch", "flagcxLocalReduceTriggers",
 ]
 
 
@@ -117,6 +136,14 @@ def lib():
         L.flagcxLocalReduceFunc.argtypes = [sp, C.POINTER(ReduceArgs)]
         L.flagcxLocalCopyFunc.restype = None
         L.flagcxLocalCopyFunc.argtypes = [sp, C.POINTER(CopyArgs)]
+        L.flagcxLocalReduceBatch.argtypes = [C.POINTER(ReduceDesc), i, i, i, i, sp]
+        L.flagcxLocalReduceTriggers.argtypes = [C.POINTER(ReduceTrigger), i, sp]
+        L.flagcxLocalSetMaxSpinCount.restype = None
+        L.flagcxLocalSetMaxSpinCount.argtypes = [C.c_int64]
+        for name in ("deviceAsyncStore", "deviceAsyncLoad"):
+            fn = getattr(L, name)
+            fn.restype = None
+            fn.argtypes = [sp, vp]
         _lib = L
     return _lib
 
@@ -192,6 +219,20 @@ def all_reduce(sendbuffs, recv, op, dtype=None, stream="current"):
     check(lib().flagcxLocalAllReduce(_ptr_array([s.data_ptr() for s in sendbuffs]), len(sendbuffs),
                                      recv.data_ptr(), recv.numel(), int(dt), int(op), _sref(st)))
     return recv
+
+
+def reduce_batch(descs, op, dtype, nranks, stream="current"):
+    """descs: list of (list_of_src_ptrs, dst_ptr, count).  One flagcxLocalReduceBatch call."""
+    st = current_stream() if stream == "current" else stream
+    keep = [_ptr_array(list(d[0])) for d in descs]
+    arr = (ReduceDesc * len(descs))(*[ReduceDesc(keep[i], d[1], d[2]) for i, d in enumerate(descs)])
+    check(lib().flagcxLocalReduceBatch(arr, len(descs), nranks, int(dtype), int(op), _sref(st)))
+
+
+def reduce_triggers(triggers, stream="current"):
+    st = current_stream() if stream == "current" else stream
+    arr = (ReduceTrigger * len(triggers))(*triggers)
+    check(lib().flagcxLocalReduceTriggers(arr, len(triggers), _sref(st)))
 
 
 def ring_chunk_table(count, dtype, nranks):

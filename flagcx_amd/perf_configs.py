@@ -1,0 +1,128 @@
+"""Timings of the benchmark configurations other than the headline one, on one GPU:
+
+    python -m flagcx_amd.perf_configs [--json out.json] [--cpu]
+
+  C1  2-input fp32 sum, 64 MiB per buffer
+  C3  fp16 avg reduce-scatter shard (8 ranks x 1 GiB, shard = 128 MiB): one fused
+      launch, and 32 launches of 4 MiB chunks (the staging ring's step size)
+  C4  4-input int32 max and min, 512 MiB per buffer
+5 warm-up + 20 timed iterations (test/perf/tools.cc:81-86), HIP events, back-to-back
+launches per iteration.  GB/s = (k+1) * n * size / time.  --cpu also times the CPU
+oracle (test infrastructure, imported only under this flag) on bounded samples.
+"""
+import argparse
+import json
+import sys
+
+import torch
+
+from flagcx_amd import local as L
+
+MiB = 1 << 20
+
+
+def timed(fn, warmup=5, iters=20):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters   # ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--json", default=None)
+    ap.add_argument("--cpu", action="store_true")
+    args = ap.parse_args()
+    torch.cuda.set_device(0)
+    L.check(L.lib().flagcxLocalInit())
+    rows = []
+
+    def report(name, nbytes, ms, note=""):
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        rows.append({"config": name, "bytes": nbytes, "ms": ms, "gbps": gbps, "pct_peak": gbps / 80.0, "note": note})
+        print("%-44s %14d B  %9.4f ms  %8.1f GB/s  %5.1f %%  %s" % (name, nbytes, ms, gbps, gbps / 80.0, note), flush=True)
+
+    # C1
+    n = 16 * MiB
+    g = torch.Generator(device="cuda").manual_seed(0)
+    a = torch.rand(n, generator=g, device="cuda") * 2 - 1
+    b = torch.rand(n, generator=g, device="cuda") * 2 - 1
+    out = torch.empty(n, device="cuda")
+    ms = timed(lambda: L.reduce([a, b], out, L.RedOp.Sum))
+    report("C1 2x fp32 sum 64 MiB (cache-resident size)", 3 * n * 4, ms)
+    ms = timed(lambda: L.all_reduce([a, b], out, L.RedOp.Sum))
+    report("C1 as ring all-reduce (2 chunk launches)", 3 * n * 4, ms)
+    del a, b, out
+
+    # C3
+    nranks, per_rank = 8, 512 * MiB
+    shard = per_rank // nranks
+    send = []
+    for r in range(nranks):
+        g = torch.Generator(device="cuda").manual_seed(100 + r)
+        buf = torch.empty(per_rank, dtype=torch.float16, device="cuda")
+        for s in range(nranks):
+            buf[s * shard:(s + 1) * shard] = (torch.randn(shard, generator=g, device="cuda") * 0.01).to(torch.float16)
+        send.append(buf)
+    recv = torch.empty(shard, dtype=torch.float16, device="cuda")
+    nb = 9 * shard * 2
+    ms = timed(lambda: L.reduce_scatter(send, 3, recv, L.RedOp.Avg))
+    report("C3 fp16 avg shard 128 MiB, fused launch", nb, ms)
+    ms = timed(lambda: L.reduce_scatter(send, 3, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE))
+    report("C3 fp16 avg shard, 32 x 4 MiB chunk launches", nb, ms, "%.2f us per chunk launch" % (ms * 1e3 / 32))
+
+    chunk_elems = L.CHUNKSIZE // 2
+    descs = []
+    for c in range(shard // chunk_elems):
+        srcs = [send[(3 + 1 + j) % nranks].data_ptr() + (3 * shard + c * chunk_elems) * 2 for j in range(nranks)]
+        descs.append((srcs, recv.data_ptr() + c * chunk_elems * 2, chunk_elems))
+    ms = timed(lambda: L.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks))
+    report("C3 fp16 avg shard, 32 chunks as one batch call", nb, ms)
+
+    def all_shards():
+        for rk in range(nranks):
+            L.reduce_scatter(send, rk, recv, L.RedOp.Avg)
+    ms = timed(all_shards, warmup=2, iters=5)
+    report("C3 all 8 shards (8 fused launches, 1 GiB out)", 8 * nb, ms)
+    del send, recv
+
+    # C4
+    n = 128 * MiB
+    g = torch.Generator(device="cuda").manual_seed(3)
+    ins = [torch.randint(-2**31, 2**31 - 1, (n,), generator=g, device="cuda", dtype=torch.int32) for _ in range(4)]
+    out = torch.empty(n, dtype=torch.int32, device="cuda")
+    for op, nm in ((L.RedOp.Max, "max"), (L.RedOp.Min, "min")):
+        ms = timed(lambda: L.reduce(ins, out, op))
+        report("C4 4x int32 %s 512 MiB" % nm, 5 * n * 4, ms)
+
+    if args.cpu:
+        import numpy as np
+        from oracle import cpu_oracle as O
+        sample = 16 * MiB
+        hosts = [t[:sample].cpu().numpy() for t in ins]
+        dst = np.empty(sample, dtype=np.int32)
+        for nth in (1, 4):
+            t = O.time_reduce(hosts, dst, O.INT32, O.MAX, nthreads=nth, warmup=1, iters=3)
+            report("CPU oracle C4 int32 max, %d thread(s), 16 Mi-elem sample" % nth, 5 * sample * 4, t * 1e3)
+        rng = np.random.default_rng(0)
+        fa = rng.uniform(-1, 1, 16 * MiB).astype(np.float32)
+        fb = rng.uniform(-1, 1, 16 * MiB).astype(np.float32)
+        fd = np.empty_like(fa)
+        for nth in (1, 2):
+            t = O.time_reduce([fa, fb], fd, O.FP32, O.SUM, nthreads=nth, warmup=1, iters=3)
+            report("CPU oracle C1 fp32 sum, %d thread(s), full size" % nth, 3 * fa.nbytes, t * 1e3)
+    if args.json:
+        with open(args.json, "w") as f:
+            json.dump(rows, f)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -200,6 +200,54 @@ flagcxResult_t flagcxLocalAllReduce(const void *const *sendbuffs, int nranks,
                                     flagcxDataType_t datatype, flagcxRedOp_t op,
                                     flagcxStream_t stream);
 
+/* Several independent reductions that share nranks, datatype and op, enqueued in
+ * as few launches as possible (one per 32 descriptors): the chunks of a pipelined
+ * collective once they are all present, or ring chunks that differ in fold order.
+ * Each descriptor is one flagcxLocalReduce.  Descriptors of one call run
+ * concurrently: no descriptor's recvbuff may overlap another descriptor's buffers
+ * (overlapping recvbuffs are rejected; inputs are the caller's responsibility). */
+typedef struct {
+  const void *const *sendbuffs; /* host array of nranks device pointers, fold order */
+  void *recvbuff;
+  size_t count;
+} flagcxLocalReduceDesc;
+
+flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int ndescs,
+                                      int nranks, flagcxDataType_t datatype,
+                                      flagcxRedOp_t op, flagcxStream_t stream);
+
+/* Consumer of the reference's reduce descriptor, which is declared but has no
+ * producer or consumer there (flagcxReduceTrigger, flagcx/include/flagcx_kernel.h:30-35,
+ * 52-73; host-producer API commented out at :96-98).  Same 256-bit layout:
+ *   value[0] addr1, value[1] addr2, value[2] addr3,
+ *   value[3] = count[0,32) | nthreads[32,48) | datatype[48,52) | redop[52,56) | reserved[63]
+ * Meaning given here, after the host templates' (res, op1, op2) order
+ * (flagcx/service/utils.h:681-709): addr3[i] = OP(addr1[i], addr2[i]), i < count;
+ * nthreads is a hint and is ignored.  Triggers are executed in order; consecutive
+ * triggers of the same datatype and op that do not depend on one another share a
+ * launch. */
+typedef struct {
+#ifdef __cplusplus
+  alignas(16)
+#endif
+  uint64_t value[4];
+} flagcxLocalReduceTrigger;
+
+static inline flagcxLocalReduceTrigger
+flagcxLocalMakeReduceTrigger(const void *addr1, const void *addr2, void *addr3, uint32_t count,
+                             uint32_t nthreads, flagcxDataType_t datatype, flagcxRedOp_t redop) {
+  flagcxLocalReduceTrigger t;
+  t.value[0] = (uint64_t)(uintptr_t)addr1;
+  t.value[1] = (uint64_t)(uintptr_t)addr2;
+  t.value[2] = (uint64_t)(uintptr_t)addr3;
+  t.value[3] = (uint64_t)count | ((uint64_t)(nthreads & 0xffffu) << 32) |
+               ((uint64_t)((unsigned)datatype & 0xfu) << 48) | ((uint64_t)((unsigned)redop & 0xfu) << 52);
+  return t;
+}
+
+flagcxResult_t flagcxLocalReduceTriggers(const flagcxLocalReduceTrigger *triggers, int ntriggers,
+                                         flagcxStream_t stream);
+
 /* The chunk table itself (bootstrap.cc:692-738): offsets[i], lengths[i] in bytes
  * for i in [0,nranks).  Host-only. */
 flagcxResult_t flagcxLocalRingChunkTable(size_t count, flagcxDataType_t datatype,
@@ -286,6 +334,18 @@ typedef struct {
 
 void flagcxLocalReduceFunc(flagcxStream_t stream, void *args /* flagcxLocalReduceArgs* */);
 void flagcxLocalCopyFunc(flagcxStream_t stream, void *args /* flagcxLocalCopyArgs* */);
+
+/* The two symbols flagcxCommInitRank resolves from FLAGCX_DEVICE_FUNC_PATH
+ * (flagcx/flagcx.cc:552-562); gfx950 versions of
+ * flagcx/kernels/device_async_kernel.dev:14-23.  args is a device bool*:
+ * Store sets it; Load returns once it is set or after the spin bound
+ * (FLAGCX_FUNC_MAX_SPIN_COUNT polls, default 2^27) - the reference spins without
+ * bound.  These keep the reference's un-prefixed names because it looks them up
+ * by name. */
+void deviceAsyncStore(flagcxStream_t stream, void *args /* bool* on the device */);
+void deviceAsyncLoad(flagcxStream_t stream, void *args /* bool* on the device */);
+/* Overrides the spin bound of deviceAsyncLoad (negative: back to the environment). */
+void flagcxLocalSetMaxSpinCount(int64_t polls);
 
 #ifdef __cplusplus
 }

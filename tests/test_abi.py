@@ -16,7 +16,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_symbols():
     text = open(os.path.join(ROOT, "include", "flagcx_amd.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(flagcxLocal\w+)\s*\(", text)))
+    names = set(re.findall(r"\b(flagcxLocal\w+|deviceAsync\w+)\s*\(", text))
+    names.discard("flagcxLocalMakeReduceTrigger")   # static inline helper, not an export
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():
@@ -122,6 +124,28 @@ def test_launcher_convention_reports_through_the_argument_block():
     cargs = local.CopyArgs(None, 0x10000, 16, -1, 0)
     L.flagcxLocalCopyFunc(C.byref(st), C.byref(cargs))
     assert cargs.result == int(local.Result.InvalidArgument)
+
+
+def test_batch_and_trigger_entry_points_validate():
+    L = local.lib()
+    st = C.byref(local.Stream(None))
+    inv = int(local.Result.InvalidArgument)
+    a, b = 0x10000, 0x90000
+    ptrs = (C.c_void_p * 2)(a, a + 0x1000)
+    d = (local.ReduceDesc * 2)(local.ReduceDesc(ptrs, b, 16), local.ReduceDesc(ptrs, b + 32, 16))
+    assert L.flagcxLocalReduceBatch(d, 2, 2, 7, 0, st) == inv            # recvbuffs overlap
+    assert b"overlaps" in L.flagcxLocalGetLastError()
+    assert L.flagcxLocalReduceBatch(d, 2, 2, 11, 0, st) == inv           # dtype
+    assert L.flagcxLocalReduceBatch(d, -1, 2, 7, 0, st) == inv
+    assert L.flagcxLocalReduceBatch(None, 1, 2, 7, 0, st) == inv
+    assert L.flagcxLocalReduceBatch(d, 0, 2, 7, 0, st) == 0
+    t = (local.ReduceTrigger * 1)(local.ReduceTrigger.make(a, a + 0x1000, b, 16, 6 + 4, 0))  # dtype 10
+    assert L.flagcxLocalReduceTriggers(t, 1, st) == inv
+    t = (local.ReduceTrigger * 1)(local.ReduceTrigger.make(a, 0, b, 16, 7, 0))                # NULL op2
+    assert L.flagcxLocalReduceTriggers(t, 1, st) == inv
+    t = (local.ReduceTrigger * 1)(local.ReduceTrigger.make(a, a, b, 0, 7, 0))                 # empty
+    assert L.flagcxLocalReduceTriggers(t, 1, st) == 0
+    assert C.sizeof(local.ReduceTrigger) == 32
 
 
 def test_error_strings():

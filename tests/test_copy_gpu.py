@@ -126,3 +126,23 @@ def test_pack_list_and_unpack_list(L, nbytes):
             g = from_dev(outs[j], np.uint8)
             assert same(g[off:off + nbytes], hs[j][off:off + nbytes]), (nbytes, off, j)
             assert (g[:off] == 0x22).all() and (g[off + nbytes:] == 0x22).all()
+
+
+def test_device_async_store_and_bounded_load(L):
+    """deviceAsyncStore sets the flag, deviceAsyncLoad returns once it is set; with
+    the flag never set the load gives up after its spin bound and exits normally."""
+    import torch
+    flag = torch.zeros(4, dtype=torch.uint8, device="cuda")
+    st = L.current_stream()
+    lib = L.lib()
+    lib.deviceAsyncStore(C.byref(st), flag.data_ptr())
+    lib.deviceAsyncLoad(C.byref(st), flag.data_ptr())      # already set: no spinning
+    torch.cuda.synchronize()
+    assert flag.cpu().tolist() == [1, 0, 0, 0]
+    lib.flagcxLocalSetMaxSpinCount(8)                      # host-forced tiny bound
+    try:
+        lib.deviceAsyncLoad(C.byref(st), flag.data_ptr() + 1)  # never set
+        torch.cuda.synchronize()
+    finally:
+        lib.flagcxLocalSetMaxSpinCount(-1)
+    assert flag.cpu().tolist() == [1, 0, 0, 0]

@@ -241,3 +241,83 @@ def test_reduce_scatter_reference_pattern(L):
         L.reduce_scatter([x] * k, rank, out, O.SUM, dtype=O.FP32)
         torch.cuda.synchronize()
         assert np.array_equal(from_dev(out, np.float32), np.full(rcount, k * rank, np.float32))
+
+
+# ------------------------------------------------------- batch and triggers
+
+@pytest.mark.parametrize("dt,op,k", [(O.BF16, O.SUM, 8), (O.FP32, O.MIN, 3), (O.INT32, O.SUM, 2), (O.FP16, O.AVG, 9)],
+                         ids=lambda v: str(v))
+def test_reduce_batch_matches_oracle(L, dt, op, k):
+    """Many descriptors of different sizes and alignments in one call; each must
+    equal its own flagcxLocalReduce / oracle result."""
+    import torch
+    ts = O.type_size(dt)
+    sizes = [1, 7, 4096, 100003, 33, 65536, 12345] * 6      # 42 descriptors -> two launches
+    srcs_h, devs, outs, descs = [], [], [], []
+    for i, n in enumerate(sizes):
+        off = i % 3                                          # some descriptors unaligned
+        hs = make_inputs(dt, k, n + 4, seed=900 + i, op=op)
+        ds = [to_dev(h) for h in hs]
+        out = dev_empty(n + 4, ts, fill=0)
+        srcs_h.append([np.ascontiguousarray(h[off:off + n]) for h in hs])
+        devs.append(ds)
+        outs.append(out)
+        descs.append(([d.data_ptr() + off * ts for d in ds], out.data_ptr() + off * ts, n))
+    L.reduce_batch(descs, op, dt, k)
+    torch.cuda.synchronize()
+    for i, n in enumerate(sizes):
+        off = i % 3
+        rc, want = O.reduce(srcs_h[i], dt, op)
+        got = from_dev(outs[i], srcs_h[i][0].dtype)[off:off + n]
+        assert same(got, want, nan_class=arith_nan_ok(dt, op), dtype=dt), (i, n)
+
+
+def test_chunk_pipeline_as_one_batch_equals_chunked(L):
+    """The 4 MiB chunks of a reduce-scatter shard as one batch call."""
+    import torch
+    nranks, rcount, rank = 8, 1 << 20, 5
+    chunk = 1 << 16
+    send = [to_dev(h) for h in make_inputs(O.FP16, nranks, nranks * rcount, seed=31)]
+    ref = dev_empty(rcount, 2)
+    L.reduce_scatter(send, rank, ref, O.AVG, dtype=O.FP16)
+    out = dev_empty(rcount, 2)
+    descs = []
+    for c in range(rcount // chunk):
+        srcs = [send[(rank + 1 + j) % nranks].data_ptr() + (rank * rcount + c * chunk) * 2 for j in range(nranks)]
+        descs.append((srcs, out.data_ptr() + c * chunk * 2, chunk))
+    L.reduce_batch(descs, O.AVG, O.FP16, nranks)
+    torch.cuda.synchronize()
+    assert torch.equal(ref, out)
+
+
+def test_reduce_triggers_in_order_with_dependencies(L):
+    """Binary reduce descriptors in the reference's 256-bit layout, executed in
+    order: a ring-style chain where each trigger consumes the previous output."""
+    import torch
+    n = 50000
+    hs = make_inputs(O.FP32, 4, n, seed=8)
+    ds = [to_dev(h) for h in hs]
+    t1 = dev_empty(n, 4)
+    t2 = dev_empty(n, 4)
+    t3 = dev_empty(n, 4)
+    other = dev_empty(n, 4)
+    T = L.ReduceTrigger.make
+    f32 = int(L.DataType.Float32)
+    trig = [T(ds[1].data_ptr(), ds[0].data_ptr(), t1.data_ptr(), n, f32, O.SUM),     # t1 = x1 + x0
+            T(ds[2].data_ptr(), t1.data_ptr(), t2.data_ptr(), n, f32, O.SUM),        # t2 = x2 + t1 (depends)
+            T(ds[3].data_ptr(), ds[0].data_ptr(), other.data_ptr(), n, f32, O.MAX),  # independent, other op
+            T(ds[3].data_ptr(), t2.data_ptr(), t3.data_ptr(), n, f32, O.SUM)]        # t3 = x3 + t2
+    L.reduce_triggers(trig)
+    torch.cuda.synchronize()
+    rc, want = O.reduce(hs, O.FP32, O.SUM)          # ((x0+x1)+x2)+x3 in the ring's operand order
+    assert same(from_dev(t3, np.float32), want)
+    rc, wmax = O.binary(O.MAX, O.FP32, hs[3], hs[0])
+    assert same(from_dev(other, np.float32), wmax)
+    # int32 min through a trigger
+    hi = make_inputs(O.INT32, 2, 1001, seed=9)
+    di = [to_dev(h) for h in hi]
+    oi = dev_empty(1001, 4)
+    L.reduce_triggers([T(di[0].data_ptr(), di[1].data_ptr(), oi.data_ptr(), 1001, int(L.DataType.Int32), O.MIN)])
+    torch.cuda.synchronize()
+    rc, wmin = O.binary(O.MIN, O.INT32, hi[0], hi[1])
+    assert same(from_dev(oi, np.int32), wmin)
