@@ -168,7 +168,7 @@ def main():
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "reduceWaveKernel<bf16,sum,K=8,U=2>", "avg_launch_ms": round(kern_ms, 5),
+                     "kernel": "reduceWaveKernel<bf16,sum,K=8,U=1>", "avg_launch_ms": round(kern_ms, 5),
                      "algorithmic_bytes_per_launch": ALGO_BYTES},
         "latency_us_4KiB": {"workload": "2-input fp32 sum, 4 KiB per buffer",
                             "back_to_back_per_launch": round(lat_stream_us, 3),

@@ -50,9 +50,12 @@ const DeviceInfo &deviceInfo() {
 }
 
 // Resident one-wave workgroups per CU by number of inputs (index 0: copies;
-// 0 = no cap).  Measured on MI355X with HBM-resident buffers; see the kernel
-// header for why fewer resident wavefronts stream faster as inputs multiply.
-static std::atomic<int> gWaves[9] = {{0}, {0}, {24}, {24}, {16}, {10}, {8}, {8}, {8}};
+// 0 = no cap).  Measured on MI355X with HBM-resident buffers over a set of
+// inter-buffer strides; the values are the ones whose WORST stride is best
+// (K = 8: 81-86 % of peak at 16, against 72-88 % at 8).  About 48-128 KiB of
+// loads in flight per CU saturates HBM; more resident wavefronts only add DRAM
+// page conflicts between the streams.
+static std::atomic<int> gWaves[9] = {{0}, {0}, {24}, {16}, {12}, {12}, {12}, {14}, {16}};
 
 int wavesPerCUFor(int k) {
   if (k < 0) k = 0;

@@ -8,14 +8,15 @@
 //
 // Streaming layout: a workgroup is ONE wavefront (64 lanes).  A lane owns one
 // 16-byte vector per load, so a wavefront-wide load is one coalesced 1 KiB
-// request; the wavefront's tile is U consecutive KiB of every input, and all K*U
-// loads are issued, input by input, before the first use.  Loads carry the `nt`
-// cache hint (streamed once), stores go out with `sc1`.  The launch reserves LDS
-// it never touches, only to cap how many wavefronts share a CU: with K = 8 inputs
-// about 8 resident wavefronts per CU (128 KiB of loads in flight) keep HBM busy
-// while staying out of each other's DRAM pages, and measured faster than a full
-// CU or a persistent grid; with one or two inputs no cap is needed.  No MFMA:
-// (K+1)*16 bytes move per lane per step against a handful of VALU ops.
+// request; the wavefront's tile is U consecutive KiB of every input (U = 1 in the
+// shipped configuration), and all K*U loads are issued, input by input, before
+// the first use.  Loads carry the `nt` cache hint (streamed once), stores go out
+// with `sc1`.  The launch reserves LDS it never touches, only to cap how many
+// wavefronts share a CU: with K = 8 inputs 16 resident wavefronts per CU (128 KiB
+// of loads in flight) keep HBM busy while staying out of each other's DRAM pages,
+// and measured faster than a full CU or a persistent grid; with one or two inputs
+// no cap is needed.  No MFMA: (K+1)*16 bytes move per lane per step against a
+// handful of VALU ops.
 #pragma once
 
 #include <hip/hip_runtime.h>

@@ -37,9 +37,11 @@ typedef bf16 elem_t;
 #define FLAGCX_CAT2(a, b) a##b
 #define FLAGCX_CAT(a, b) FLAGCX_CAT2(a, b)
 
-// Unroll (KiB of each input per wavefront): measured best on MI355X with buffers
-// large enough to stream from HBM (1 GiB for K <= 4, 256 MiB for K = 8).
-constexpr int unrollFor(int K) { return K <= 4 ? 1 : 2; }
+// Unroll (KiB of each input per wavefront).  One KiB per input measured best or
+// equal for every K on MI355X once buffers are large enough to stream from HBM,
+// and is the least sensitive to how the inputs' addresses alias in the HBM
+// channel hash (tried: inter-buffer strides of 128 MiB .. 1 GiB plus 0 .. 33 MiB).
+constexpr int unrollFor(int) { return 1; }
 
 constexpr uint64_t kMaxGrid = 1u << 24;
 
