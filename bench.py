@@ -37,7 +37,7 @@ ALGO_BYTES = (K + 1) * N_ELEM * 2   # k reads + 1 write
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/reduce8_bf16_sum_256MiB_pmc.txt), scaled by a copy kernel of known size.
-MEASURED_TRAFFIC_BYTES = 2415730688
+MEASURED_TRAFFIC_BYTES = 2415727813
 
 
 def log(*a):
