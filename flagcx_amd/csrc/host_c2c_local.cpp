@@ -1,0 +1,665 @@
+// host_c2c_local.cpp - replays C2C plans on ONE GPU that holds the buffers of all
+// simulated ranks, using only the library's own C ABI (flagcxLocalReduce*,
+// flagcxLocalMemcpy, flagcxLocalRefresh).
+//
+// A plan is what flagcxC2cPlanner keeps per rank (flagcx/core/c2c_algo.h:205-268):
+// step counts, one refresh function and four step tables of homo / hetero
+// functions, in the XML format its exportXml / importXml use
+// (flagcx/core/c2c_algo.cc:973-1087, serializers in flagcx/core/c2c_ir.h:62-176).
+// The field names below are the reference's.  Execution follows
+// flagcxC2cPlanner::execute (c2c_algo.cc:2142-2290) stage by stage, with all
+// ranks advanced in lock step:
+//   - a homo function is the same collective on every member of a cluster
+//     (homoType 1: on the cluster's inter-ranks only, c2c_algo.cc:293-295); where
+//     the reference calls the vendor CCL (c2c_algo.cc:309-481) the members'
+//     buffers are reduced / copied by the local kernels, folding in homo-rank
+//     order 0..n-1;
+//   - a hetero function's P2P ops (c2c_algo.cc:565-584) are matched send-to-recv
+//     between ranks and become device copies;
+//   - the refresh function is flagcxLocalRefresh (c2c_algo.cc:586-608).
+// Two rank-local primitives the reference's plan DSL reserves but its executor
+// lacks (LocCpy = 12, LocRed = 13, flagcx/tools/utils.py:43-44) are accepted as
+// commOp values: LocCpy copies send[sendOffset..) to recv[recvOffset..); LocRed
+// sets recv[recvOffset..) = OP(send[sendOffset..), recv[recvOffset..)).
+//
+// Not replayed (flagcxNotSupported): Send/Recv homo functions of homoType 1, which
+// need the planner's inter-rank buffer lists (c2c_algo.cc:386-400,434-452), and
+// AlltoAllv.
+#include "../../include/flagcx_amd.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace {
+
+enum { kLocCpy = 12, kLocRed = 13 };
+
+struct HomoFunc {
+  int rootRank_ = -1, sendType_ = 0, recvType_ = 1;
+  size_t sendOffset_ = 0, recvOffset_ = 0, count_ = 0;
+  int homoType_ = 0;
+  int commOp_ = flagcxCommNoOp;
+};
+struct P2pOp {
+  int rank_ = 0, peerRank_ = 0;
+  size_t offset_ = 0, count_ = 0;
+  int isRecv_ = 0;
+};
+struct HeteroFunc {
+  std::vector<P2pOp> p2pOps_;
+};
+struct RefreshFunc {
+  int bufftype_ = -1;
+  size_t start_ = 0, offset_ = 0, count_ = 0, totalCount_ = 0;
+  int redOp_ = flagcxSum;
+};
+struct RankPlan {
+  size_t nchunks_ = 1;
+  int nSeqPreSteps_ = 0, nPipePreSteps_ = 0, nSeqInterSteps_ = 0, nPipePostSteps_ = 0, nSeqPostSteps_ = 0;
+  RefreshFunc refreshFunc_;
+  std::vector<std::vector<HomoFunc>> preHomoFuncSteps_, homoInterFuncSteps_, postHomoFuncSteps_;
+  std::vector<std::vector<HeteroFunc>> heteroFuncSteps_;
+};
+
+// ------------------------------------------------------------ tiny XML tree
+struct Node {
+  std::string name, text;
+  std::vector<Node> kids;
+  const Node *child(const char *n) const {
+    for (auto &k : kids) if (k.name == n) return &k;
+    return nullptr;
+  }
+  long long num(const char *n, long long dflt = 0) const {
+    const Node *c = child(n);
+    return c ? strtoll(c->text.c_str(), nullptr, 10) : dflt;
+  }
+  size_t size(const char *n) const {
+    const Node *c = child(n);
+    return c ? (size_t)strtoull(c->text.c_str(), nullptr, 10) : 0;
+  }
+};
+
+static bool parseNode(const std::string &s, size_t &pos, Node &out) {
+  // expects pos at '<' of an opening (or self-closing) tag
+  size_t gt = s.find('>', pos);
+  if (gt == std::string::npos) return false;
+  std::string tag = s.substr(pos + 1, gt - pos - 1);
+  pos = gt + 1;
+  if (!tag.empty() && tag.back() == '/') {
+    out.name = tag.substr(0, tag.size() - 1);
+    return true;
+  }
+  out.name = tag;
+  for (;;) {
+    size_t lt = s.find('<', pos);
+    if (lt == std::string::npos) return false;
+    out.text += s.substr(pos, lt - pos);
+    if (s.compare(lt, 2, "</") == 0) {
+      size_t end = s.find('>', lt);
+      if (end == std::string::npos || s.substr(lt + 2, end - lt - 2) != out.name) return false;
+      pos = end + 1;
+      // trim
+      size_t a = out.text.find_first_not_of(" \t\r\n"), b = out.text.find_last_not_of(" \t\r\n");
+      out.text = a == std::string::npos ? "" : out.text.substr(a, b - a + 1);
+      return true;
+    }
+    pos = lt;
+    Node kid;
+    if (!parseNode(s, pos, kid)) return false;
+    out.kids.push_back(kid);
+  }
+}
+
+static HomoFunc homoFrom(const Node &n, size_t chunksize) {
+  HomoFunc f;
+  f.rootRank_ = (int)n.num("rootRank", -1);
+  f.sendType_ = (int)n.num("sendType");
+  f.recvType_ = (int)n.num("recvType");
+  f.sendOffset_ = n.size("sendOffset") * chunksize;
+  f.recvOffset_ = n.size("recvOffset") * chunksize;
+  f.count_ = n.size("count") * chunksize;
+  f.homoType_ = (int)n.num("homoType");
+  f.commOp_ = (int)n.num("commOp");
+  return f;
+}
+
+static void homoSteps(const Node *table, size_t chunksize, std::vector<std::vector<HomoFunc>> &out) {
+  out.clear();
+  if (!table) return;
+  for (auto &step : table->kids) {
+    if (step.name != "Step") continue;
+    std::vector<HomoFunc> fs;
+    for (auto &f : step.kids) if (f.name == "HomoFunc") fs.push_back(homoFrom(f, chunksize));
+    out.push_back(fs);
+  }
+}
+
+static void heteroSteps(const Node *table, size_t chunksize, std::vector<std::vector<HeteroFunc>> &out) {
+  out.clear();
+  if (!table) return;
+  for (auto &step : table->kids) {
+    if (step.name != "Step") continue;
+    std::vector<HeteroFunc> fs;
+    for (auto &f : step.kids) {
+      if (f.name != "HeteroFunc") continue;
+      HeteroFunc h;
+      for (auto &o : f.kids) {
+        if (o.name != "P2pOp") continue;
+        P2pOp p;
+        p.rank_ = (int)o.num("rank");
+        p.peerRank_ = (int)o.num("peerRank");
+        p.offset_ = o.size("offset") * chunksize;
+        p.count_ = o.size("count") * chunksize;
+        p.isRecv_ = (int)o.num("isRecv");
+        h.p2pOps_.push_back(p);
+      }
+      fs.push_back(h);
+    }
+    out.push_back(fs);
+  }
+}
+
+static void writeHomoSteps(FILE *f, const char *tag, const std::vector<std::vector<HomoFunc>> &steps, size_t cs) {
+  // layout of serializeFunc2DVector / serializeHomoFunc (c2c_ir.h:76-92,121-144)
+  fprintf(f, "  <%s>\n", tag);
+  for (auto &step : steps) {
+    if (step.empty()) { fprintf(f, "    <Step/>\n"); continue; }
+    fprintf(f, "    <Step>\n");
+    for (auto &h : step) {
+      fprintf(f, "      <HomoFunc>\n");
+      fprintf(f, "        <rootRank>%d</rootRank>\n", h.rootRank_);
+      fprintf(f, "        <sendType>%d</sendType>\n", h.sendType_);
+      fprintf(f, "        <recvType>%d</recvType>\n", h.recvType_);
+      fprintf(f, "        <sendOffset>%zu</sendOffset>\n", h.sendOffset_ / cs);
+      fprintf(f, "        <recvOffset>%zu</recvOffset>\n", h.recvOffset_ / cs);
+      fprintf(f, "        <count>%zu</count>\n", h.count_ / cs);
+      fprintf(f, "        <homoType>%d</homoType>\n", h.homoType_);
+      fprintf(f, "        <commOp>%d</commOp>\n", h.commOp_);
+      fprintf(f, "      </HomoFunc>\n");
+    }
+    fprintf(f, "    </Step>\n");
+  }
+  fprintf(f, "  </%s>\n", tag);
+}
+
+} // namespace
+
+struct flagcxLocalPlan {
+  int nranks = 0;
+  std::vector<int> clusterOf, isInter;
+  std::vector<std::vector<int>> clusterRanks, clusterInterRanks; // global ranks, ascending
+  std::vector<int> homoRank, homoInterRank;                      // per global rank (-1: none)
+  size_t totalCount = 0;
+  int commOp = flagcxCommNoOp, redOp = flagcxSum;
+  std::vector<RankPlan> ranks;
+  int algorithm = 2; // flagcxAlgoInput: what importXml sets (c2c_algo.h:15-19, c2c_algo.cc:974)
+  bool loaded = false;
+  char err[256] = "";
+};
+
+namespace {
+
+static flagcxResult_t planFail(flagcxLocalPlan *p, flagcxResult_t code, const char *fmt, const char *a = "",
+                               long long b = 0, long long c = 0) {
+  snprintf(p->err, sizeof(p->err), fmt, a, b, c);
+  return code;
+}
+
+struct Bufs {
+  const void *const *send;
+  void *const *recv;
+  void *const *scratch;
+};
+
+static char *pick(const Bufs &b, int rank, int type) {
+  // sendType_: 0 user send, 1 recv, 2 scratch; recvType_: 1 recv, else scratch (c2c_algo.cc:297-300)
+  if (type == 0) return (char *)const_cast<void *>(b.send[rank]);
+  if (type == 1) return (char *)b.recv[rank];
+  return b.scratch ? (char *)b.scratch[rank] : nullptr;
+}
+
+#define LCHECK(call)                                                           \
+  do {                                                                         \
+    flagcxResult_t r_ = (call);                                                \
+    if (r_ != flagcxSuccess) return r_;                                        \
+  } while (0)
+
+// One homo function slot (step s, index i of one table) across all ranks.
+static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const HomoFunc *> &fn, const Bufs &b,
+                                  flagcxDataType_t dt, int root, flagcxStream_t stream) {
+  const size_t ts = flagcxLocalGetDataTypeSize(dt);
+  const int ncl = (int)p->clusterRanks.size();
+  for (int cl = 0; cl < ncl; cl++) {
+    // members that hold a function in this slot; homoType 1 runs on inter-ranks only
+    std::vector<int> mem;
+    const HomoFunc *first = nullptr;
+    for (int r : p->clusterRanks[cl]) {
+      const HomoFunc *f = fn[r];
+      if (!f) continue;
+      if (f->homoType_ == 1 && p->homoInterRank[r] == -1) continue; // c2c_algo.cc:293-295
+      if (!first) first = f;
+      mem.push_back(r);
+    }
+    if (!first) continue;
+    const int op = first->commOp_;
+    // rank-local primitives need no peers
+    if (op == kLocCpy || op == kLocRed) {
+      for (int r : mem) {
+        const HomoFunc *f = fn[r];
+        char *s = pick(b, r, f->sendType_), *d = pick(b, r, f->recvType_ == 1 ? 1 : 2);
+        if (!s || !d) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+        s += f->sendOffset_ * ts;
+        d += f->recvOffset_ * ts;
+        if (op == kLocCpy) {
+          LCHECK(flagcxLocalMemcpy(d, s, f->count_ * ts, stream));
+        } else {
+          const void *srcs[2] = {d, s}; // acc = recv slice; acc = OP(send slice, acc)
+          LCHECK(flagcxLocalReduce(srcs, 2, d, f->count_, dt, (flagcxRedOp_t)p->redOp, stream));
+        }
+      }
+      continue;
+    }
+    // the communicator the reference would use: homoInterComm for homoType 1, else homo_comm
+    const std::vector<int> &comm = first->homoType_ == 1 ? p->clusterInterRanks[cl] : p->clusterRanks[cl];
+    const int n = (int)comm.size();
+    std::vector<char *> S(n, nullptr), D(n, nullptr);
+    std::vector<size_t> cnt(n, 0);
+    for (int h = 0; h < n; h++) {
+      const int r = comm[h];
+      const HomoFunc *f = fn[r];
+      if (!f || f->commOp_ != op)
+        return planFail(p, flagcxInvalidUsage, "rank %s%lld has no matching homo function (commOp %lld)", "", r, op);
+      char *s = pick(b, r, f->sendType_), *d = pick(b, r, f->recvType_ == 1 ? 1 : 2);
+      if (!s || !d) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+      S[h] = s + f->sendOffset_ * ts;
+      D[h] = d + f->recvOffset_ * ts;
+      cnt[h] = f->count_;
+    }
+    const size_t count = cnt[0];
+    auto homoRoot = [&](const HomoFunc *f) { return f->rootRank_ == -1 ? root : f->rootRank_; };
+    const flagcxRedOp_t rop = (flagcxRedOp_t)p->redOp;
+    switch (op) {
+      case flagcxCommOpReduce: {
+        const int rt = homoRoot(first);
+        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
+        LCHECK(flagcxLocalReduce((const void *const *)S.data(), n, D[rt], count, dt, rop, stream));
+        break;
+      }
+      case flagcxCommOpAllReduce: {
+        // every member ends with the same bytes: reduce once, then copy
+        LCHECK(flagcxLocalReduce((const void *const *)S.data(), n, D[0], count, dt, rop, stream));
+        for (int h = 1; h < n; h++) LCHECK(flagcxLocalMemcpy(D[h], D[0], count * ts, stream));
+        break;
+      }
+      case flagcxCommOpReduceScatter: {
+        // member h receives the fold of everybody's h-th block; one batch launch
+        std::vector<std::vector<const void *>> srcs(n, std::vector<const void *>(n));
+        std::vector<flagcxLocalReduceDesc> descs(n);
+        for (int h = 0; h < n; h++) {
+          for (int j = 0; j < n; j++) srcs[h][j] = S[j] + (size_t)h * count * ts;
+          descs[h] = {srcs[h].data(), D[h], count};
+        }
+        LCHECK(flagcxLocalReduceBatch(descs.data(), n, n, dt, rop, stream));
+        break;
+      }
+      case flagcxCommOpAllGather:
+        for (int h = 0; h < n; h++)
+          for (int j = 0; j < n; j++)
+            LCHECK(flagcxLocalMemcpy(D[h] + (size_t)j * count * ts, S[j], count * ts, stream));
+        break;
+      case flagcxCommOpGather: {
+        const int rt = homoRoot(first);
+        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
+        for (int j = 0; j < n; j++) LCHECK(flagcxLocalMemcpy(D[rt] + (size_t)j * count * ts, S[j], count * ts, stream));
+        break;
+      }
+      case flagcxCommOpScatter: {
+        const int rt = homoRoot(first);
+        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
+        for (int h = 0; h < n; h++) LCHECK(flagcxLocalMemcpy(D[h], S[rt] + (size_t)h * count * ts, count * ts, stream));
+        break;
+      }
+      case flagcxCommOpBroadcast: {
+        const int rt = homoRoot(first);
+        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
+        for (int h = 0; h < n; h++) LCHECK(flagcxLocalMemcpy(D[h], S[rt], count * ts, stream));
+        break;
+      }
+      case flagcxCommOpAlltoAll:
+        for (int h = 0; h < n; h++)
+          for (int j = 0; j < n; j++)
+            LCHECK(flagcxLocalMemcpy(D[h] + (size_t)j * count * ts, S[j] + (size_t)h * count * ts, count * ts, stream));
+        break;
+      case flagcxCommNoOp:
+        break;
+      default:
+        return planFail(p, flagcxNotSupported, "homo function commOp %s%lld is not replayed", "", op);
+    }
+  }
+  return flagcxSuccess;
+}
+
+static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream);
+
+static flagcxResult_t runHomoStep(flagcxLocalPlan *p, std::vector<std::vector<HomoFunc>> RankPlan::*table, int s,
+                                  const Bufs &b, flagcxDataType_t dt, int root, flagcxStream_t stream,
+                                  int onlyIndex = -1, bool refreshBeforeEach = false) {
+  size_t width = 0;
+  for (auto &rp : p->ranks) {
+    auto &t = rp.*table;
+    if (s < (int)t.size() && t[s].size() > width) width = t[s].size();
+  }
+  for (size_t i = 0; i < width; i++) {
+    if (onlyIndex >= 0 && (int)i != onlyIndex) continue;
+    if (refreshBeforeEach) LCHECK(runRefresh(p, b, dt, stream));
+    std::vector<const HomoFunc *> fn(p->nranks, nullptr);
+    for (int r = 0; r < p->nranks; r++) {
+      auto &t = p->ranks[r].*table;
+      if (s < (int)t.size() && i < t[s].size()) fn[r] = &t[s][i];
+    }
+    LCHECK(runHomoSlot(p, fn, b, dt, root, stream));
+  }
+  return flagcxSuccess;
+}
+
+// Hetero function i of step s on every rank: match each send with the peer's
+// next unmatched receive from that sender (order of appearance).
+static flagcxResult_t runHeteroSlot(flagcxLocalPlan *p, int s, int i, const std::vector<char *> &sendTmp,
+                                    const std::vector<char *> &recvTmp, flagcxDataType_t dt,
+                                    flagcxStream_t stream) {
+  const size_t ts = flagcxLocalGetDataTypeSize(dt);
+  std::map<std::pair<int, int>, std::vector<const P2pOp *>> recvs; // (receiver, sender) -> ops
+  for (int r = 0; r < p->nranks; r++) {
+    auto &t = p->ranks[r].heteroFuncSteps_;
+    if (s >= (int)t.size() || i >= (int)t[s].size()) continue;
+    for (auto &op : t[s][i].p2pOps_)
+      if (op.isRecv_) recvs[{r, op.peerRank_}].push_back(&op);
+  }
+  std::map<std::pair<int, int>, size_t> used;
+  for (int r = 0; r < p->nranks; r++) {
+    auto &t = p->ranks[r].heteroFuncSteps_;
+    if (s >= (int)t.size() || i >= (int)t[s].size()) continue;
+    for (auto &op : t[s][i].p2pOps_) {
+      if (op.isRecv_) continue;
+      const int peer = op.peerRank_;
+      if (peer < 0 || peer >= p->nranks) return planFail(p, flagcxInvalidArgument, "P2pOp peer %s%lld out of range", "", peer);
+      auto key = std::make_pair(peer, r);
+      size_t &u = used[key];
+      auto it = recvs.find(key);
+      if (it == recvs.end() || u >= it->second.size())
+        return planFail(p, flagcxInvalidUsage, "send %s%lld -> %lld has no matching receive", "", r, peer);
+      const P2pOp *rv = it->second[u++];
+      if (rv->count_ != op.count_)
+        return planFail(p, flagcxInvalidUsage, "send/recv count mismatch between ranks %s%lld and %lld", "", r, peer);
+      LCHECK(flagcxLocalMemcpy(recvTmp[peer] + rv->offset_ * ts, sendTmp[r] + op.offset_ * ts, op.count_ * ts, stream));
+    }
+  }
+  for (auto &kv : recvs)
+    if (used[kv.first] != kv.second.size())
+      return planFail(p, flagcxInvalidUsage, "receive on rank %s%lld from %lld has no matching send", "", kv.first.first, kv.first.second);
+  return flagcxSuccess;
+}
+
+static size_t heteroWidth(flagcxLocalPlan *p, int s) {
+  size_t w = 0;
+  for (auto &rp : p->ranks)
+    if (s < (int)rp.heteroFuncSteps_.size() && rp.heteroFuncSteps_[s].size() > w) w = rp.heteroFuncSteps_[s].size();
+  return w;
+}
+
+static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream) {
+  for (int r = 0; r < p->nranks; r++) {
+    const RefreshFunc &f = p->ranks[r].refreshFunc_;
+    // bufftype -1 resolves to recv (1) without scratch, scratch (2) with it (c2c_algo.cc:2156-2164)
+    int bt = f.bufftype_;
+    if (bt == -1) bt = (b.scratch && b.scratch[r]) ? 2 : 1;
+    void *buff = bt == 1 ? b.recv[r] : (b.scratch ? b.scratch[r] : nullptr);
+    if (f.totalCount_ == 0) continue;
+    if (!buff) return planFail(p, flagcxInvalidArgument, "refresh needs a scratch buffer%s", "");
+    LCHECK(flagcxLocalRefresh(buff, f.start_, f.offset_, f.count_, f.totalCount_, dt, (flagcxRedOp_t)f.redOp_, stream));
+  }
+  return flagcxSuccess;
+}
+
+} // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+flagcxResult_t flagcxLocalPlanCreate(flagcxLocalPlan **plan, int nranks, const int *clusterIds,
+                                     const int *isInterRank, size_t totalCount, flagcxCommOp_t commOp,
+                                     flagcxRedOp_t redOp) {
+  if (!plan || nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS || !clusterIds || totalCount == 0)
+    return flagcxInvalidArgument;
+  flagcxLocalPlan *p = new flagcxLocalPlan();
+  p->nranks = nranks;
+  p->totalCount = totalCount;
+  p->commOp = (int)commOp;
+  p->redOp = (int)redOp;
+  int ncl = 0;
+  for (int r = 0; r < nranks; r++) {
+    if (clusterIds[r] < 0 || clusterIds[r] >= nranks) { delete p; return flagcxInvalidArgument; }
+    if (clusterIds[r] + 1 > ncl) ncl = clusterIds[r] + 1;
+  }
+  p->clusterOf.assign(clusterIds, clusterIds + nranks);
+  p->isInter.resize(nranks);
+  p->clusterRanks.resize(ncl);
+  p->clusterInterRanks.resize(ncl);
+  p->homoRank.assign(nranks, -1);
+  p->homoInterRank.assign(nranks, -1);
+  for (int r = 0; r < nranks; r++) {
+    const int cl = clusterIds[r];
+    p->isInter[r] = isInterRank ? (isInterRank[r] != 0) : 1;
+    p->homoRank[r] = (int)p->clusterRanks[cl].size();
+    p->clusterRanks[cl].push_back(r);
+    if (p->isInter[r]) {
+      p->homoInterRank[r] = (int)p->clusterInterRanks[cl].size();
+      p->clusterInterRanks[cl].push_back(r);
+    }
+  }
+  p->ranks.resize(nranks);
+  *plan = p;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalPlanDestroy(flagcxLocalPlan *plan) {
+  delete plan;
+  return flagcxSuccess;
+}
+
+const char *flagcxLocalPlanGetLastError(flagcxLocalPlan *plan) { return plan ? plan->err : ""; }
+
+// 0 sequential, 1 pipeline, 2 input (flagcxAlgorithm_t, c2c_algo.h:15-19): selects
+// where execute() refreshes, for plans exported by a planner that was not in
+// input mode.
+flagcxResult_t flagcxLocalPlanSetAlgorithm(flagcxLocalPlan *plan, int algorithm) {
+  if (!plan || algorithm < 0 || algorithm > 2) return flagcxInvalidArgument;
+  plan->algorithm = algorithm;
+  return flagcxSuccess;
+}
+
+// Reads <prefix>_<rank>.xml for every rank (file naming of importXml, c2c_algo.cc:975-976).
+flagcxResult_t flagcxLocalPlanImportXml(flagcxLocalPlan *p, const char *prefix) {
+  if (!p || !prefix) return flagcxInvalidArgument;
+  for (int r = 0; r < p->nranks; r++) {
+    char filename[512];
+    snprintf(filename, sizeof(filename), "%s_%d.xml", prefix, r);
+    FILE *f = fopen(filename, "r");
+    if (!f) return planFail(p, flagcxInternalError, "cannot open %s", filename); // same code as the reference
+    std::string text;
+    char buf[4096];
+    size_t got;
+    while ((got = fread(buf, 1, sizeof(buf), f)) > 0) text.append(buf, got);
+    fclose(f);
+    size_t pos = text.find('<');
+    Node rootNode;
+    if (pos == std::string::npos || !parseNode(text, pos, rootNode) || rootNode.name != "FlagcxC2cPlanner")
+      return planFail(p, flagcxInvalidArgument, "%s is not a FlagcxC2cPlanner document", filename);
+    RankPlan &rp = p->ranks[r];
+    rp.nchunks_ = rootNode.size("nChunks");
+    if (rp.nchunks_ == 0 || p->totalCount % rp.nchunks_)
+      return planFail(p, flagcxInvalidArgument, "%s: nChunks must divide the total count", filename);
+    const size_t cs = p->totalCount / rp.nchunks_; // chunksize = totalCount_ / nchunks_ (c2c_algo.cc:989)
+    rp.nSeqPreSteps_ = (int)rootNode.num("nSeqPreSteps");
+    rp.nPipePreSteps_ = (int)rootNode.num("nPipePreSteps");
+    rp.nSeqInterSteps_ = (int)rootNode.num("nSeqInterSteps");
+    rp.nPipePostSteps_ = (int)rootNode.num("nPipePostSteps");
+    rp.nSeqPostSteps_ = (int)rootNode.num("nSeqPostSteps");
+    if (const Node *rf = rootNode.child("RefreshFunc")) {
+      rp.refreshFunc_.bufftype_ = (int)rf->num("buffType", -1);
+      rp.refreshFunc_.start_ = rf->size("start") * cs;
+      rp.refreshFunc_.offset_ = rf->size("offset") * cs;
+      rp.refreshFunc_.count_ = rf->size("count") * cs;
+      rp.refreshFunc_.totalCount_ = rf->size("totalCount") * cs;
+      rp.refreshFunc_.redOp_ = (int)rf->num("redOp");
+    }
+    homoSteps(rootNode.child("PreHomoFuncSteps"), cs, rp.preHomoFuncSteps_);
+    heteroSteps(rootNode.child("HeteroFuncSteps"), cs, rp.heteroFuncSteps_);
+    homoSteps(rootNode.child("HomoInterFuncSteps"), cs, rp.homoInterFuncSteps_);
+    homoSteps(rootNode.child("PostHomoFuncSteps"), cs, rp.postHomoFuncSteps_);
+    // the executor indexes the tables by these counts
+    if ((int)rp.preHomoFuncSteps_.size() < rp.nSeqPreSteps_ + rp.nPipePreSteps_ ||
+        (int)rp.heteroFuncSteps_.size() < rp.nPipePreSteps_ + rp.nSeqInterSteps_ + rp.nPipePostSteps_ ||
+        (int)rp.postHomoFuncSteps_.size() < rp.nPipePostSteps_ + rp.nSeqPostSteps_)
+      return planFail(p, flagcxInvalidArgument, "%s: step tables shorter than the step counts", filename);
+    rp.homoInterFuncSteps_.resize(rp.heteroFuncSteps_.size());
+  }
+  for (int r = 1; r < p->nranks; r++) {
+    const RankPlan &a = p->ranks[0], &b = p->ranks[r];
+    if (a.nSeqPreSteps_ != b.nSeqPreSteps_ || a.nPipePreSteps_ != b.nPipePreSteps_ ||
+        a.nSeqInterSteps_ != b.nSeqInterSteps_ || a.nPipePostSteps_ != b.nPipePostSteps_ ||
+        a.nSeqPostSteps_ != b.nSeqPostSteps_)
+      return planFail(p, flagcxInvalidUsage, "ranks disagree on the step counts%s", "");
+  }
+  p->loaded = true;
+  return flagcxSuccess;
+}
+
+// Writes <prefix>_<rank>.xml in the layout of exportXml (c2c_algo.cc:1050-1087).
+flagcxResult_t flagcxLocalPlanExportXml(flagcxLocalPlan *p, const char *prefix) {
+  if (!p || !prefix || !p->loaded) return flagcxInvalidArgument;
+  for (int r = 0; r < p->nranks; r++) {
+    char filename[512];
+    snprintf(filename, sizeof(filename), "%s_%d.xml", prefix, r);
+    FILE *f = fopen(filename, "w");
+    if (!f) return planFail(p, flagcxInternalError, "cannot open %s", filename);
+    const RankPlan &rp = p->ranks[r];
+    const size_t cs = p->totalCount / rp.nchunks_;
+    fprintf(f, "<FlagcxC2cPlanner>\n");
+    fprintf(f, "  <nChunks>%zu</nChunks>\n", rp.nchunks_);
+    fprintf(f, "  <nSeqPreSteps>%d</nSeqPreSteps>\n", rp.nSeqPreSteps_);
+    fprintf(f, "  <nPipePreSteps>%d</nPipePreSteps>\n", rp.nPipePreSteps_);
+    fprintf(f, "  <nSeqInterSteps>%d</nSeqInterSteps>\n", rp.nSeqInterSteps_);
+    fprintf(f, "  <nPipePostSteps>%d</nPipePostSteps>\n", rp.nPipePostSteps_);
+    fprintf(f, "  <nSeqPostSteps>%d</nSeqPostSteps>\n", rp.nSeqPostSteps_);
+    fprintf(f, "  <RefreshFunc>\n");
+    fprintf(f, "    <buffType>%d</buffType>\n", rp.refreshFunc_.bufftype_);
+    fprintf(f, "    <start>%zu</start>\n", rp.refreshFunc_.start_ / cs);
+    fprintf(f, "    <offset>%zu</offset>\n", rp.refreshFunc_.offset_ / cs);
+    fprintf(f, "    <count>%zu</count>\n", rp.refreshFunc_.count_ / cs);
+    fprintf(f, "    <totalCount>%zu</totalCount>\n", rp.refreshFunc_.totalCount_ / cs);
+    fprintf(f, "    <redOp>%d</redOp>\n", rp.refreshFunc_.redOp_);
+    fprintf(f, "  </RefreshFunc>\n");
+    writeHomoSteps(f, "PreHomoFuncSteps", rp.preHomoFuncSteps_, cs);
+    fprintf(f, "  <HeteroFuncSteps>\n");
+    for (auto &step : rp.heteroFuncSteps_) {
+      if (step.empty()) { fprintf(f, "    <Step/>\n"); continue; }
+      fprintf(f, "    <Step>\n");
+      for (auto &h : step) {
+        fprintf(f, "      <HeteroFunc>\n");
+        for (auto &o : h.p2pOps_) {
+          fprintf(f, "        <P2pOp>\n");
+          fprintf(f, "          <rank>%d</rank>\n", o.rank_);
+          fprintf(f, "          <peerRank>%d</peerRank>\n", o.peerRank_);
+          fprintf(f, "          <offset>%zu</offset>\n", o.offset_ / cs);
+          fprintf(f, "          <count>%zu</count>\n", o.count_ / cs);
+          fprintf(f, "          <isRecv>%d</isRecv>\n", o.isRecv_);
+          fprintf(f, "        </P2pOp>\n");
+        }
+        fprintf(f, "      </HeteroFunc>\n");
+      }
+      fprintf(f, "    </Step>\n");
+    }
+    fprintf(f, "  </HeteroFuncSteps>\n");
+    writeHomoSteps(f, "HomoInterFuncSteps", rp.homoInterFuncSteps_, cs);
+    writeHomoSteps(f, "PostHomoFuncSteps", rp.postHomoFuncSteps_, cs);
+    fprintf(f, "</FlagcxC2cPlanner>\n");
+    fclose(f);
+  }
+  return flagcxSuccess;
+}
+
+// sendbuffs / recvbuffs / scratchbuffs: host arrays with one device pointer per
+// rank (scratchbuffs may be NULL when no function or refresh names scratch).
+flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan *p, const void *const *sendbuffs, void *const *recvbuffs,
+                                      void *const *scratchbuffs, flagcxDataType_t datatype, int root,
+                                      flagcxStream_t stream) {
+  if (!p || !sendbuffs || !recvbuffs) return flagcxInvalidArgument;
+  if (!p->loaded) return planFail(p, flagcxInvalidUsage, "no plan imported%s", "");
+  // redOp validation of flagcxC2cPlanner::execute (c2c_algo.cc:2047-2053)
+  if (p->redOp != flagcxRedNoOp && p->redOp != flagcxSum && p->redOp != flagcxMax && p->redOp != flagcxMin)
+    return planFail(p, flagcxNotSupported, "Unsupported reduction operation %s%lld", "", p->redOp);
+  if (!flagcxLocalGetDataTypeSize(datatype)) return planFail(p, flagcxInvalidArgument, "unsupported data type%s", "");
+  for (int r = 0; r < p->nranks; r++)
+    if (!sendbuffs[r] || !recvbuffs[r]) return planFail(p, flagcxInvalidArgument, "rank %s%lld has a NULL buffer", "", r);
+  const Bufs b{sendbuffs, recvbuffs, scratchbuffs};
+  const RankPlan &c = p->ranks[0];
+  // staging buffers of the hetero functions (c2c_algo.cc:2129-2137)
+  std::vector<char *> recvTmp(p->nranks), sendTmp(p->nranks);
+  for (int r = 0; r < p->nranks; r++) {
+    char *scratch = scratchbuffs ? (char *)scratchbuffs[r] : nullptr;
+    recvTmp[r] = scratch ? scratch : (char *)recvbuffs[r];
+    const bool fromSend = p->commOp == flagcxCommOpAlltoAll || p->commOp == flagcxCommOpAlltoAllv ||
+                          (p->commOp == flagcxCommOpScatter && r == root);
+    sendTmp[r] = fromSend ? (char *)const_cast<void *>(sendbuffs[r]) : recvTmp[r];
+  }
+  const bool anyPipe = c.nPipePreSteps_ > 0 || c.nPipePostSteps_ > 0;
+  // when the reference refreshes around sequential steps (c2c_algo.cc:2205-2208,2226-2229,2276-2279)
+  const bool refreshSeq = p->algorithm == 0 || !anyPipe;
+  const bool refreshAfterInter = p->algorithm == 1 && anyPipe;
+
+  // sequential preHomoFunc steps
+  for (int s = 0; s < c.nSeqPreSteps_; s++)
+    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, s, b, datatype, root, stream));
+  LCHECK(runRefresh(p, b, datatype, stream));
+  // pipelined preHomoFunc + heteroFunc steps
+  for (int s = 0; s < c.nPipePreSteps_; s++) {
+    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, c.nSeqPreSteps_ + s, b, datatype, root, stream));
+    for (size_t i = 0; i < heteroWidth(p, s); i++) {
+      LCHECK(runHeteroSlot(p, s, (int)i, sendTmp, recvTmp, datatype, stream));
+      LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, s, b, datatype, root, stream, (int)i));
+      LCHECK(runRefresh(p, b, datatype, stream));
+    }
+  }
+  // sequential heteroFunc steps
+  for (int s = 0; s < c.nSeqInterSteps_; s++) {
+    const int hs = c.nPipePreSteps_ + s;
+    for (size_t i = 0; i < heteroWidth(p, hs); i++) {
+      if (refreshSeq) LCHECK(runRefresh(p, b, datatype, stream));
+      LCHECK(runHeteroSlot(p, hs, (int)i, sendTmp, recvTmp, datatype, stream));
+      LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, root, stream, (int)i));
+      if (refreshAfterInter) LCHECK(runRefresh(p, b, datatype, stream));
+    }
+  }
+  // pipelined heteroFunc + postHomoFunc steps
+  for (int s = 0; s < c.nPipePostSteps_; s++) {
+    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, s, b, datatype, root, stream));
+    const int hs = c.nPipePreSteps_ + c.nSeqInterSteps_ + s;
+    for (size_t i = 0; i < heteroWidth(p, hs); i++) {
+      LCHECK(runHeteroSlot(p, hs, (int)i, sendTmp, recvTmp, datatype, stream));
+      LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, root, stream, (int)i));
+    }
+  }
+  // sequential postHomoFunc steps
+  for (int s = 0; s < c.nSeqPostSteps_; s++)
+    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, c.nPipePostSteps_ + s, b, datatype, root, stream, -1,
+                       refreshSeq));
+  return flagcxSuccess;
+}
+
+} // extern "C"
+#pragma GCC visibility pop

@@ -96,6 +96,8 @@ EXPORTS = [
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
     "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
     "flagcxLocalReduceBatch", "flagcxLocalReduceTriggers",
+    "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
+    "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
 ]
 
 
@@ -138,6 +140,14 @@ def lib():
         L.flagcxLocalCopyFunc.argtypes = [sp, C.POINTER(CopyArgs)]
         L.flagcxLocalReduceBatch.argtypes = [C.POINTER(ReduceDesc), i, i, i, i, sp]
         L.flagcxLocalReduceTriggers.argtypes = [C.POINTER(ReduceTrigger), i, sp]
+        L.flagcxLocalPlanCreate.argtypes = [C.POINTER(vp), i, C.POINTER(i), C.POINTER(i), sz, i, i]
+        L.flagcxLocalPlanDestroy.argtypes = [vp]
+        L.flagcxLocalPlanImportXml.argtypes = [vp, C.c_char_p]
+        L.flagcxLocalPlanExportXml.argtypes = [vp, C.c_char_p]
+        L.flagcxLocalPlanSetAlgorithm.argtypes = [vp, i]
+        L.flagcxLocalPlanExecute.argtypes = [vp, pp, pp, pp, i, i, sp]
+        L.flagcxLocalPlanGetLastError.restype = C.c_char_p
+        L.flagcxLocalPlanGetLastError.argtypes = [vp]
         L.flagcxLocalSetMaxSpinCount.restype = None
         L.flagcxLocalSetMaxSpinCount.argtypes = [C.c_int64]
         for name in ("deviceAsyncStore", "deviceAsyncLoad"):
@@ -276,3 +286,48 @@ def pack_list(dst_ptr, src_ptrs, nbytes, stream="current"):
 def unpack_list(dst_ptrs, src_ptr, nbytes, stream="current"):
     st = current_stream() if stream == "current" else stream
     check(lib().flagcxLocalUnpackList(_ptr_array(dst_ptrs), src_ptr, len(dst_ptrs), nbytes, _sref(st)))
+
+
+class Plan:
+    """A set of per-rank C2C plans replayed on one GPU (flagcxLocalPlan*)."""
+
+    def __init__(self, cluster_ids, total_count, comm_op, red_op, is_inter=None):
+        n = len(cluster_ids)
+        self.nranks = n
+        self._h = C.c_void_p()
+        cl = (C.c_int * n)(*cluster_ids)
+        it = (C.c_int * n)(*is_inter) if is_inter is not None else None
+        rc = lib().flagcxLocalPlanCreate(C.byref(self._h), n, cl, it, total_count, int(comm_op), int(red_op))
+        if rc:
+            raise FlagcxError(rc, "flagcxLocalPlanCreate")
+
+    def _check(self, rc):
+        if rc:
+            raise FlagcxError(rc, lib().flagcxLocalPlanGetLastError(self._h).decode() or
+                              lib().flagcxLocalGetLastError().decode())
+
+    def import_xml(self, prefix):
+        self._check(lib().flagcxLocalPlanImportXml(self._h, prefix.encode()))
+
+    def export_xml(self, prefix):
+        self._check(lib().flagcxLocalPlanExportXml(self._h, prefix.encode()))
+
+    def set_algorithm(self, algo):
+        self._check(lib().flagcxLocalPlanSetAlgorithm(self._h, algo))
+
+    def execute(self, send_ptrs, recv_ptrs, scratch_ptrs, dtype, root=-1, stream="current"):
+        st = current_stream() if stream == "current" else stream
+        sc = _ptr_array(scratch_ptrs) if scratch_ptrs is not None else None
+        self._check(lib().flagcxLocalPlanExecute(self._h, _ptr_array(send_ptrs), _ptr_array(recv_ptrs), sc,
+                                                 int(dtype), root, _sref(st)))
+
+    def close(self):
+        if self._h:
+            lib().flagcxLocalPlanDestroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -304,6 +304,44 @@ flagcxResult_t flagcxLocalUnpackList(void *const *dsts, const void *src, int n,
                                      size_t bytes, flagcxStream_t stream);
 
 /* ------------------------------------------------------------------------- */
+/* C2C plan replay on one GPU                                                  */
+/* ------------------------------------------------------------------------- */
+/* Replays, for ALL simulated ranks in lock step, the per-rank plans that
+ * flagcxC2cPlanner exports and imports as XML (flagcx/core/c2c_algo.cc:973-1087,
+ * format in flagcx/core/c2c_ir.h:62-176), stage by stage as
+ * flagcxC2cPlanner::execute does (c2c_algo.cc:2142-2290).  Homo functions
+ * (flagcxC2cHomoFunc::run, c2c_algo.cc:286-511) run on the ranks of a cluster
+ * (homoType 1: on its inter-ranks) with the local reduce / copy kernels in place
+ * of the vendor CCL, folding in homo-rank order; hetero P2P ops become device
+ * copies between the ranks' buffers; the refresh function is flagcxLocalRefresh.
+ * commOp 12 (LocCpy) and 13 (LocRed), reserved by the reference's plan DSL
+ * (flagcx/tools/utils.py:43-44), are rank-local copy and
+ * recv = OP(send, recv).  Host-side errors of a plan are reported through
+ * flagcxLocalPlanGetLastError. */
+typedef struct flagcxLocalPlan *flagcxLocalPlan_t;
+
+/* clusterIds[r]: cluster of global rank r (0-based, dense).  isInterRank[r] != 0:
+ * rank r is one of its cluster's inter-ranks (NULL: every rank is).  totalCount:
+ * elements of the collective (send or recv count, as flagcxC2cPlanner's
+ * totalCount_).  redOp other than sum/max/min is flagcxNotSupported at execute,
+ * like c2c_algo.cc:2047-2053. */
+flagcxResult_t flagcxLocalPlanCreate(flagcxLocalPlan_t *plan, int nranks, const int *clusterIds,
+                                     const int *isInterRank, size_t totalCount,
+                                     flagcxCommOp_t commOp, flagcxRedOp_t redOp);
+flagcxResult_t flagcxLocalPlanDestroy(flagcxLocalPlan_t plan);
+/* Reads / writes <prefix>_<rank>.xml for every rank. */
+flagcxResult_t flagcxLocalPlanImportXml(flagcxLocalPlan_t plan, const char *prefix);
+flagcxResult_t flagcxLocalPlanExportXml(flagcxLocalPlan_t plan, const char *prefix);
+/* 0 sequential, 1 pipeline, 2 input (default after import). */
+flagcxResult_t flagcxLocalPlanSetAlgorithm(flagcxLocalPlan_t plan, int algorithm);
+/* Host arrays of one device pointer per rank; scratchbuffs may be NULL when the
+ * plan never names scratch.  Enqueues everything on `stream`. */
+flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan_t plan, const void *const *sendbuffs,
+                                      void *const *recvbuffs, void *const *scratchbuffs,
+                                      flagcxDataType_t datatype, int root, flagcxStream_t stream);
+const char *flagcxLocalPlanGetLastError(flagcxLocalPlan_t plan);
+
+/* ------------------------------------------------------------------------- */
 /* Launcher-convention symbols                                                */
 /* ------------------------------------------------------------------------- */
 /* These have the reference's device-function shape
