@@ -43,6 +43,8 @@ static long long maxSpin() {
   return v;
 }
 
+long long asyncMaxSpin() { return maxSpin(); }
+
 } // namespace flagcx_amd
 
 using namespace flagcx_amd;

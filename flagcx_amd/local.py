@@ -83,6 +83,30 @@ class ReduceTrigger(C.Structure):    # flagcxLocalReduceTrigger, 16-byte aligned
         return t
 
 
+class DeviceTrigger(C.Structure):    # flagcxLocalDeviceTrigger
+    _fields_ = [("fst", C.c_uint64), ("snd", C.c_uint64)]
+
+    @property
+    def addr(self):
+        return self.fst
+
+    @property
+    def count(self):
+        return self.snd & 0xffffffff
+
+    @property
+    def peer(self):
+        return (self.snd >> 32) & 0xfffff
+
+    @property
+    def datatype(self):
+        return (self.snd >> 52) & 0xf
+
+    @property
+    def prim(self):
+        return (self.snd >> 56) & 0xf
+
+
 class CopyArgs(C.Structure):         # flagcxLocalCopyArgs
     _fields_ = [("dst", C.c_void_p), ("src", C.c_void_p), ("size", C.c_uint64), ("result", C.c_int32),
                 ("reserved", C.c_int32)]
@@ -96,6 +120,7 @@ EXPORTS = [
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
     "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
     "flagcxLocalReduceBatch", "flagcxLocalReduceTriggers",
+    "flagcxLocalFifoInit", "flagcxLocalFifoDestroy", "flagcxLocalFifoDequeue", "flagcxLocalP2pDemo",
     "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
     "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
 ]
@@ -140,6 +165,10 @@ def lib():
         L.flagcxLocalCopyFunc.argtypes = [sp, C.POINTER(CopyArgs)]
         L.flagcxLocalReduceBatch.argtypes = [C.POINTER(ReduceDesc), i, i, i, i, sp]
         L.flagcxLocalReduceTriggers.argtypes = [C.POINTER(ReduceTrigger), i, sp]
+        L.flagcxLocalFifoInit.argtypes = [C.POINTER(vp)]
+        L.flagcxLocalFifoDestroy.argtypes = [vp]
+        L.flagcxLocalFifoDequeue.argtypes = [vp, C.POINTER(DeviceTrigger)]
+        L.flagcxLocalP2pDemo.argtypes = [vp, vp, sz, i, i, i, vp, sp]
         L.flagcxLocalPlanCreate.argtypes = [C.POINTER(vp), i, C.POINTER(i), C.POINTER(i), sz, i, i]
         L.flagcxLocalPlanDestroy.argtypes = [vp]
         L.flagcxLocalPlanImportXml.argtypes = [vp, C.c_char_p]

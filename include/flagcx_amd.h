@@ -304,6 +304,45 @@ flagcxResult_t flagcxLocalUnpackList(void *const *dsts, const void *src, int n,
                                      size_t bytes, flagcxStream_t stream);
 
 /* ------------------------------------------------------------------------- */
+/* Device-producer / host-consumer trigger FIFO                                */
+/* ------------------------------------------------------------------------- */
+/* The reference's kernel FIFO (flagcx/include/flagcx_kernel.h:7-49,75-88): a pinned
+ * host buffer of 64-bit words [capacity, consumed, produced, entries...]; an entry
+ * is {fst, snd} with fst = address and
+ * snd = count[0,32) | peerRank[32,52) | datatype[52,56) | prim[56,60). */
+#define FLAGCX_LOCAL_FIFO_CAPACITY 16 /* FLAGCX_KERNEL_FIFO_CAPACITY */
+#define FLAGCX_LOCAL_PRIM_SEND 0      /* flagcxDevicePrimSend .. Wait, flagcx_kernel.h:9-14 */
+#define FLAGCX_LOCAL_PRIM_RECV 1
+#define FLAGCX_LOCAL_PRIM_TERM 2
+#define FLAGCX_LOCAL_PRIM_WAIT 3
+
+typedef struct {
+  uint64_t fst;
+  uint64_t snd;
+} flagcxLocalDeviceTrigger;
+
+/* Getters of flagcxDeviceTrigger (flagcx/core/flagcx_kernel_host.cc:9-29). */
+static inline uint64_t flagcxLocalTriggerAddr(const flagcxLocalDeviceTrigger *t) { return t->fst; }
+static inline uint64_t flagcxLocalTriggerCount(const flagcxLocalDeviceTrigger *t) { return t->snd & 0xffffffffull; }
+static inline uint64_t flagcxLocalTriggerPeerRank(const flagcxLocalDeviceTrigger *t) { return (t->snd >> 32) & 0xfffffull; }
+static inline uint64_t flagcxLocalTriggerDatatype(const flagcxLocalDeviceTrigger *t) { return (t->snd >> 52) & 0xfull; }
+static inline uint64_t flagcxLocalTriggerType(const flagcxLocalDeviceTrigger *t) { return (t->snd >> 56) & 0xfull; }
+
+/* flagcxFifo::flagcxFifoInit / flagcxFifoDestroy (flagcx_kernel_host.cc:31-50):
+ * allocates (setup time, not the hot path) and frees the pinned buffer. */
+flagcxResult_t flagcxLocalFifoInit(void **fifoBuffer);
+flagcxResult_t flagcxLocalFifoDestroy(void *fifoBuffer);
+/* Host side: dequeue (flagcx_kernel_host.cc:52-73).  An empty queue yields a zero
+ * trigger and flagcxSuccess. */
+flagcxResult_t flagcxLocalFifoDequeue(void *fifoBuffer, flagcxLocalDeviceTrigger *trigger);
+/* flagcxP2pDemo (flagcx/kernels/device_collective_demo.cu:27-34): one lane enqueues
+ * Send, Recv, Term and Wait triggers, then waits until the host has drained the
+ * queue.  All device-side waits give up after the spin bound of deviceAsyncLoad. */
+flagcxResult_t flagcxLocalP2pDemo(const void *sendbuff, void *recvbuff, size_t count,
+                                  flagcxDataType_t datatype, int sendPeer, int recvPeer,
+                                  void *fifoBuffer, flagcxStream_t stream);
+
+/* ------------------------------------------------------------------------- */
 /* C2C plan replay on one GPU                                                  */
 /* ------------------------------------------------------------------------- */
 /* Replays, for ALL simulated ranks in lock step, the per-rank plans that

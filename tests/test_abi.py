@@ -17,7 +17,9 @@ def declared_symbols():
     text = open(os.path.join(ROOT, "include", "flagcx_amd.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = set(re.findall(r"\b(flagcxLocal\w+|deviceAsync\w+)\s*\(", text))
-    names.discard("flagcxLocalMakeReduceTrigger")   # static inline helper, not an export
+    for inline in ("flagcxLocalMakeReduceTrigger", "flagcxLocalTriggerAddr", "flagcxLocalTriggerCount",
+                   "flagcxLocalTriggerPeerRank", "flagcxLocalTriggerDatatype", "flagcxLocalTriggerType"):
+        names.discard(inline)                       # static inline helpers, not exports
     return sorted(names)
 
 

@@ -146,3 +146,59 @@ def test_device_async_store_and_bounded_load(L):
     finally:
         lib.flagcxLocalSetMaxSpinCount(-1)
     assert flag.cpu().tolist() == [1, 0, 0, 0]
+
+
+def test_device_fifo_producer_host_consumer(L):
+    """One lane enqueues Send, Recv, Term, Wait into the pinned FIFO; the host
+    dequeues them in order; the kernel's final wait ends once the queue is drained."""
+    import time
+    import torch
+    lib = L.lib()
+    fifo = C.c_void_p()
+    assert lib.flagcxLocalFifoInit(C.byref(fifo)) == 0
+    words = (C.c_uint64 * 3).from_address(fifo.value)
+    assert list(words) == [16, 0, 0]
+    empty = L.DeviceTrigger(1, 1)
+    assert lib.flagcxLocalFifoDequeue(fifo, C.byref(empty)) == 0 and (empty.fst, empty.snd) == (0, 0)
+    send = torch.zeros(1000, dtype=torch.float32, device="cuda")
+    recv = torch.zeros(1000, dtype=torch.float32, device="cuda")
+    lib.flagcxLocalSetMaxSpinCount(1 << 22)          # seconds, not minutes, if the host stalls
+    try:
+        st = L.current_stream()
+        assert lib.flagcxLocalP2pDemo(send.data_ptr(), recv.data_ptr(), 1000, int(L.DataType.Float32), 3, 5,
+                                      fifo, C.byref(st)) == 0
+        got = []
+        deadline = time.time() + 20
+        while len(got) < 4 and time.time() < deadline:
+            t = L.DeviceTrigger()
+            assert lib.flagcxLocalFifoDequeue(fifo, C.byref(t)) == 0
+            if words[1] > len(got):                  # consumed advanced: a real entry
+                got.append((t.addr, t.count, t.peer, t.datatype, t.prim))
+        torch.cuda.synchronize()
+    finally:
+        lib.flagcxLocalSetMaxSpinCount(-1)
+    f32 = int(L.DataType.Float32)
+    assert got == [(send.data_ptr(), 1000, 3, f32, 0), (recv.data_ptr(), 1000, 5, f32, 1),
+                   (0, 0, 0, 0, 2), (0, 0, 0, 0, 3)]
+    assert list(words) == [16, 4, 4]
+    assert lib.flagcxLocalFifoDestroy(fifo) == 0
+
+
+def test_device_fifo_full_queue_gives_up(L):
+    """Nobody dequeues and the queue is pre-filled: the producer's bounded wait
+    expires and the kernel exits without writing."""
+    import torch
+    lib = L.lib()
+    fifo = C.c_void_p()
+    assert lib.flagcxLocalFifoInit(C.byref(fifo)) == 0
+    words = (C.c_uint64 * 3).from_address(fifo.value)
+    words[2] = 16                                    # produced - consumed == capacity
+    lib.flagcxLocalSetMaxSpinCount(4)
+    try:
+        st = L.current_stream()
+        assert lib.flagcxLocalP2pDemo(1 << 20, 1 << 21, 8, 7, 0, 1, fifo, C.byref(st)) == 0
+        torch.cuda.synchronize()
+    finally:
+        lib.flagcxLocalSetMaxSpinCount(-1)
+    assert list(words) == [16, 0, 16]
+    assert lib.flagcxLocalFifoDestroy(fifo) == 0
