@@ -1,0 +1,161 @@
+// host_staging_ring.cpp - the staging pipeline either side of the local reduce.
+//
+// The reference moves every message between ranks through a ring of
+// FLAGCX_P2P_STEPS (16) slots of FLAGCX_P2P_CHUNKSIZE (4 MiB)
+// (flagcx/core/p2p.h:11-15, same numbers in flagcx/core/net.h:19-22): the sender's
+// proxy copies min(chunk, size - copied) bytes into slot (step & 15) and bumps
+// sendHead once the copy's event has fired (flagcx/core/p2p.cc:75-107); the
+// receiver copies the slot out and bumps recvTail, which frees the slot for step
+// + 16 (p2p.cc:170-205).  Here both sides live on one GPU: a producer stream
+// plays the sender's proxy, a consumer stream the receiver's, and the head / tail
+// counters become one "filled" and one "freed" HIP event per slot.  The consumer
+// either copies the slot out (send/recv) or - the reduce-scatter form - folds the
+// slots of all peers and the local slice straight into the output, so the reduce
+// of chunk i overlaps the staging copies of chunk i+1.
+//
+// Ring memory belongs to the caller (steps * npeers * chunkBytes); creating the
+// object allocates only the events.
+#include "../../include/flagcx_amd.h"
+
+#include <hip/hip_runtime.h>
+
+#include <vector>
+
+struct flagcxLocalRing {
+  char *buffer = nullptr;
+  size_t chunkBytes = 0;
+  int steps = 0, npeers = 0;
+  std::vector<hipEvent_t> filled, freed;
+  hipEvent_t start = nullptr;
+};
+
+namespace {
+
+inline hipStream_t hipOf(flagcxStream_t s) { return s ? *reinterpret_cast<hipStream_t *>(s) : nullptr; }
+
+#define RCHECK(call)                                                           \
+  do {                                                                         \
+    flagcxResult_t r_ = (call);                                                \
+    if (r_ != flagcxSuccess) return r_;                                        \
+  } while (0)
+#define HCHECK(call)                                                           \
+  do {                                                                         \
+    if ((call) != hipSuccess) return flagcxUnhandledDeviceError;               \
+  } while (0)
+
+inline char *slotOf(flagcxLocalRing *r, size_t step, int peer) {
+  return r->buffer + ((step % (size_t)r->steps) * (size_t)r->npeers + (size_t)peer) * r->chunkBytes;
+}
+
+} // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+flagcxResult_t flagcxLocalRingCreate(flagcxLocalRing **ring, void *ringBuffer, size_t ringBytes, int npeers,
+                                     size_t chunkBytes, int steps) {
+  if (!ring || !ringBuffer || npeers < 1 || npeers >= FLAGCX_LOCAL_MAX_RANKS) return flagcxInvalidArgument;
+  if (chunkBytes == 0) chunkBytes = FLAGCX_LOCAL_CHUNKSIZE;
+  if (steps == 0) steps = FLAGCX_LOCAL_STEPS;
+  if (steps < 1 || steps > 1024 || (chunkBytes & 15u)) return flagcxInvalidArgument;
+  if (ringBytes < (size_t)steps * (size_t)npeers * chunkBytes) return flagcxInvalidArgument;
+  flagcxLocalRing *r = new flagcxLocalRing();
+  r->buffer = static_cast<char *>(ringBuffer);
+  r->chunkBytes = chunkBytes;
+  r->steps = steps;
+  r->npeers = npeers;
+  r->filled.resize(steps);
+  r->freed.resize(steps);
+  bool ok = hipEventCreateWithFlags(&r->start, hipEventDisableTiming) == hipSuccess;
+  for (int i = 0; ok && i < steps; i++) {
+    ok = hipEventCreateWithFlags(&r->filled[i], hipEventDisableTiming) == hipSuccess &&
+         hipEventCreateWithFlags(&r->freed[i], hipEventDisableTiming) == hipSuccess;
+  }
+  if (!ok) {
+    delete r; // events created so far are few; the process is in trouble anyway
+    return flagcxUnhandledDeviceError;
+  }
+  *ring = r;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalRingDestroy(flagcxLocalRing *r) {
+  if (!r) return flagcxSuccess;
+  for (auto e : r->filled) if (e) (void)hipEventDestroy(e);
+  for (auto e : r->freed) if (e) (void)hipEventDestroy(e);
+  if (r->start) (void)hipEventDestroy(r->start);
+  delete r;
+  return flagcxSuccess;
+}
+
+// One message through the ring: producer copies src -> slot, consumer slot -> dst.
+flagcxResult_t flagcxLocalRingSendRecv(flagcxLocalRing *r, void *dst, const void *src, size_t size,
+                                       flagcxStream_t copyStream, flagcxStream_t stream) {
+  if (!r || !copyStream || !stream) return flagcxInvalidArgument;
+  if (size == 0) return flagcxSuccess;
+  if (!dst || !src) return flagcxInvalidArgument;
+  hipStream_t ps = hipOf(copyStream), cs = hipOf(stream);
+  HCHECK(hipEventRecord(r->start, cs)); // what the consumer stream produced so far is the sender's input
+  HCHECK(hipStreamWaitEvent(ps, r->start, 0));
+  const size_t nsteps = (size + r->chunkBytes - 1) / r->chunkBytes; // chunkSteps (flagcx/core/group.cc:179-181)
+  for (size_t step = 0; step < nsteps; step++) {
+    const int slot = (int)(step % (size_t)r->steps);
+    const size_t off = step * r->chunkBytes;
+    const size_t n = size - off < r->chunkBytes ? size - off : r->chunkBytes;
+    if (step >= (size_t)r->steps) HCHECK(hipStreamWaitEvent(ps, r->freed[slot], 0)); // recvTail > copied
+    RCHECK(flagcxLocalMemcpy(slotOf(r, step, 0), (const char *)src + off, n, copyStream));
+    HCHECK(hipEventRecord(r->filled[slot], ps));                                       // sendHead
+    HCHECK(hipStreamWaitEvent(cs, r->filled[slot], 0));
+    RCHECK(flagcxLocalMemcpy((char *)dst + off, slotOf(r, step, 0), n, stream));
+    HCHECK(hipEventRecord(r->freed[slot], cs));                                        // recvTail
+  }
+  return flagcxSuccess;
+}
+
+// Rank `rank`'s reduce-scatter shard with the nranks-1 peers' slices arriving
+// through the ring, chunk by chunk; result identical to flagcxLocalReduceScatter.
+flagcxResult_t flagcxLocalRingReduceScatter(flagcxLocalRing *r, const void *const *sendbuffs, int nranks,
+                                            int rank, void *recvbuff, size_t recvcount,
+                                            flagcxDataType_t datatype, flagcxRedOp_t op,
+                                            flagcxStream_t copyStream, flagcxStream_t stream) {
+  if (!r || !sendbuffs || !copyStream || !stream) return flagcxInvalidArgument;
+  if (nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS || rank < 0 || rank >= nranks) return flagcxInvalidArgument;
+  if (nranks - 1 > r->npeers) return flagcxInvalidArgument;
+  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  if (!ts || (r->chunkBytes % ts)) return flagcxInvalidArgument;
+  if (recvcount == 0) return flagcxSuccess;
+  if (nranks == 1) // nothing to stage (flagcx/service/bootstrap.cc:856-861)
+    return flagcxLocalReduceScatter(sendbuffs, 1, 0, recvbuff, recvcount, datatype, op, stream);
+  hipStream_t ps = hipOf(copyStream), cs = hipOf(stream);
+  HCHECK(hipEventRecord(r->start, cs));
+  HCHECK(hipStreamWaitEvent(ps, r->start, 0));
+  const size_t size = recvcount * ts;
+  const size_t nsteps = (size + r->chunkBytes - 1) / r->chunkBytes;
+  const void *peerSrc[FLAGCX_LOCAL_MAX_RANKS];
+  const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
+  for (size_t step = 0; step < nsteps; step++) {
+    const int slot = (int)(step % (size_t)r->steps);
+    const size_t off = step * r->chunkBytes;
+    const size_t n = size - off < r->chunkBytes ? size - off : r->chunkBytes;
+    // ring order rank+1, ..., rank: the first nranks-1 are peers, the last is local
+    for (int j = 0; j < nranks - 1; j++) {
+      const int peer = (rank + 1 + j) % nranks;
+      peerSrc[j] = (const char *)sendbuffs[peer] + (size_t)rank * size + off;
+      ordered[j] = slotOf(r, step, j);
+    }
+    ordered[nranks - 1] = (const char *)sendbuffs[rank] + (size_t)rank * size + off;
+    if (step >= (size_t)r->steps) HCHECK(hipStreamWaitEvent(ps, r->freed[slot], 0));
+    // the slot's peer regions are contiguous: one launch stages all peers' chunks
+    RCHECK(flagcxLocalPackList(slotOf(r, step, 0), peerSrc, nranks - 1, n, copyStream));
+    if (n != r->chunkBytes) // ragged last chunk: regions are n apart after a pack
+      for (int j = 0; j < nranks - 1; j++) ordered[j] = slotOf(r, step, 0) + (size_t)j * n;
+    HCHECK(hipEventRecord(r->filled[slot], ps));
+    HCHECK(hipStreamWaitEvent(cs, r->filled[slot], 0));
+    RCHECK(flagcxLocalReduce(ordered, nranks, (char *)recvbuff + off, n / ts, datatype, op, stream));
+    HCHECK(hipEventRecord(r->freed[slot], cs));
+  }
+  return flagcxSuccess;
+}
+
+} // extern "C"
+#pragma GCC visibility pop

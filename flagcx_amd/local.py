@@ -121,6 +121,8 @@ EXPORTS = [
     "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
     "flagcxLocalReduceBatch", "flagcxLocalReduceTriggers",
     "flagcxLocalFifoInit", "flagcxLocalFifoDestroy", "flagcxLocalFifoDequeue", "flagcxLocalP2pDemo",
+    "flagcxLocalRingCreate", "flagcxLocalRingDestroy", "flagcxLocalRingSendRecv",
+    "flagcxLocalRingReduceScatter",
     "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
     "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
 ]
@@ -169,6 +171,10 @@ def lib():
         L.flagcxLocalFifoDestroy.argtypes = [vp]
         L.flagcxLocalFifoDequeue.argtypes = [vp, C.POINTER(DeviceTrigger)]
         L.flagcxLocalP2pDemo.argtypes = [vp, vp, sz, i, i, i, vp, sp]
+        L.flagcxLocalRingCreate.argtypes = [C.POINTER(vp), vp, sz, i, sz, i]
+        L.flagcxLocalRingDestroy.argtypes = [vp]
+        L.flagcxLocalRingSendRecv.argtypes = [vp, vp, vp, sz, sp, sp]
+        L.flagcxLocalRingReduceScatter.argtypes = [vp, pp, i, i, vp, sz, i, i, sp, sp]
         L.flagcxLocalPlanCreate.argtypes = [C.POINTER(vp), i, C.POINTER(i), C.POINTER(i), sz, i, i]
         L.flagcxLocalPlanDestroy.argtypes = [vp]
         L.flagcxLocalPlanImportXml.argtypes = [vp, C.c_char_p]
@@ -353,6 +359,38 @@ class Plan:
     def close(self):
         if self._h:
             lib().flagcxLocalPlanDestroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Ring:
+    """Staging ring over caller memory (flagcxLocalRing*); ring_tensor stays referenced."""
+
+    def __init__(self, ring_tensor, npeers, chunkbytes=0, steps=0):
+        self._keep = ring_tensor
+        self._h = C.c_void_p()
+        rc = lib().flagcxLocalRingCreate(C.byref(self._h), ring_tensor.data_ptr(),
+                                         ring_tensor.numel() * ring_tensor.element_size(), npeers, chunkbytes, steps)
+        if rc:
+            raise FlagcxError(rc, "flagcxLocalRingCreate")
+
+    def send_recv(self, dst_ptr, src_ptr, size, copy_stream, stream):
+        check(lib().flagcxLocalRingSendRecv(self._h, dst_ptr, src_ptr, size, C.byref(copy_stream), C.byref(stream)))
+
+    def reduce_scatter(self, sendbuffs, rank, recv, op, copy_stream, stream, dtype=None):
+        dt = dtype_of(recv, dtype)
+        check(lib().flagcxLocalRingReduceScatter(self._h, _ptr_array([s.data_ptr() for s in sendbuffs]),
+                                                 len(sendbuffs), rank, recv.data_ptr(), recv.numel(), int(dt),
+                                                 int(op), C.byref(copy_stream), C.byref(stream)))
+
+    def close(self):
+        if self._h:
+            lib().flagcxLocalRingDestroy(self._h)
             self._h = C.c_void_p()
 
     def __del__(self):

@@ -86,6 +86,18 @@ def main():
     ms = timed(lambda: L.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks))
     report("C3 fp16 avg shard, 32 chunks as one batch call", nb, ms)
 
+    # the same shard with the 7 peers' slices staged through a 16 x 4 MiB ring on a second stream
+    ring_mem = torch.empty(L.CHUNKSIZE * 16 * (nranks - 1), dtype=torch.uint8, device="cuda")
+    ring = L.Ring(ring_mem, nranks - 1)
+    copy_t = torch.cuda.Stream()
+    cs, ms_ = L.Stream(copy_t.cuda_stream), L.current_stream()
+    ms = timed(lambda: ring.reduce_scatter(send, 3, recv, L.RedOp.Avg, cs, ms_))
+    # staging moves 2 x 7/8 of the inputs on top of the reduce's 9 x shard
+    report("C3 shard through the staging ring (2 streams)", nb, ms,
+           "HBM bytes incl. staging: %d" % (nb + 2 * (nranks - 1) * shard * 2))
+    ring.close()
+    del ring_mem
+
     def all_shards():
         for rk in range(nranks):
             L.reduce_scatter(send, rk, recv, L.RedOp.Avg)

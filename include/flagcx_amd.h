@@ -343,6 +343,36 @@ flagcxResult_t flagcxLocalP2pDemo(const void *sendbuff, void *recvbuff, size_t c
                                   void *fifoBuffer, flagcxStream_t stream);
 
 /* ------------------------------------------------------------------------- */
+/* Staging ring (the pipeline either side of the reduce)                       */
+/* ------------------------------------------------------------------------- */
+/* The 16 x 4 MiB staging ring of the reference's proxies
+ * (FLAGCX_P2P_STEPS x FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15;
+ * MAXSTEPS x CHUNKSIZE, flagcx/core/net.h:19-22) on one GPU: a producer stream
+ * copies chunk `step` into slot step % steps like flagcxP2pProxySend
+ * (flagcx/core/p2p.cc:75-107), a consumer stream takes it out like
+ * flagcxP2pProxyRecv (p2p.cc:170-205); sendHead / recvTail are one "filled" and
+ * one "freed" event per slot.  ringBuffer is the caller's device memory of at
+ * least steps * npeers * chunkBytes bytes (0 selects 4 MiB / 16); Create
+ * allocates events only.  Calls on one ring must not overlap. */
+typedef struct flagcxLocalRing *flagcxLocalRing_t;
+flagcxResult_t flagcxLocalRingCreate(flagcxLocalRing_t *ring, void *ringBuffer, size_t ringBytes,
+                                     int npeers, size_t chunkBytes, int steps);
+flagcxResult_t flagcxLocalRingDestroy(flagcxLocalRing_t ring);
+/* One message src -> ring -> dst in chunk steps (send/recv staging).  Work is
+ * enqueued on copyStream (producer) and stream (consumer); the result is complete
+ * when `stream` is.  Neither stream may be NULL. */
+flagcxResult_t flagcxLocalRingSendRecv(flagcxLocalRing_t ring, void *dst, const void *src, size_t size,
+                                       flagcxStream_t copyStream, flagcxStream_t stream);
+/* flagcxLocalReduceScatter with the nranks-1 peers' slices arriving through the
+ * ring: per chunk one launch stages all peers' pieces into the slot and one
+ * reduce folds them with the local piece into recvbuff, so the reduce of chunk i
+ * overlaps the staging of chunk i+1.  Same bytes as flagcxLocalReduceScatter. */
+flagcxResult_t flagcxLocalRingReduceScatter(flagcxLocalRing_t ring, const void *const *sendbuffs,
+                                            int nranks, int rank, void *recvbuff, size_t recvcount,
+                                            flagcxDataType_t datatype, flagcxRedOp_t op,
+                                            flagcxStream_t copyStream, flagcxStream_t stream);
+
+/* ------------------------------------------------------------------------- */
 /* C2C plan replay on one GPU                                                  */
 /* ------------------------------------------------------------------------- */
 /* Replays, for ALL simulated ranks in lock step, the per-rank plans that

@@ -1,0 +1,92 @@
+"""The staging ring: messages and reduce-scatter shards streamed through slots in
+chunk steps on two streams must give the bytes of the direct calls."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from tests.util import dev_empty, from_dev, make_inputs, same, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def L():
+    import torch
+    assert torch.cuda.is_available()
+    from flagcx_amd import local
+    assert local.lib().flagcxLocalInit() == 0
+    return local
+
+
+def streams(L):
+    import torch
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    return a, b, L.Stream(a.cuda_stream), L.Stream(b.cuda_stream)
+
+
+@pytest.mark.parametrize("size,chunk,steps", [(1, 4096, 4), (4096 * 3, 4096, 4), (4096 * 37 + 100, 4096, 4),
+                                              (1 << 20, 65536, 16), ((9 << 20) + 16, 0, 0)])
+def test_ring_send_recv(L, size, chunk, steps):
+    import torch
+    ring_mem = torch.empty((steps or 16) * (chunk or L.CHUNKSIZE), dtype=torch.uint8, device="cuda")
+    ring = L.Ring(ring_mem, 1, chunk, steps)
+    h = np.random.default_rng(size).integers(0, 256, size, dtype=np.uint8)
+    src = to_dev(h)
+    dst = torch.full((size + 16,), 0x5A, dtype=torch.uint8, device="cuda")
+    ta, tb, sa, sb = streams(L)
+    torch.cuda.synchronize()
+    ring.send_recv(dst.data_ptr(), src.data_ptr(), size, sa, sb)
+    tb.synchronize()
+    ta.synchronize()
+    got = from_dev(dst, np.uint8)
+    assert same(got[:size], h) and (got[size:] == 0x5A).all()
+    ring.close()
+
+
+@pytest.mark.parametrize("dt,op,nranks,rcount,chunk,steps", [
+    (O.FP32, O.SUM, 4, 10000, 4096, 4),          # many wraps of a small ring, ragged last chunk
+    (O.BF16, O.SUM, 8, 1 << 20, 1 << 18, 16),
+    (O.FP16, O.AVG, 8, (1 << 21) + 24, 0, 0),     # default 16 x 4 MiB ring
+    (O.INT32, O.MAX, 2, 5000, 4096, 2),
+])
+def test_ring_reduce_scatter_equals_direct(L, dt, op, nranks, rcount, chunk, steps):
+    import torch
+    ts = O.type_size(dt)
+    send_h = make_inputs(dt, nranks, nranks * rcount, seed=17 + dt, op=op)
+    send = [to_dev(h) for h in send_h]
+    ring_mem = torch.empty((steps or 16) * (nranks - 1) * (chunk or L.CHUNKSIZE), dtype=torch.uint8, device="cuda")
+    ring = L.Ring(ring_mem, nranks - 1, chunk, steps)
+    ta, tb, sa, sb = streams(L)
+    for rank in (0, nranks - 1):
+        direct = dev_empty(rcount, ts)
+        staged = dev_empty(rcount, ts, fill=0)
+        L.reduce_scatter(send, rank, direct, op, dtype=dt)
+        torch.cuda.synchronize()
+        ring.reduce_scatter(send, rank, staged, op, sa, sb, dtype=dt)
+        tb.synchronize()
+        ta.synchronize()
+        assert torch.equal(direct, staged), rank
+        rc, want = O.reduce_scatter_rank(send_h, rank, rcount, dt, op)
+        nan_ok = dt in (O.FP16, O.BF16, O.FP32) and op in (O.SUM, O.AVG)
+        assert same(from_dev(staged, send_h[0].dtype), want, nan_class=nan_ok, dtype=dt)
+    ring.close()
+
+
+def test_ring_rejects_bad_arguments(L):
+    import torch
+    mem = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    h = C.c_void_p()
+    lib = L.lib()
+    inv = int(L.Result.InvalidArgument)
+    assert lib.flagcxLocalRingCreate(C.byref(h), mem.data_ptr(), 1 << 20, 1, 0, 0) == inv      # 64 MiB needed
+    assert lib.flagcxLocalRingCreate(C.byref(h), mem.data_ptr(), 1 << 20, 0, 4096, 4) == inv
+    assert lib.flagcxLocalRingCreate(C.byref(h), mem.data_ptr(), 1 << 20, 1, 4100, 4) == inv   # chunk % 16
+    assert lib.flagcxLocalRingCreate(C.byref(h), None, 1 << 20, 1, 4096, 4) == inv
+    assert lib.flagcxLocalRingCreate(C.byref(h), mem.data_ptr(), 1 << 20, 1, 4096, 4) == 0
+    st = L.current_stream()
+    assert lib.flagcxLocalRingSendRecv(h, mem.data_ptr(), mem.data_ptr() + 4096, 16, None, C.byref(st)) == inv
+    ptrs = (C.c_void_p * 3)(mem.data_ptr(), mem.data_ptr(), mem.data_ptr())
+    assert lib.flagcxLocalRingReduceScatter(h, ptrs, 3, 0, mem.data_ptr(), 16, 7, 0, C.byref(st), C.byref(st)) == inv
+    assert lib.flagcxLocalRingDestroy(h) == 0
