@@ -60,6 +60,10 @@ def build(verbose=False, jobs=None):
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(one, units))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    # C++ timing driver that links the C ABI (no Python in the launch path)
+    perf = os.path.join(HERE, "perf", "local_perf.cpp")
+    _run([HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", perf, "-o",
+          os.path.join(LIBDIR, "local_perf"), "-L" + LIBDIR, "-lflagcx_amd", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", LIB, os.path.getsize(LIB), "bytes")
     return LIB

@@ -123,6 +123,7 @@ EXPORTS = [
     "flagcxLocalFifoInit", "flagcxLocalFifoDestroy", "flagcxLocalFifoDequeue", "flagcxLocalP2pDemo",
     "flagcxLocalRingCreate", "flagcxLocalRingDestroy", "flagcxLocalRingSendRecv",
     "flagcxLocalRingReduceScatter",
+    "flagcxLocalGetDeviceAdaptor", "flagcxLocalDeviceAdaptorLayout",
     "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
     "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
 ]
@@ -175,6 +176,9 @@ def lib():
         L.flagcxLocalRingDestroy.argtypes = [vp]
         L.flagcxLocalRingSendRecv.argtypes = [vp, vp, vp, sz, sp, sp]
         L.flagcxLocalRingReduceScatter.argtypes = [vp, pp, i, i, vp, sz, i, i, sp, sp]
+        L.flagcxLocalGetDeviceAdaptor.restype = vp
+        L.flagcxLocalGetDeviceAdaptor.argtypes = []
+        L.flagcxLocalDeviceAdaptorLayout.argtypes = [C.POINTER(sz), i]
         L.flagcxLocalPlanCreate.argtypes = [C.POINTER(vp), i, C.POINTER(i), C.POINTER(i), sz, i, i]
         L.flagcxLocalPlanDestroy.argtypes = [vp]
         L.flagcxLocalPlanImportXml.argtypes = [vp, C.c_char_p]
@@ -398,3 +402,27 @@ class Ring:
             self.close()
         except Exception:
             pass
+
+
+ADAPTOR_SLOTS = [
+    "deviceSynchronize", "deviceMemcpy", "deviceMemset", "deviceMalloc", "deviceFree", "setDevice", "getDevice",
+    "getDeviceCount", "getVendor", "hostGetDevicePointer", "memHandleInit", "memHandleDestroy", "gdrMemAlloc",
+    "gdrMemFree", "hostShareMemAlloc", "hostShareMemFree", "gdrPtrMmap", "gdrPtrMunmap", "streamCreate",
+    "streamDestroy", "streamCopy", "streamFree", "streamSynchronize", "streamQuery", "streamWaitEvent",
+    "eventCreate", "eventDestroy", "eventRecord", "eventSynchronize", "eventQuery", "ipcMemHandleCreate",
+    "ipcMemHandleGet", "ipcMemHandleOpen", "ipcMemHandleClose", "ipcMemHandleFree", "launchKernel", "copyArgsInit",
+    "copyArgsFree", "launchDeviceFunc", "getDeviceProperties", "getDevicePciBusId", "getDeviceByPciBusId",
+    "launchHostFunc", "dmaSupport", "getHandleForAddressRange", "eventElapsedTime",
+]
+
+
+def device_adaptor():
+    """(name, {slot: address or None}) of the exported flagcxDeviceAdaptor table."""
+    base = lib().flagcxLocalGetDeviceAdaptor()
+    name = C.string_at(base, 32).split(b"\0")[0].decode()
+    ptrs = (C.c_void_p * len(ADAPTOR_SLOTS)).from_address(base + 32)
+    return name, {n: ptrs[k] for k, n in enumerate(ADAPTOR_SLOTS)}
+
+
+def adaptor_fn(slots, name, restype, *argtypes):
+    return C.CFUNCTYPE(restype, *argtypes)(slots[name])

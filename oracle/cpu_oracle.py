@@ -82,8 +82,16 @@ def ref_lib():
         L = C.CDLL(path)
         L.ref_binary.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
         L.ref_enum.argtypes = [C.c_char_p]
+        L.ref_adaptor_layout.argtypes = [C.POINTER(C.c_size_t), C.c_int]
         _ref = L
     return _ref
+
+
+def ref_adaptor_layout():
+    """sizeof / member offsets of the reference's struct flagcxDeviceAdaptor."""
+    out = (C.c_size_t * 64)()
+    n = ref_lib().ref_adaptor_layout(out, 64)
+    return list(out[:n])
 
 
 def _ptr(a):

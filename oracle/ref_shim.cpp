@@ -48,3 +48,26 @@ extern "C" int ref_enum(const char *name) {
 #undef E
   return -1;
 }
+
+// Layout of the reference's device-adaptor table as ITS header defines it
+// (flagcx/adaptor/include/adaptor.h:145-233): sizeof, every member offset in
+// declaration order, sizeof(struct flagcxDevProps).
+#include "adaptor.h"
+#include <cstddef>
+extern "C" int ref_adaptor_layout(size_t *out, int cap) {
+#define O(m) offsetof(struct flagcxDeviceAdaptor, m),
+  const size_t v[] = {sizeof(struct flagcxDeviceAdaptor),
+      O(name) O(deviceSynchronize) O(deviceMemcpy) O(deviceMemset) O(deviceMalloc) O(deviceFree) O(setDevice)
+      O(getDevice) O(getDeviceCount) O(getVendor) O(hostGetDevicePointer) O(memHandleInit) O(memHandleDestroy)
+      O(gdrMemAlloc) O(gdrMemFree) O(hostShareMemAlloc) O(hostShareMemFree) O(gdrPtrMmap) O(gdrPtrMunmap)
+      O(streamCreate) O(streamDestroy) O(streamCopy) O(streamFree) O(streamSynchronize) O(streamQuery)
+      O(streamWaitEvent) O(eventCreate) O(eventDestroy) O(eventRecord) O(eventSynchronize) O(eventQuery)
+      O(ipcMemHandleCreate) O(ipcMemHandleGet) O(ipcMemHandleOpen) O(ipcMemHandleClose) O(ipcMemHandleFree)
+      O(launchKernel) O(copyArgsInit) O(copyArgsFree) O(launchDeviceFunc) O(getDeviceProperties)
+      O(getDevicePciBusId) O(getDeviceByPciBusId) O(launchHostFunc) O(dmaSupport) O(getHandleForAddressRange)
+      O(eventElapsedTime) sizeof(struct flagcxDevProps)};
+#undef O
+  const int n = (int)(sizeof(v) / sizeof(v[0]));
+  for (int i = 0; i < n && i < cap; i++) out[i] = v[i];
+  return n;
+}

@@ -15,6 +15,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def declared_symbols():
     text = open(os.path.join(ROOT, "include", "flagcx_amd.h")).read()
+    text += open(os.path.join(ROOT, "include", "flagcx_amd_adaptor.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = set(re.findall(r"\b(flagcxLocal\w+|deviceAsync\w+)\s*\(", text))
     for inline in ("flagcxLocalMakeReduceTrigger", "flagcxLocalTriggerAddr", "flagcxLocalTriggerCount",
@@ -155,3 +156,38 @@ def test_error_strings():
     for code in range(0, 11):
         s = L.flagcxLocalGetErrorString(code)
         assert s and isinstance(s, bytes)
+
+
+def test_device_adaptor_table_layout_and_slots():
+    """The exported table has the reference's layout (checked against ITS header where
+    the reference tree was available at build time) and fills every slot the
+    reference's complete (NVIDIA) table fills."""
+    L = local.lib()
+    out = (C.c_size_t * 64)()
+    n = L.flagcxLocalDeviceAdaptorLayout(out, 64)
+    mine = list(out[:n])
+    assert n == 49 and mine[0] == 32 + 46 * 8 and mine[1] == 0 and mine[2] == 32
+    assert mine[2:48] == [32 + 8 * k for k in range(46)] and mine[48] == 256 + 12
+    if O.ref_lib() is not None:
+        assert mine == O.ref_adaptor_layout()
+    name, slots = local.device_adaptor()
+    assert name == "HIP"
+    null_in_reference_too = {"memHandleInit", "memHandleDestroy", "hostShareMemAlloc", "hostShareMemFree",
+                             "gdrPtrMmap", "gdrPtrMunmap", "launchKernel", "copyArgsInit", "copyArgsFree"}
+    for k, v in slots.items():
+        assert (v is None) == (k in null_in_reference_too), k
+    # slots that need no device
+    buf = C.create_string_buffer(128)
+    assert local.adaptor_fn(slots, "getVendor", C.c_int, C.c_char_p)(buf) == 0 and buf.value == b"AMD"
+    assert local.adaptor_fn(slots, "getVendor", C.c_int, C.c_char_p)(None) == 4
+    called = []
+    cb = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)(lambda s, a: called.append((s, a)))
+    ldf = local.adaptor_fn(slots, "launchDeviceFunc", C.c_int, C.c_void_p, C.c_void_p, C.c_void_p)
+    assert ldf(None, cb, 5) == 0 and called == []            # NULL stream: not called (hip_adaptor.cc:263-269)
+    st = local.Stream(None)
+    assert ldf(C.addressof(st), cb, 5) == 0 and called == [(C.addressof(st), 5)]
+    assert ldf(C.addressof(st), None, 5) == 4
+    flag = C.c_bool(True)
+    assert local.adaptor_fn(slots, "dmaSupport", C.c_int, C.POINTER(C.c_bool))(C.byref(flag)) == 0 and not flag.value
+    assert local.adaptor_fn(slots, "eventElapsedTime", C.c_int, C.c_void_p, C.c_void_p, C.c_void_p)(None, None, None) == 4
+    assert local.adaptor_fn(slots, "streamFree", C.c_int, C.c_void_p)(None) == 0
