@@ -165,3 +165,34 @@ def test_c5_sweep_reduce2_and_strided_pack_unpack(L, log2):
     bv = back.view(8, n)
     assert torch.equal(bv[:, :ce], sparse.view(8, n)[:, :ce])
     assert bool((bv[:, ce:] == -3.0).all())
+
+
+def test_buffers_beyond_4GiB(L):
+    """Counts and byte offsets past 2^32: reduce, copy, fill and strided pack."""
+    import torch
+    n = (1 << 32) + 4099
+    g = torch.Generator(device="cuda").manual_seed(7)
+    a = torch.randint(0, 256, (n,), generator=g, device="cuda", dtype=torch.uint8)
+    b = torch.randint(0, 256, (n,), generator=g, device="cuda", dtype=torch.uint8)
+    out = torch.empty(n, dtype=torch.uint8, device="cuda")
+    L.reduce([a, b], out, L.RedOp.Sum)                       # uint8 sum wraps modulo 256
+    torch.cuda.synchronize()
+    assert torch.equal(out, a + b)
+    L.reduce([a, b], out, L.RedOp.Max)
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.maximum(a, b))
+    out.zero_()
+    L.memcpy(out.data_ptr() + 1, a.data_ptr() + 1, n - 1)    # unaligned head on both sides
+    torch.cuda.synchronize()
+    assert torch.equal(out[1:], a[1:]) and int(out[0]) == 0
+    L.memset(out.data_ptr() + 3, 0x5A, n - 6)
+    torch.cuda.synchronize()
+    assert bool((out[3:n - 3] == 0x5A).all()) and out[:3].tolist() == [0, int(a[1]), int(a[2])]
+    assert out[n - 3:].tolist() == a[n - 3:].tolist()
+    del out, b
+    # 2 chunks of 2^31 + 16 bytes at stride 2^31 + 2048: offsets of the second chunk exceed 2^31
+    chunk, stride = (1 << 31) + 16, (1 << 31) + 2048
+    staged = torch.empty(2 * chunk, dtype=torch.uint8, device="cuda")
+    L.pack(staged.data_ptr(), a.data_ptr(), 2, chunk, stride)
+    torch.cuda.synchronize()
+    assert torch.equal(staged[:chunk], a[:chunk]) and torch.equal(staged[chunk:], a[stride:stride + chunk])
