@@ -177,7 +177,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "8-input bf16 sum reduce, fp32 accumulation, 256 MiB per input buffer "
-                               "(128Mi elements), N(0,1) from seeds 0..7 (BASELINE.json configs[1])",
+                               "(128Mi elements), N(0,1) from seeds 0..7",
                    "nranks": K, "elements": N_ELEM, "bytes_per_step": ALGO_BYTES, "accumulate": "fp32"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

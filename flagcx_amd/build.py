@@ -60,10 +60,12 @@ def build(verbose=False, jobs=None):
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(one, units))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
-    # C++ timing driver that links the C ABI (no Python in the launch path)
-    perf = os.path.join(HERE, "perf", "local_perf.cpp")
-    _run([HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", perf, "-o",
-          os.path.join(LIBDIR, "local_perf"), "-L" + LIBDIR, "-lflagcx_amd", "-Wl,-rpath,$ORIGIN"])
+    # C++ programs that link the C ABI: timing driver and the collective test
+    # (host-only C++; they reach the GPU through the library)
+    for prog in ("local_perf", "local_coll_test"):
+        src = os.path.join(HERE, "perf", prog + ".cpp")
+        _run([HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", src, "-o",
+              os.path.join(LIBDIR, prog), "-L" + LIBDIR, "-lflagcx_amd", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", LIB, os.path.getsize(LIB), "bytes")
     return LIB

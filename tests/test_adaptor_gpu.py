@@ -158,3 +158,16 @@ def test_device_queries_and_ipc_handle(A):
     assert A.ipc_free(h) == 0
     assert A.free(mem, MEM_DEVICE, None) == 0
     assert A.dmabuf(None, None, 0, 0) == 9
+
+
+def test_cpp_collective_test_program():
+    """The C++ caller test (reference unit-test patterns over 8 simulated ranks,
+    buffers from the device-adaptor table) passes."""
+    import os
+    import subprocess
+    from flagcx_amd import local
+    exe = os.path.join(os.path.dirname(local.lib_path()), "local_coll_test")
+    assert os.path.exists(exe), "build it with python -m flagcx_amd.build"
+    r = subprocess.run([exe, "-n", "8", "-c", str(1 << 22)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "PASSED" in r.stdout and r.stdout.count("ok ") == 6

@@ -1,4 +1,4 @@
-"""The benchmark configurations at their full sizes (BASELINE.json configs 1-5),
+"""The five benchmark configurations at their full sizes (C1-C5),
 checked against the oracle where it finishes in seconds and through
 size-independent properties elsewhere.  All GPU work goes through the C ABI."""
 import numpy as np
