@@ -55,7 +55,7 @@ const DeviceInfo &deviceInfo() {
 // (K = 8: 81-86 % of peak at 16, against 72-88 % at 8).  About 48-128 KiB of
 // loads in flight per CU saturates HBM; more resident wavefronts only add DRAM
 // page conflicts between the streams.
-static std::atomic<int> gWaves[9] = {{0}, {0}, {24}, {16}, {12}, {12}, {12}, {14}, {16}};
+static std::atomic<int> gWaves[9] = {{0}, {0}, {24}, {14}, {12}, {12}, {14}, {14}, {16}};
 
 int wavesPerCUFor(int k) {
   if (k < 0) k = 0;
@@ -232,6 +232,13 @@ flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU) {
   if (nranks < 0 || nranks > 8 || wavesPerCU < 0 || wavesPerCU > 64)
     return fail(flagcxInvalidArgument, "flagcxLocalTune: nranks %d / wavesPerCU %d out of range", nranks, wavesPerCU);
   setWavesPerCU(nranks, wavesPerCU);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalGetTune(int nranks, int *wavesPerCU) {
+  if (nranks < 0 || nranks > 8 || !wavesPerCU)
+    return fail(flagcxInvalidArgument, "flagcxLocalGetTune: nranks %d out of range or NULL result", nranks);
+  *wavesPerCU = wavesPerCUFor(nranks);
   return flagcxSuccess;
 }
 

@@ -114,7 +114,7 @@ class CopyArgs(C.Structure):         # flagcxLocalCopyArgs
 
 EXPORTS = [
     "flagcxLocalGetDataTypeSize", "flagcxLocalInit", "flagcxLocalGetErrorString", "flagcxLocalGetLastError",
-    "flagcxLocalTune", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
+    "flagcxLocalTune", "flagcxLocalGetTune", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
     "flagcxLocalAllReduce", "flagcxLocalRingChunkTable", "flagcxLocalMemcpy", "flagcxLocalMemset",
     "flagcxLocalRefresh", "flagcxLocalPack", "flagcxLocalUnpack", "flagcxLocalPackList",
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
@@ -150,6 +150,7 @@ def lib():
         L.flagcxLocalGetErrorString.argtypes = [i]
         L.flagcxLocalGetLastError.restype = C.c_char_p
         L.flagcxLocalTune.argtypes = [i, i]
+        L.flagcxLocalGetTune.argtypes = [i, C.POINTER(i)]
         L.flagcxLocalReduce.argtypes = [pp, i, vp, sz, i, i, sp]
         L.flagcxLocalReduceScatter.argtypes = [pp, i, i, vp, sz, i, i, sp]
         L.flagcxLocalReduceScatterChunked.argtypes = [pp, i, i, vp, sz, i, i, sz, sp]

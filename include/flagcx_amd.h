@@ -132,6 +132,7 @@ const char *flagcxLocalGetLastError(void);
  * inputs (1..8; 0 selects the copy kernels).  wavesPerCU == 0 removes the cap.
  * Process-wide; the defaults are the measured optimum on MI355X. */
 flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU);
+flagcxResult_t flagcxLocalGetTune(int nranks, int *wavesPerCU);
 
 /* ------------------------------------------------------------------------- */
 /* N-way elementwise reduction                                                */
