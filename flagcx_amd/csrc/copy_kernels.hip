@@ -35,13 +35,13 @@ struct ListParams {
 
 // LIST: 0 both sides strided, 1 sources from a pointer list, 2 destinations from one
 template <int U, int LIST>
-__global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p, ListParams l) {
+__device__ __forceinline__ void copyWaveBody(const CopyParams &p, const ListParams *l) {
   constexpr uint32_t kTileBytes = 64u * U * 16u;
   const uint64_t ntiles = (p.body + kTileBytes - 1) / kTileBytes;
   const uint32_t voff = threadIdx.x * 16u;
   for (uint64_t c = blockIdx.y; c < p.nchunks; c += gridDim.y) {
-    const char *s = (LIST == 1 ? l.src[c] : p.src + c * p.srcStride) + p.head;
-    char *d = (LIST == 2 ? l.dst[c] : p.dst + c * p.dstStride) + p.head;
+    const char *s = (LIST == 1 ? l->src[c] : p.src + c * p.srcStride) + p.head;
+    char *d = (LIST == 2 ? l->dst[c] : p.dst + c * p.dstStride) + p.head;
     for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
       const uint64_t off = t * kTileBytes;
       const uint64_t left = p.body - off;
@@ -60,23 +60,42 @@ __global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p, ListParams l)
     const uint64_t edge = p.head + p.tail;
     if (threadIdx.x < edge) {
       const uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.body + (threadIdx.x - p.head);
-      const char *s = (LIST == 1 ? l.src[0] : p.src);
-      char *d = (LIST == 2 ? l.dst[0] : p.dst);
+      const char *s = (LIST == 1 ? l->src[0] : p.src);
+      char *d = (LIST == 2 ? l->dst[0] : p.dst);
       d[i] = s[i];
     }
   }
 }
 
+// The strided form carries 72 bytes of arguments; only the list forms pay for the
+// pointer tables.
+template <int U>
+__global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p) {
+  copyWaveBody<U, 0>(p, nullptr);
+}
+template <int U, int LIST>
+__global__ void __launch_bounds__(64) copyWaveListKernel(CopyParams p, ListParams l) {
+  copyWaveBody<U, LIST>(p, &l);
+}
+
 // Element path: W-byte units, chunk by chunk.
 template <typename W, int LIST>
-__global__ void __launch_bounds__(256) copyElemKernel(CopyParams p, ListParams l) {
+__device__ __forceinline__ void copyElemBody(const CopyParams &p, const ListParams *l) {
   const uint64_t n = p.chunkBytes / sizeof(W);
   const uint64_t stride = (uint64_t)gridDim.x * 256;
   for (uint64_t c = blockIdx.y; c < p.nchunks; c += gridDim.y) {
-    const W *s = (const W *)(LIST == 1 ? l.src[c] : p.src + c * p.srcStride);
-    W *d = (W *)(LIST == 2 ? l.dst[c] : p.dst + c * p.dstStride);
+    const W *s = (const W *)(LIST == 1 ? l->src[c] : p.src + c * p.srcStride);
+    W *d = (W *)(LIST == 2 ? l->dst[c] : p.dst + c * p.dstStride);
     for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) d[i] = s[i];
   }
+}
+template <typename W>
+__global__ void __launch_bounds__(256) copyElemKernel(CopyParams p) {
+  copyElemBody<W, 0>(p, nullptr);
+}
+template <typename W, int LIST>
+__global__ void __launch_bounds__(256) copyElemListKernel(CopyParams p, ListParams l) {
+  copyElemBody<W, LIST>(p, &l);
 }
 
 template <int LIST>
@@ -89,7 +108,10 @@ static int launchCopyT(const CopyParams &p, const ListParams &l, bool vector, un
     if (gx < 1) gx = 1;
     if (gx > kMaxGridX) gx = kMaxGridX;
     const int lds = ldsReservation(wavesPerCUFor(0));
-    copyWaveKernel<kCopyUnroll, LIST><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), lds, stream>>>(p, l);
+    if (LIST == 0)
+      copyWaveKernel<kCopyUnroll><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), lds, stream>>>(p);
+    else
+      copyWaveListKernel<kCopyUnroll, LIST><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), lds, stream>>>(p, l);
     return (int)hipGetLastError();
   }
   uint64_t gx = (p.chunkBytes / width + 255) / 256;
@@ -97,12 +119,18 @@ static int launchCopyT(const CopyParams &p, const ListParams &l, bool vector, un
   if (gx > cap) gx = cap;
   if (gx < 1) gx = 1;
   const dim3 grid((unsigned)gx, (unsigned)gy);
+#define FLAGCX_ELEM(W)                                                           \
+  do {                                                                         \
+    if (LIST == 0) copyElemKernel<W><<<grid, dim3(256), 0, stream>>>(p);       \
+    else copyElemListKernel<W, LIST><<<grid, dim3(256), 0, stream>>>(p, l);    \
+  } while (0)
   switch (width) {
-    case 8: copyElemKernel<uint64_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
-    case 4: copyElemKernel<uint32_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
-    case 2: copyElemKernel<uint16_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
-    default: copyElemKernel<uint8_t, LIST><<<grid, dim3(256), 0, stream>>>(p, l); break;
+    case 8: FLAGCX_ELEM(uint64_t); break;
+    case 4: FLAGCX_ELEM(uint32_t); break;
+    case 2: FLAGCX_ELEM(uint16_t); break;
+    default: FLAGCX_ELEM(uint8_t); break;
   }
+#undef FLAGCX_ELEM
   return (int)hipGetLastError();
 }
 
