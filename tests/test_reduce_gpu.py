@@ -321,3 +321,34 @@ def test_reduce_triggers_in_order_with_dependencies(L):
     torch.cuda.synchronize()
     rc, wmin = O.binary(O.MIN, O.INT32, hi[0], hi[1])
     assert same(from_dev(oi, np.int32), wmin)
+
+
+@pytest.mark.parametrize("dt", [O.FP16, O.BF16, O.FP32, O.FP64], ids=lambda d: DT_NAME[d])
+def test_special_values_on_the_generic_and_element_paths(L, dt):
+    """NaN / inf / signed zero / subnormal handling must not depend on which kernel
+    runs: 9 inputs take the any-k kernel, mismatched alignment the element kernel."""
+    import torch
+    npdt = np.dtype(O.NP_OF[dt])
+    if dt == O.BF16:
+        sp = np.array([0x0000, 0x8000, 0x7f80, 0xff80, 0x7fc0, 0x0001, 0x8001, 0x0080, 0x7f7f, 0xff7f,
+                       0x3f80, 0xbf80, 0x3f81, 0x4040, 0x007f, 0x4b80], dtype=np.uint16)
+    else:
+        fi = np.finfo(npdt)
+        sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, fi.smallest_subnormal, -fi.smallest_subnormal, fi.tiny,
+                       fi.max, -fi.max, 1.0, -1.0, 1.0 + fi.eps, 3.0, fi.tiny / 2, 2.0 ** (fi.nmant + 1)], dtype=npdt)
+    m = len(sp)
+    rows = [np.ascontiguousarray(np.roll(np.tile(sp, m), 3 * j) if j % 2 else np.repeat(sp, m)) for j in range(9)]
+    ts = O.type_size(dt)
+    for op in ALL_OPS:
+        rc, want = O.reduce(rows, dt, op)
+        got = gpu_reduce(L, rows, dt, op)                       # k = 9: any-k kernel
+        assert same(got, want, nan_class=arith_nan_ok(dt, op), dtype=dt), (DT_NAME[dt], OP_NAME[op], "k9")
+        # k = 3 with one input offset by one element: element kernel
+        pads = [np.concatenate([r, r[:4]]) for r in rows[:3]]
+        devs = [to_dev(p) for p in pads]
+        out = dev_empty(m * m, ts)
+        views = [devs[0][1:1 + m * m], devs[1][0:m * m], devs[2][0:m * m]]
+        L.reduce(views, out, op, dtype=dt)
+        torch.cuda.synchronize()
+        rc, want = O.reduce([np.ascontiguousarray(pads[0][1:1 + m * m]), rows[1], rows[2]], dt, op)
+        assert same(from_dev(out, npdt), want, nan_class=arith_nan_ok(dt, op), dtype=dt), (DT_NAME[dt], OP_NAME[op], "elem")
