@@ -255,37 +255,55 @@ __global__ void __launch_bounds__(64) reduceBatchKernel(ReduceBatchParams<K> bp)
   reduceWaveBody<T, OP, K, U>(bp.seg[blockIdx.y]);
 }
 
-// Aligned body, any k up to FLAGCX_MAX_RANKS: inputs are consumed in batches of
-// eight loads so that the memory pipeline stays full without k-specific code.
-template <typename T, int OP, int BLOCK, bool NT>
-__global__ void __launch_bounds__(BLOCK) reduceVecAnyKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
+// Aligned body, any k up to FLAGCX_MAX_RANKS, same streaming shape as above: one
+// wavefront per workgroup, one KiB of every input per tile.  Inputs are consumed in
+// order in batches of eight loads; the accumulators stay in registers between
+// batches, so the fold and its single final rounding are unchanged.
+template <typename T, int OP>
+__global__ void __launch_bounds__(64) reduceWaveAnyKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
   typedef Fold<T, OP> F;
   constexpr int N = 16 / sizeof(T);
   constexpr int B = 8;
+  constexpr uint32_t kTileBytes = 1024u;
   const int k = p.k;
-  const uint64_t stride = (uint64_t)gridDim.x * BLOCK;
-  for (uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x; i < p.nvec; i += stride) {
+  const uint64_t bodyBytes = p.nvec * 16;
+  const uint64_t ntiles = (bodyBytes + kTileBytes - 1) / kTileBytes;
+  const uint64_t headBytes = p.head * sizeof(T);
+  const uint32_t voff = threadIdx.x * 16u;
+  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const uint64_t off = t * kTileBytes;
+    const uint64_t left = bodyBytes - off;
+    const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
     typename F::acc_t acc[N];
-    Vec16<T> x;
-    x.v = loadVec<NT>((const u32x4 *)((const T *)p.src[0] + p.head) + i);
-#pragma unroll
-    for (int e = 0; e < N; e++) acc[e] = F::init(x.e[e]);
-    for (int j0 = 1; j0 < k; j0 += B) {
+    for (int j0 = 0; j0 < k; j0 += B) {
       u32x4 in[B];
 #pragma unroll
       for (int b = 0; b < B; b++)
-        if (j0 + b < k) in[b] = loadVec<NT>((const u32x4 *)((const T *)p.src[j0 + b] + p.head) + i);
+        if (j0 + b < k) {
+          __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+              (void *)((const char *)p.src[j0 + b] + headBytes + off), 0, span, kRsrcFlags);
+          in[b] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kLoadAux);
+        }
 #pragma unroll
       for (int b = 0; b < B; b++)
         if (j0 + b < k) {
+          Vec16<T> x;
           x.v = in[b];
+          if (j0 + b == 0) {
 #pragma unroll
-          for (int e = 0; e < N; e++) acc[e] = F::step(x.e[e], acc[e]);
+            for (int e = 0; e < N; e++) acc[e] = F::init(x.e[e]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < N; e++) acc[e] = F::step(x.e[e], acc[e]);
+          }
         }
     }
+    Vec16<T> r;
 #pragma unroll
-    for (int e = 0; e < N; e++) x.e[e] = F::fin(acc[e], k);
-    storeVec<NT>((u32x4 *)((T *)p.dst + p.head) + i, x.v);
+    for (int e = 0; e < N; e++) r.e[e] = F::fin(acc[e], k);
+    __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((char *)p.dst + headBytes + off), 0, span, kRsrcFlags);
+    __builtin_amdgcn_raw_buffer_store_b128(r.v, rd, voff, 0, kStoreAux);
   }
   if (blockIdx.x == gridDim.x - 1) {
     const uint64_t edge = p.head + p.tail;

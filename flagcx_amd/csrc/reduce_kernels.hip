@@ -99,16 +99,20 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   p.head = s.head;
   p.tail = s.tail;
   p.k = c.k;
+  if (s.vector) {
+    uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
+    if (tiles < 1) tiles = 1;
+    if (tiles > kMaxGrid) tiles = kMaxGrid;
+    const int lds = ldsReservation(wavesPerCUFor(8));
+    reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
+    return (int)hipGetLastError();
+  }
   constexpr int BLOCK = 256;
-  const uint64_t work = s.vector ? s.nvec : s.tail;
-  uint64_t blocks = (work + BLOCK - 1) / BLOCK;
+  uint64_t blocks = (s.tail + BLOCK - 1) / BLOCK;
   const uint64_t cap = (uint64_t)deviceInfo().numCU * 32;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
-  if (s.vector)
-    reduceVecAnyKernel<elem_t, OP, BLOCK, true><<<dim3((unsigned)blocks), dim3(BLOCK), 0, c.stream>>>(p);
-  else
-    reduceElemKernel<elem_t, OP, BLOCK><<<dim3((unsigned)blocks), dim3(BLOCK), 0, c.stream>>>(p);
+  reduceElemKernel<elem_t, OP, BLOCK><<<dim3((unsigned)blocks), dim3(BLOCK), 0, c.stream>>>(p);
   return (int)hipGetLastError();
 }
 
