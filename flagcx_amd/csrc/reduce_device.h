@@ -141,15 +141,6 @@ union Vec16 {
   T e[16 / sizeof(T)];
 };
 
-template <bool NT>
-__device__ __forceinline__ u32x4 loadVec(const u32x4 *p) {
-  return NT ? __builtin_nontemporal_load(p) : *p;
-}
-template <bool NT>
-__device__ __forceinline__ void storeVec(u32x4 *p, u32x4 v) {
-  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
-}
-
 // Fold one 16-byte vector position across K registers.
 template <typename T, int OP, int K>
 __device__ __forceinline__ u32x4 foldVec(const u32x4 (&in)[K], int k) {
@@ -171,7 +162,7 @@ __device__ __forceinline__ u32x4 foldVec(const u32x4 (&in)[K], int k) {
   return r.v;
 }
 
-// One element, inputs addressed individually (head/tail and unaligned path).
+// One element, inputs addressed individually (head and tail elements).
 template <typename T, int OP>
 __device__ __forceinline__ void foldScalar(const void *const *src, int k, void *dst, uint64_t i) {
   typedef Fold<T, OP> F;
@@ -314,13 +305,60 @@ __global__ void __launch_bounds__(64) reduceWaveAnyKernel(ReduceParams<FLAGCX_MA
   }
 }
 
-// Pointers that do not share an address modulo 16: one element per lane per step
-// (still coalesced).  p.tail carries the element count.
-template <typename T, int OP, int BLOCK>
-__global__ void __launch_bounds__(BLOCK) reduceElemKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
-  const uint64_t stride = (uint64_t)gridDim.x * BLOCK;
-  for (uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x; i < p.tail; i += stride)
-    foldScalar<T, OP>(p.src, p.k, p.dst, i);
+// Sources that do not share the destination's address modulo 16.  The tiling is
+// the destination's (aligned 16-byte stores after p.head elements); each source
+// is read with 16-byte loads at whatever byte offset it happens to have, which
+// the hardware's unaligned access mode serves from at most one extra cache line
+// per wavefront request.  Plain global loads: a clipped buffer descriptor would
+// need an aligned base.
+typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(64) reduceWaveUnalignedKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
+  typedef Fold<T, OP> F;
+  constexpr int N = 16 / sizeof(T);
+  constexpr int B = 8;
+  const int k = p.k;
+  const uint64_t ntiles = (p.nvec + 63) / 64;
+  const uint64_t headBytes = p.head * sizeof(T);
+  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const uint64_t i = t * 64 + threadIdx.x;
+    if (i < p.nvec) {
+      typename F::acc_t acc[N];
+      for (int j0 = 0; j0 < k; j0 += B) {
+        u32x4 in[B];
+#pragma unroll
+        for (int b = 0; b < B; b++)
+          if (j0 + b < k)
+            in[b] = __builtin_nontemporal_load(
+                (const u32x4_unaligned *)((const char *)p.src[j0 + b] + headBytes + i * 16));
+#pragma unroll
+        for (int b = 0; b < B; b++)
+          if (j0 + b < k) {
+            Vec16<T> x;
+            x.v = in[b];
+            if (j0 + b == 0) {
+#pragma unroll
+              for (int e = 0; e < N; e++) acc[e] = F::init(x.e[e]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < N; e++) acc[e] = F::step(x.e[e], acc[e]);
+            }
+          }
+      }
+      Vec16<T> r;
+#pragma unroll
+      for (int e = 0; e < N; e++) r.e[e] = F::fin(acc[e], k);
+      *(u32x4 *)((char *)p.dst + headBytes + i * 16) = r.v;
+    }
+  }
+  if (blockIdx.x == gridDim.x - 1) {
+    const uint64_t edge = p.head + p.tail;
+    if (threadIdx.x < edge) {
+      uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
+      foldScalar<T, OP>(p.src, k, p.dst, i);
+    }
+  }
 }
 
 } // namespace flagcx_amd

@@ -47,21 +47,18 @@ constexpr uint64_t kMaxGrid = 1u << 24;
 
 struct Split {
   uint64_t head, nvec, tail;
-  bool vector;
+  bool vector; // every pointer shares the destination's offset inside a 16-byte line
 };
 
-// Decide between the 16-byte path and the element path.  The 16-byte path needs
-// every pointer at the same offset inside a 16-byte line.
+// The body is tiled on the destination: head elements up to its next 16-byte
+// line, then whole vectors, then a tail.  Sources at another offset modulo 16
+// take the unaligned-load kernel.
 static Split splitFor(const ReduceCall &c) {
   constexpr uint64_t N = 16 / sizeof(elem_t);
   Split s{0, 0, 0, true};
   const uintptr_t mis = (uintptr_t)c.dst & 15u;
   for (int j = 0; j < c.k; j++)
     if (((uintptr_t)c.src[j] & 15u) != mis) s.vector = false;
-  if (!s.vector) {
-    s.tail = c.count;
-    return s;
-  }
   uint64_t head = ((16u - mis) & 15u) / sizeof(elem_t);
   if (head > c.count) head = c.count;
   s.head = head;
@@ -99,20 +96,14 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   p.head = s.head;
   p.tail = s.tail;
   p.k = c.k;
-  if (s.vector) {
-    uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
-    if (tiles < 1) tiles = 1;
-    if (tiles > kMaxGrid) tiles = kMaxGrid;
-    const int lds = ldsReservation(wavesPerCUFor(8));
+  uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
+  if (tiles < 1) tiles = 1;
+  if (tiles > kMaxGrid) tiles = kMaxGrid;
+  const int lds = ldsReservation(wavesPerCUFor(c.k > 8 ? 8 : c.k));
+  if (s.vector)
     reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
-    return (int)hipGetLastError();
-  }
-  constexpr int BLOCK = 256;
-  uint64_t blocks = (s.tail + BLOCK - 1) / BLOCK;
-  const uint64_t cap = (uint64_t)deviceInfo().numCU * 32;
-  if (blocks > cap) blocks = cap;
-  if (blocks < 1) blocks = 1;
-  reduceElemKernel<elem_t, OP, BLOCK><<<dim3((unsigned)blocks), dim3(BLOCK), 0, c.stream>>>(p);
+  else
+    reduceWaveUnalignedKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
   return (int)hipGetLastError();
 }
 
