@@ -6,9 +6,10 @@
 // 1 KiB request and a tile is U consecutive KiB of one chunk.  blockIdx.y walks
 // chunks (or list entries), blockIdx.x walks tiles inside a chunk.  Buffer
 // descriptors are clipped to the tile, so ragged chunk ends need no branches.
-// Bytes that cannot be moved as 16-byte vectors (different address modulo 16 on
-// the two sides, chunk sizes or strides that are not multiples of 16) go through
-// an element path at the widest width every address shares.
+// A contiguous copy whose two sides differ modulo 16 is tiled on the destination
+// and reads its source with unaligned 16-byte loads; strided forms whose chunk
+// sizes or strides are not multiples of 16 go through an element path at the
+// widest width every address shares.
 // HBM bound: 2 bytes of traffic per payload byte (1 for fills); no LDS, no MFMA.
 #include "launch.h"
 #include "reduce_device.h"
@@ -76,6 +77,29 @@ __global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p) {
 template <int U, int LIST>
 __global__ void __launch_bounds__(64) copyWaveListKernel(CopyParams p, ListParams l) {
   copyWaveBody<U, LIST>(p, &l);
+}
+
+// One contiguous run whose two sides sit at different offsets modulo 16: tiled on
+// the destination (aligned stores), source read with unaligned 16-byte loads.
+__global__ void __launch_bounds__(64) copyWaveUnalignedKernel(CopyParams p, const char *src0, char *dst0) {
+  const uint64_t nvec = p.body / 16;
+  const uint64_t ntiles = (nvec + 63) / 64;
+  const char *s = src0 + p.head;
+  char *d = dst0 + p.head;
+  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const uint64_t i = t * 64 + threadIdx.x;
+    if (i < nvec) {
+      const u32x4 v = __builtin_nontemporal_load((const u32x4_unaligned *)(s + i * 16));
+      *(u32x4 *)(d + i * 16) = v;
+    }
+  }
+  if (blockIdx.x == gridDim.x - 1) {
+    const uint64_t edge = p.head + p.tail;
+    if (threadIdx.x < edge) {
+      const uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.body + (threadIdx.x - p.head);
+      dst0[i] = src0[i];
+    }
+  }
 }
 
 // Element path: W-byte units, chunk by chunk.
@@ -170,14 +194,22 @@ int launchCopy2D(const Copy2D &c) {
 
   bool vector;
   if (c.nchunks == 1) {
-    // one contiguous run: peel bytes up to the next 16-byte line, then vectors
+    // one contiguous run: peel bytes up to the destination's next 16-byte line,
+    // then vectors; a source at another offset modulo 16 is read unaligned
+    const char *src0 = list == 1 ? l.src[0] : p.src;
+    char *dst0 = list == 2 ? l.dst[0] : p.dst;
+    uint64_t head = (16u - lowBits((uint64_t)dst0)) & 15u;
+    if (head > c.chunkBytes) head = c.chunkBytes;
+    p.head = head;
+    p.body = (c.chunkBytes - head) & ~15ull;
+    p.tail = c.chunkBytes - head - p.body;
     vector = sameMis;
-    if (vector) {
-      uint64_t head = (16u - lowBits((uint64_t)(list == 2 ? (uint64_t)l.dst[0] : (uint64_t)c.dst))) & 15u;
-      if (head > c.chunkBytes) head = c.chunkBytes;
-      p.head = head;
-      p.body = (c.chunkBytes - head) & ~15ull;
-      p.tail = c.chunkBytes - head - p.body;
+    if (!vector) {
+      uint64_t gx = (p.body / 16 + 63) / 64;
+      if (gx < 1) gx = 1;
+      if (gx > kMaxGridX) gx = kMaxGridX;
+      copyWaveUnalignedKernel<<<dim3((unsigned)gx), dim3(64), 0, c.stream>>>(p, src0, dst0);
+      return (int)hipGetLastError();
     }
   } else {
     vector = allAligned && (c.chunkBytes & 15u) == 0;
