@@ -106,6 +106,26 @@ ReduceLauncher reduceLauncherFor(int dtype) {
 }
 
 // ----------------------------------------------------------------- helpers
+// Enum arguments arrive from C callers and may hold any int; read their bits
+// instead of loading them as enums so that out-of-range values stay defined.
+template <typename E>
+static inline int bitsOf(const E &e) {
+  static_assert(sizeof(E) == sizeof(int), "flagcx enums are int sized");
+  int v;
+  memcpy(&v, &e, sizeof(v));
+  return v;
+}
+
+static inline size_t typeSize(int dt) {
+  switch (dt) {
+    case flagcxInt8: case flagcxUint8: return 1;
+    case flagcxFloat16: case flagcxBfloat16: return 2;
+    case flagcxInt32: case flagcxUint32: case flagcxFloat: return 4;
+    case flagcxInt64: case flagcxUint64: case flagcxFloat64: return 8;
+    default: return 0;
+  }
+}
+
 // First member of the AMD stream wrapper is the hipStream_t
 // (flagcx/adaptor/include/amd_adaptor.h:14-16).
 static inline hipStream_t hipStreamOf(flagcxStream_t s) {
@@ -131,7 +151,7 @@ static flagcxResult_t prepareReduce(const void *const *srcs, int k, void *dst, u
                                     int dtype, int op, hipStream_t stream, const char *who,
                                     ReduceCall &c, bool *empty) {
   *empty = true;
-  const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
+  const size_t ts = typeSize(dtype);
   if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, dtype);
   if (op < 0 || op >= (int)flagcxNumRedOps)
     return fail(flagcxInvalidArgument, "%s: unsupported reduction operation %d", who, op);
@@ -194,15 +214,7 @@ using namespace flagcx_amd;
 #pragma GCC visibility push(default)
 extern "C" {
 
-size_t flagcxLocalGetDataTypeSize(flagcxDataType_t dtype) {
-  switch ((int)dtype) {
-    case flagcxInt8: case flagcxUint8: return 1;
-    case flagcxFloat16: case flagcxBfloat16: return 2;
-    case flagcxInt32: case flagcxUint32: case flagcxFloat: return 4;
-    case flagcxInt64: case flagcxUint64: case flagcxFloat64: return 8;
-    default: return 0;
-  }
-}
+size_t flagcxLocalGetDataTypeSize(flagcxDataType_t dtype) { return typeSize(bitsOf(dtype)); }
 
 flagcxResult_t flagcxLocalInit(void) {
   (void)deviceInfo();
@@ -211,7 +223,7 @@ flagcxResult_t flagcxLocalInit(void) {
 }
 
 const char *flagcxLocalGetErrorString(flagcxResult_t result) {
-  switch ((int)result) {
+  switch (bitsOf(result)) {
     case flagcxSuccess: return "no error";
     case flagcxUnhandledDeviceError: return "unhandled device error";
     case flagcxSystemError: return "unhandled system error";
@@ -246,7 +258,7 @@ flagcxResult_t flagcxLocalReduce(const void *const *sendbuffs, int nranks, void 
                                  size_t count, flagcxDataType_t datatype, flagcxRedOp_t op,
                                  flagcxStream_t stream) {
   if (!sendbuffs) return fail(flagcxInvalidArgument, "flagcxLocalReduce: sendbuffs is NULL");
-  flagcxResult_t r = reduceOrdered(sendbuffs, nranks, recvbuff, count, (int)datatype, (int)op,
+  flagcxResult_t r = reduceOrdered(sendbuffs, nranks, recvbuff, count, bitsOf(datatype), bitsOf(op),
                                    hipStreamOf(stream), "flagcxLocalReduce");
   if (r != flagcxSuccess) return r;
   return finish(stream, 0, "flagcxLocalReduce");
@@ -265,7 +277,8 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
   if (ndescs < 0) return fail(flagcxInvalidArgument, "%s: ndescs %d is negative", who, ndescs);
   if (ndescs == 0) return flagcxSuccess;
   if (!descs) return fail(flagcxInvalidArgument, "%s: descs is NULL", who);
-  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  const int dt = bitsOf(datatype), rop = bitsOf(op);
+  const size_t ts = typeSize(dt);
   hipStream_t hs = hipStreamOf(stream);
   constexpr int kGroup = 64;
   ReduceCall calls[kGroup];
@@ -276,8 +289,8 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
       const flagcxLocalReduceDesc &d = descs[base + i];
       if (!d.sendbuffs) return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs is NULL", who, base + i);
       bool empty;
-      flagcxResult_t r = prepareReduce(d.sendbuffs, nranks, d.recvbuff, d.count, (int)datatype, (int)op,
-                                       hs, who, calls[ncalls], &empty);
+      flagcxResult_t r = prepareReduce(d.sendbuffs, nranks, d.recvbuff, d.count, dt, rop, hs, who,
+                                       calls[ncalls], &empty);
       if (r != flagcxSuccess) return r;
       if (empty) continue;
       for (int e = 0; e < ncalls; e++)
@@ -286,7 +299,7 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
           return fail(flagcxInvalidArgument, "%s: recvbuff of descs[%d] overlaps an earlier one", who, base + i);
       ncalls++;
     }
-    flagcxResult_t r = launchBatch(calls, ncalls, (int)datatype, who);
+    flagcxResult_t r = launchBatch(calls, ncalls, dt, who);
     if (r != flagcxSuccess) return r;
   }
   return finish(stream, 0, who);
@@ -309,7 +322,7 @@ flagcxResult_t flagcxLocalReduceTriggers(const flagcxLocalReduceTrigger *trigger
     void *res = (void *)(uintptr_t)v[2];
     const uint64_t count = v[3] & 0xffffffffull;
     const int dt = (int)((v[3] >> 48) & 0xf), op = (int)((v[3] >> 52) & 0xf);
-    const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dt);
+    const size_t ts = typeSize(dt);
     const uint64_t bytes = count * ts;
     // a trigger that touches what an earlier trigger of the group writes, or
     // writes what one reads, must wait for it: close the group first
@@ -344,17 +357,16 @@ flagcxResult_t flagcxLocalReduceTriggers(const flagcxLocalReduceTrigger *trigger
   return finish(stream, 0, who);
 }
 
-flagcxResult_t flagcxLocalReduceScatterChunked(const void *const *sendbuffs, int nranks, int rank,
-                                               void *recvbuff, size_t recvcount,
-                                               flagcxDataType_t datatype, flagcxRedOp_t op,
-                                               size_t chunkbytes, flagcxStream_t stream) {
+static flagcxResult_t reduceScatterImpl(const void *const *sendbuffs, int nranks, int rank, void *recvbuff,
+                                        size_t recvcount, int dt, int rop, size_t chunkbytes,
+                                        flagcxStream_t stream) {
   const char *who = "flagcxLocalReduceScatter";
   if (!sendbuffs) return fail(flagcxInvalidArgument, "%s: sendbuffs is NULL", who);
   if (nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS)
     return fail(flagcxInvalidArgument, "%s: nranks %d outside [1, %d]", who, nranks, FLAGCX_LOCAL_MAX_RANKS);
   if (rank < 0 || rank >= nranks) return fail(flagcxInvalidArgument, "%s: rank %d outside [0, %d)", who, rank, nranks);
-  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
-  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, (int)datatype);
+  const size_t ts = typeSize(dt);
+  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, dt);
   if (chunkbytes == 0) chunkbytes = recvcount * ts ? recvcount * ts : ts; // one launch
   if (chunkbytes % ts) return fail(flagcxInvalidArgument, "%s: chunkbytes %zu not a multiple of %zu", who, chunkbytes, ts);
   for (int j = 0; j < nranks; j++)
@@ -370,24 +382,31 @@ flagcxResult_t flagcxLocalReduceScatterChunked(const void *const *sendbuffs, int
       const int r = (rank + 1 + j) % nranks;
       ordered[j] = (const char *)sendbuffs[r] + ((size_t)rank * recvcount + done) * ts;
     }
-    flagcxResult_t res = reduceOrdered(ordered, nranks, (char *)recvbuff + done * ts, n, (int)datatype,
-                                       (int)op, hs, who);
+    flagcxResult_t res = reduceOrdered(ordered, nranks, (char *)recvbuff + done * ts, n, dt, rop, hs, who);
     if (res != flagcxSuccess) return res;
     done += n;
   } while (done < recvcount);
   return finish(stream, 0, who);
 }
 
+flagcxResult_t flagcxLocalReduceScatterChunked(const void *const *sendbuffs, int nranks, int rank,
+                                               void *recvbuff, size_t recvcount,
+                                               flagcxDataType_t datatype, flagcxRedOp_t op,
+                                               size_t chunkbytes, flagcxStream_t stream) {
+  return reduceScatterImpl(sendbuffs, nranks, rank, recvbuff, recvcount, bitsOf(datatype), bitsOf(op),
+                           chunkbytes, stream);
+}
+
 flagcxResult_t flagcxLocalReduceScatter(const void *const *sendbuffs, int nranks, int rank,
                                         void *recvbuff, size_t recvcount, flagcxDataType_t datatype,
                                         flagcxRedOp_t op, flagcxStream_t stream) {
-  return flagcxLocalReduceScatterChunked(sendbuffs, nranks, rank, recvbuff, recvcount, datatype, op, 0,
-                                         stream);
+  return reduceScatterImpl(sendbuffs, nranks, rank, recvbuff, recvcount, bitsOf(datatype), bitsOf(op), 0,
+                           stream);
 }
 
 flagcxResult_t flagcxLocalRingChunkTable(size_t count, flagcxDataType_t datatype, int nranks,
                                          size_t *offsets, size_t *lengths) {
-  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  const size_t ts = typeSize(bitsOf(datatype));
   if (!ts || nranks < 1 || !offsets || !lengths)
     return fail(flagcxInvalidArgument, "flagcxLocalRingChunkTable: bad argument");
   ringChunkTable((uint64_t)count * ts, ts, nranks, offsets, lengths);
@@ -401,8 +420,9 @@ flagcxResult_t flagcxLocalAllReduce(const void *const *sendbuffs, int nranks, vo
   if (!sendbuffs) return fail(flagcxInvalidArgument, "%s: sendbuffs is NULL", who);
   if (nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS)
     return fail(flagcxInvalidArgument, "%s: nranks %d outside [1, %d]", who, nranks, FLAGCX_LOCAL_MAX_RANKS);
-  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
-  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, (int)datatype);
+  const int dt = bitsOf(datatype), rop = bitsOf(op);
+  const size_t ts = typeSize(dt);
+  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, dt);
   for (int j = 0; j < nranks; j++)
     if (!sendbuffs[j]) return fail(flagcxInvalidArgument, "%s: sendbuffs[%d] is NULL", who, j);
   size_t offset[FLAGCX_LOCAL_MAX_RANKS], length[FLAGCX_LOCAL_MAX_RANKS];
@@ -410,8 +430,8 @@ flagcxResult_t flagcxLocalAllReduce(const void *const *sendbuffs, int nranks, vo
   hipStream_t hs = hipStreamOf(stream);
   const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
   // The validation of op has to happen even when every chunk is empty.
-  if ((int)op < 0 || (int)op >= (int)flagcxNumRedOps)
-    return fail(flagcxInvalidArgument, "%s: unsupported reduction operation %d", who, (int)op);
+  if (rop < 0 || rop >= (int)flagcxNumRedOps)
+    return fail(flagcxInvalidArgument, "%s: unsupported reduction operation %d", who, rop);
   ReduceCall calls[FLAGCX_LOCAL_MAX_RANKS];
   int ncalls = 0;
   for (int c = 0; c < nranks; c++) {
@@ -420,14 +440,14 @@ flagcxResult_t flagcxLocalAllReduce(const void *const *sendbuffs, int nranks, vo
       ordered[j] = (const char *)sendbuffs[(c + 1 + j) % nranks] + offset[c];
     bool empty;
     flagcxResult_t res = prepareReduce(ordered, nranks, (char *)recvbuff + offset[c], length[c] / ts,
-                                       (int)datatype, (int)op, hs, who, calls[ncalls], &empty);
+                                       dt, rop, hs, who, calls[ncalls], &empty);
     if (res != flagcxSuccess) return res;
     if (!empty) ncalls++;
   }
   if (ncalls == 0) return flagcxSuccess;
   (void)deviceInfo();
   // all chunks in one launch; each chunk keeps its own fold order
-  return finish(stream, reduceBatchLauncherFor((int)datatype)(calls, ncalls), who);
+  return finish(stream, reduceBatchLauncherFor(dt)(calls, ncalls), who);
 }
 
 // ------------------------------------------------------------ byte movers
@@ -458,11 +478,11 @@ flagcxResult_t flagcxLocalRefresh(void *buff, size_t start, size_t offset, size_
                                   size_t totalcount, flagcxDataType_t datatype, flagcxRedOp_t op,
                                   flagcxStream_t stream) {
   const char *who = "flagcxLocalRefresh";
-  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
-  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, (int)datatype);
+  const size_t ts = typeSize(bitsOf(datatype));
+  if (!ts) return fail(flagcxInvalidArgument, "%s: unsupported data type %d", who, bitsOf(datatype));
   if (offset + count > totalcount || offset + count < offset)
     return fail(flagcxInvalidArgument, "%s: offset %zu + count %zu exceeds totalcount %zu", who, offset, count, totalcount);
-  if (op != flagcxSum) return flagcxSuccess; // flagcx/core/c2c_algo.cc:596
+  if (bitsOf(op) != flagcxSum) return flagcxSuccess; // flagcx/core/c2c_algo.cc:596
   if (totalcount == count) return flagcxSuccess;
   if (!buff) return fail(flagcxInvalidArgument, "%s: NULL pointer", who);
   char *base = (char *)buff + start * ts;
@@ -534,8 +554,14 @@ flagcxResult_t flagcxLocalUnpackList(void *const *dsts, const void *src, int n, 
 void flagcxLocalReduceFunc(flagcxStream_t stream, void *args) {
   flagcxLocalReduceArgs *a = static_cast<flagcxLocalReduceArgs *>(args);
   if (!a) return;
-  a->result = (int32_t)flagcxLocalReduce(a->sendbuffs, a->nranks, a->recvbuff, (size_t)a->count,
-                                         (flagcxDataType_t)a->datatype, (flagcxRedOp_t)a->op, stream);
+  if (!a->sendbuffs) {
+    a->result = (int32_t)fail(flagcxInvalidArgument, "flagcxLocalReduceFunc: sendbuffs is NULL");
+    return;
+  }
+  flagcxResult_t r = reduceOrdered(a->sendbuffs, a->nranks, a->recvbuff, (uint64_t)a->count, a->datatype, a->op,
+                                   hipStreamOf(stream), "flagcxLocalReduceFunc");
+  if (r == flagcxSuccess) r = finish(stream, 0, "flagcxLocalReduceFunc");
+  a->result = (int32_t)r;
 }
 
 void flagcxLocalCopyFunc(flagcxStream_t stream, void *args) {

@@ -438,8 +438,8 @@ flagcxResult_t flagcxLocalPlanCreate(flagcxLocalPlan **plan, int nranks, const i
   flagcxLocalPlan *p = new flagcxLocalPlan();
   p->nranks = nranks;
   p->totalCount = totalCount;
-  p->commOp = (int)commOp;
-  p->redOp = (int)redOp;
+  memcpy(&p->commOp, &commOp, sizeof(int)); // enum bits as they came from the caller
+  memcpy(&p->redOp, &redOp, sizeof(int));
   int ncl = 0;
   for (int r = 0; r < nranks; r++) {
     if (clusterIds[r] < 0 || clusterIds[r] >= nranks) { delete p; return flagcxInvalidArgument; }

@@ -31,10 +31,20 @@ namespace {
 
 inline hipStream_t hs(flagcxStream_t s) { return s ? s->base : nullptr; }
 
+// Enum arguments come from C callers and may hold any int: read their bits.
+template <typename E>
+inline int bitsOf(const E &e) {
+  static_assert(sizeof(E) == sizeof(int), "flagcx enums are int sized");
+  int v;
+  memcpy(&v, &e, sizeof(v));
+  return v;
+}
+
 flagcxResult_t aDeviceSynchronize(void) { DEV(hipDeviceSynchronize()); return flagcxSuccess; }
 
-flagcxResult_t aDeviceMemcpy(void *dst, void *src, size_t size, flagcxMemcpyType_t type, flagcxStream_t stream,
+flagcxResult_t aDeviceMemcpy(void *dst, void *src, size_t size, flagcxMemcpyType_t type_, flagcxStream_t stream,
                              void *) {
+  const int type = bitsOf(type_);
   if (type == flagcxMemcpyDeviceToDevice) return flagcxLocalMemcpy(dst, src, size, stream);
   const hipMemcpyKind kind = type == flagcxMemcpyHostToDevice ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost;
   if (type != flagcxMemcpyHostToDevice && type != flagcxMemcpyDeviceToHost) return flagcxInvalidArgument;
@@ -44,7 +54,7 @@ flagcxResult_t aDeviceMemcpy(void *dst, void *src, size_t size, flagcxMemcpyType
 }
 
 flagcxResult_t aDeviceMemset(void *ptr, int value, size_t size, flagcxMemType_t type, flagcxStream_t stream) {
-  if (type == flagcxMemHost) {
+  if (bitsOf(type) == flagcxMemHost) {
     if (!ptr && size) return flagcxInvalidArgument;
     memset(ptr, value, size);
     return flagcxSuccess;
@@ -54,7 +64,7 @@ flagcxResult_t aDeviceMemset(void *ptr, int value, size_t size, flagcxMemType_t 
 
 flagcxResult_t aDeviceMalloc(void **ptr, size_t size, flagcxMemType_t type, flagcxStream_t stream) {
   if (!ptr) return flagcxInvalidArgument;
-  switch (type) {
+  switch (bitsOf(type)) {
     case flagcxMemHost: DEV(hipHostMalloc(ptr, size, hipHostMallocMapped)); break;
     case flagcxMemManaged: DEV(hipMallocManaged(ptr, size, hipMemAttachGlobal)); break;
     case flagcxMemDevice:
@@ -66,8 +76,9 @@ flagcxResult_t aDeviceMalloc(void **ptr, size_t size, flagcxMemType_t type, flag
   return flagcxSuccess;
 }
 
-flagcxResult_t aDeviceFree(void *ptr, flagcxMemType_t type, flagcxStream_t stream) {
+flagcxResult_t aDeviceFree(void *ptr, flagcxMemType_t type_, flagcxStream_t stream) {
   if (!ptr) return flagcxSuccess;
+  const int type = bitsOf(type_);
   if (type == flagcxMemHost) DEV(hipHostFree(ptr));
   else if (type == flagcxMemDevice && stream) DEV(hipFreeAsync(ptr, stream->base));
   else DEV(hipFree(ptr));
@@ -135,7 +146,7 @@ flagcxResult_t aEventCreate(flagcxEvent_t *event, flagcxEventType_t type) {
   if (!event) return flagcxInvalidArgument;
   flagcxEvent_t e = static_cast<flagcxEvent_t>(calloc(1, sizeof(struct flagcxEvent)));
   if (!e) return flagcxSystemError;
-  const unsigned flags = type == flagcxEventDisableTiming ? hipEventDisableTiming : hipEventDefault;
+  const unsigned flags = bitsOf(type) == flagcxEventDisableTiming ? hipEventDisableTiming : hipEventDefault;
   if (hipEventCreateWithFlags(&e->base, flags) != hipSuccess) { free(e); return flagcxUnhandledDeviceError; }
   *event = e;
   return flagcxSuccess;
