@@ -62,7 +62,7 @@ def build(verbose=False, jobs=None):
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
     # C++ programs that link the C ABI: timing driver and the collective test
     # (host-only C++; they reach the GPU through the library)
-    for prog in ("local_perf", "local_coll_test"):
+    for prog in ("local_perf", "local_coll_test", "fifo_perf"):
         src = os.path.join(HERE, "perf", prog + ".cpp")
         _run([HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", src, "-o",
               os.path.join(LIBDIR, prog), "-L" + LIBDIR, "-lflagcx_amd", "-Wl,-rpath,$ORIGIN"])

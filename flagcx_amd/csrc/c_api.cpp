@@ -97,6 +97,20 @@ ReduceBatchLauncher reduceBatchLauncherFor(int dtype) {
   return (dtype >= 0 && dtype < 10) ? table[dtype] : nullptr;
 }
 
+#define FLAGCX_DECL_QUEUE(n) \
+  int launchReduceQueue_##n(int, const QueueKernelArgs &, int, int, int, unsigned, hipStream_t, unsigned *);
+FLAGCX_DECL_QUEUE(0) FLAGCX_DECL_QUEUE(1) FLAGCX_DECL_QUEUE(2) FLAGCX_DECL_QUEUE(3) FLAGCX_DECL_QUEUE(4)
+FLAGCX_DECL_QUEUE(5) FLAGCX_DECL_QUEUE(6) FLAGCX_DECL_QUEUE(7) FLAGCX_DECL_QUEUE(8) FLAGCX_DECL_QUEUE(9)
+#undef FLAGCX_DECL_QUEUE
+
+ReduceQueueLauncher reduceQueueLauncherFor(int dtype) {
+  static const ReduceQueueLauncher table[10] = {
+      launchReduceQueue_0, launchReduceQueue_1, launchReduceQueue_2, launchReduceQueue_3,
+      launchReduceQueue_4, launchReduceQueue_5, launchReduceQueue_6, launchReduceQueue_7,
+      launchReduceQueue_8, launchReduceQueue_9};
+  return (dtype >= 0 && dtype < 10) ? table[dtype] : nullptr;
+}
+
 ReduceLauncher reduceLauncherFor(int dtype) {
   static const ReduceLauncher table[10] = {launchReduce_0, launchReduce_1, launchReduce_2,
                                            launchReduce_3, launchReduce_4, launchReduce_5,

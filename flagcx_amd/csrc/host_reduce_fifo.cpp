@@ -1,0 +1,334 @@
+// host_reduce_fifo.cpp - host side of the host-producer / device-consumer reduce
+// queue: the pair `enqueue(flagcxReduceTrigger)` / device `dequeue` that the
+// reference declares and leaves commented out
+// (flagcx/include/flagcx_kernel.h:52-73,96-98).  Allocation mirrors
+// flagcxFifo::flagcxFifoInit (flagcx/core/flagcx_kernel_host.cc:31-45): a pinned,
+// device-mapped buffer of 64-bit words [capacity, consumed, produced, ...] followed
+// by the entries; the consumer is one resident kernel on a stream the queue owns
+// (reduce_queue_device.h), the way the kernel proxy owns a dedicated stream
+// (flagcx/core/proxy.cc:1094-1097).
+//
+// A queue is typed (element type, op) when it is created: a collective has one
+// type and one op, and the consumer kernel is compiled per pair.  Entries carry
+// 1..8 inputs; the host validates every entry and splits it into head / 16-byte
+// body / tail before the device sees it.
+#include "../../include/flagcx_amd.h"
+#include "launch.h"
+
+#include <sched.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+using namespace flagcx_amd;
+
+struct flagcxLocalReduceFifo {
+  uint64_t *header = nullptr;       // pinned: kQueueHeaderWords words, then the entry ring
+  QueueEntry *hostEntries = nullptr;
+  void *devBlock = nullptr;         // device ring | devProduced | progress words
+  QueueEntry *devEntries = nullptr;
+  uint64_t *devProduced = nullptr;
+  uint32_t *progress = nullptr;
+  uint32_t capacity = 0;
+  unsigned maxGrid = 0;
+  unsigned grid = 0;
+  int maxRanks = 0, dtype = 0, op = 0;
+  size_t typeSize = 0;
+  hipStream_t stream = nullptr;
+  uint64_t produced = 0;            // host copy of header[kQueueProduced]
+  bool launched = false;            // a consumer has been launched and not yet joined
+  bool stopSent = false;
+  std::mutex mu;                    // producers may be several threads
+  char lastError[256] = "";
+};
+
+namespace {
+
+flagcxResult_t qfail(flagcxLocalReduceFifo *q, flagcxResult_t code, const char *fmt, ...)
+    __attribute__((format(printf, 3, 4)));
+flagcxResult_t qfail(flagcxLocalReduceFifo *q, flagcxResult_t code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  if (q) vsnprintf(q->lastError, sizeof(q->lastError), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+inline uint64_t headerLoad(const flagcxLocalReduceFifo *q, int word) {
+  return __atomic_load_n(q->header + word, __ATOMIC_ACQUIRE);
+}
+
+inline bool overlaps(uintptr_t x, uintptr_t y, uint64_t bytes) { return x < y + bytes && y < x + bytes; }
+
+// Appends one validated entry; the caller holds the mutex.
+flagcxResult_t appendEntry(flagcxLocalReduceFifo *q, const QueueEntry &e, uint64_t *ticket, const char *who) {
+  if (!q->launched || q->stopSent) return qfail(q, flagcxInvalidUsage, "%s: the queue is not running", who);
+  const uint64_t state = headerLoad(q, kQueueState);
+  if (state != kQueueRunning)
+    return qfail(q, flagcxInternalError, "%s: the consumer has exited (state %lld)", who, (long long)state);
+  if (q->produced - headerLoad(q, kQueueConsumed) >= q->capacity) return flagcxInProgress; // full: retry
+  memcpy(q->hostEntries + q->produced % q->capacity, &e, sizeof(e));
+  q->produced++;
+  __atomic_store_n(q->header + kQueueProduced, q->produced, __ATOMIC_RELEASE);
+  if (ticket) *ticket = q->produced;
+  return flagcxSuccess;
+}
+
+flagcxResult_t buildEntry(flagcxLocalReduceFifo *q, const void *const *srcs, int k, void *dst, uint64_t count,
+                          QueueEntry &e, bool *empty, const char *who) {
+  *empty = true;
+  if (k < 1 || k > q->maxRanks) return qfail(q, flagcxInvalidArgument, "%s: nranks %d outside [1, %d]", who, k, q->maxRanks);
+  if (count == 0) return flagcxSuccess;
+  const size_t ts = q->typeSize;
+  if (!dst) return qfail(q, flagcxInvalidArgument, "%s: recvbuff is NULL", who);
+  if ((uintptr_t)dst % ts) return qfail(q, flagcxInvalidArgument, "%s: recvbuff not aligned to its element size", who);
+  if (count > UINT64_MAX / ts) return qfail(q, flagcxInvalidArgument, "%s: count overflows", who);
+  const uint64_t bytes = count * ts;
+  memset(&e, 0, sizeof(e));
+  const uintptr_t mis = (uintptr_t)dst & 15u;
+  e.vector = 1;
+  for (int j = 0; j < k; j++) {
+    const uintptr_t s = (uintptr_t)srcs[j];
+    if (!s) return qfail(q, flagcxInvalidArgument, "%s: sendbuffs[%d] is NULL", who, j);
+    if (s % ts) return qfail(q, flagcxInvalidArgument, "%s: sendbuffs[%d] not aligned to its element size", who, j);
+    if (s != (uintptr_t)dst && overlaps(s, (uintptr_t)dst, bytes))
+      return qfail(q, flagcxInvalidArgument, "%s: recvbuff partially overlaps sendbuffs[%d]", who, j);
+    if ((s & 15u) != mis) e.vector = 0;
+    e.src[j] = (uint64_t)s;
+  }
+  e.dst = (uint64_t)(uintptr_t)dst;
+  const uint64_t perVec = 16 / ts;
+  uint64_t head = ((16u - mis) & 15u) / ts;
+  if (head > count) head = count;
+  e.head = (uint32_t)head;
+  e.nvec = (count - head) / perVec;
+  e.tail = (uint32_t)(count - head - e.nvec * perVec);
+  e.k = (uint32_t)k;
+  *empty = false;
+  return flagcxSuccess;
+}
+
+// Waits for the consumer kernel to leave the GPU and forgets it.
+flagcxResult_t joinConsumer(flagcxLocalReduceFifo *q) {
+  if (!q->launched) return flagcxSuccess;
+  const hipError_t e = hipStreamSynchronize(q->stream);
+  q->launched = false;
+  q->stopSent = false;
+  return e == hipSuccess ? flagcxSuccess
+                         : qfail(q, flagcxUnhandledDeviceError, "flagcxLocalReduceFifo: %s", hipGetErrorString(e));
+}
+
+} // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int capacity, int maxRanks,
+                                           flagcxDataType_t datatype, flagcxRedOp_t op) {
+  if (!fifo) return flagcxInvalidArgument;
+  *fifo = nullptr;
+  int dt, rop;
+  memcpy(&dt, &datatype, sizeof(int));
+  memcpy(&rop, &op, sizeof(int));
+  const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)(dt >= 0 && dt < (int)flagcxNumTypes ? dt : 0));
+  if (dt < 0 || dt >= (int)flagcxNumTypes || !ts || !reduceQueueLauncherFor(dt)) return flagcxInvalidArgument;
+  if (rop < 0 || rop >= (int)flagcxNumRedOps) return flagcxInvalidArgument;
+  if (capacity < 1 || capacity > 65536 || maxRanks < 1 || maxRanks > 8) return flagcxInvalidArgument;
+  flagcxLocalReduceFifo *q = new (std::nothrow) flagcxLocalReduceFifo;
+  if (!q) return flagcxSystemError;
+  q->capacity = (uint32_t)capacity;
+  q->maxRanks = maxRanks;
+  q->dtype = dt;
+  q->op = rop;
+  q->typeSize = ts;
+  const DeviceInfo &info = deviceInfo();
+  q->maxGrid = (unsigned)info.numCU * 16u;
+  const size_t hostBytes = kQueueHeaderWords * sizeof(uint64_t) + (size_t)capacity * sizeof(QueueEntry);
+  const size_t devBytes = (size_t)capacity * sizeof(QueueEntry) + 128 + (size_t)q->maxGrid * sizeof(uint64_t);
+  void *host = nullptr;
+  hipError_t e = hipHostMalloc(&host, hostBytes, hipHostMallocMapped);
+  if (e == hipSuccess) e = hipMalloc(&q->devBlock, devBytes);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&q->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    if (host) (void)hipHostFree(host);
+    if (q->devBlock) (void)hipFree(q->devBlock);
+    delete q;
+    return flagcxUnhandledDeviceError;
+  }
+  memset(host, 0, hostBytes);
+  q->header = static_cast<uint64_t *>(host);
+  q->header[kQueueCapacity] = (uint64_t)capacity;
+  q->hostEntries = reinterpret_cast<QueueEntry *>(q->header + kQueueHeaderWords);
+  q->devEntries = static_cast<QueueEntry *>(q->devBlock);
+  q->devProduced = reinterpret_cast<uint64_t *>(q->devEntries + capacity);
+  q->progress = reinterpret_cast<uint32_t *>(q->devProduced + 16);
+  *fifo = q;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduceFifoStart(flagcxLocalReduceFifo_t q) {
+  if (!q) return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(q->mu);
+  const char *who = "flagcxLocalReduceFifoStart";
+  if (q->launched) {
+    if (headerLoad(q, kQueueState) == kQueueRunning) return qfail(q, flagcxInvalidUsage, "%s: already running", who);
+    flagcxResult_t r = joinConsumer(q); // the previous consumer stopped or timed out
+    if (r != flagcxSuccess) return r;
+  }
+  q->produced = 0;
+  q->header[kQueueConsumed] = 0;
+  q->header[kQueueProduced] = 0;
+  __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueRunning, __ATOMIC_RELEASE);
+  const size_t clearBytes = 128 + (size_t)q->maxGrid * sizeof(uint64_t);
+  hipError_t e = hipMemsetAsync(q->devProduced, 0, clearBytes, q->stream);
+  if (e != hipSuccess) return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString(e));
+  QueueKernelArgs a;
+  a.hostHeader = q->header;
+  a.hostEntries = q->hostEntries;
+  a.devEntries = q->devEntries;
+  a.devProduced = q->devProduced;
+  a.progress = q->progress;
+  a.capacity = q->capacity;
+  a.maxSpin = asyncMaxSpin();
+  // LDS is reserved only to spread the resident wavefronts evenly over the CUs, in
+  // whole 1280-byte allocation granules so that exactly `waves` fit per CU
+  // (at most 16: half of a CU's wavefront slots, so that residency never depends
+  // on the last slot being free)
+  int waves = wavesPerCUFor(q->maxRanks);
+  if (waves <= 0 || waves > 16) waves = 16;
+  const int lds = (deviceInfo().ldsPerCU / waves) / 1280 * 1280;
+  const int err = reduceQueueLauncherFor(q->dtype)(q->op, a, waves, deviceInfo().numCU, lds, q->maxGrid, q->stream,
+                                                   &q->grid);
+  if (err) {
+    __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueIdle, __ATOMIC_RELEASE);
+    return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString((hipError_t)err));
+  }
+  q->launched = true;
+  q->stopSent = false;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduceFifoEnqueueReduce(flagcxLocalReduceFifo_t q, const void *const *sendbuffs, int nranks,
+                                                  void *recvbuff, size_t count, uint64_t *ticket) {
+  if (!q) return flagcxInvalidArgument;
+  const char *who = "flagcxLocalReduceFifoEnqueueReduce";
+  if (!sendbuffs) return qfail(q, flagcxInvalidArgument, "%s: sendbuffs is NULL", who);
+  std::lock_guard<std::mutex> lock(q->mu);
+  QueueEntry e;
+  bool empty;
+  flagcxResult_t r = buildEntry(q, sendbuffs, nranks, recvbuff, count, e, &empty, who);
+  if (r != flagcxSuccess) return r;
+  if (empty) {
+    if (ticket) *ticket = q->produced;
+    return flagcxSuccess;
+  }
+  return appendEntry(q, e, ticket, who);
+}
+
+flagcxResult_t flagcxLocalReduceFifoEnqueue(flagcxLocalReduceFifo_t q, const flagcxLocalReduceTrigger *trigger,
+                                            uint64_t *ticket) {
+  if (!q) return flagcxInvalidArgument;
+  const char *who = "flagcxLocalReduceFifoEnqueue";
+  if (!trigger) return qfail(q, flagcxInvalidArgument, "%s: trigger is NULL", who);
+  const uint64_t *v = trigger->value;
+  const int dt = (int)((v[3] >> 48) & 0xf), op = (int)((v[3] >> 52) & 0xf);
+  if (dt != q->dtype || op != q->op)
+    return qfail(q, flagcxInvalidArgument, "%s: trigger datatype %d / redop %d differ from the queue's", who, dt, op);
+  // addr3 = OP(addr1, addr2): fold order acc = addr2; acc = OP(addr1, acc)
+  const void *srcs[2] = {(const void *)(uintptr_t)v[1], (const void *)(uintptr_t)v[0]};
+  std::lock_guard<std::mutex> lock(q->mu);
+  if (q->maxRanks < 2) return qfail(q, flagcxInvalidArgument, "%s: the queue was created for one input", who);
+  QueueEntry e;
+  bool empty;
+  flagcxResult_t r = buildEntry(q, srcs, 2, (void *)(uintptr_t)v[2], v[3] & 0xffffffffull, e, &empty, who);
+  if (r != flagcxSuccess) return r;
+  if (empty) {
+    if (ticket) *ticket = q->produced;
+    return flagcxSuccess;
+  }
+  return appendEntry(q, e, ticket, who);
+}
+
+flagcxResult_t flagcxLocalReduceFifoQuery(flagcxLocalReduceFifo_t q, uint64_t *produced, uint64_t *consumed,
+                                          int *state) {
+  if (!q) return flagcxInvalidArgument;
+  if (consumed) *consumed = headerLoad(q, kQueueConsumed);
+  if (produced) *produced = headerLoad(q, kQueueProduced);
+  if (state) *state = (int)headerLoad(q, kQueueState);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduceFifoWait(flagcxLocalReduceFifo_t q, uint64_t ticket) {
+  if (!q) return flagcxInvalidArgument;
+  const char *who = "flagcxLocalReduceFifoWait";
+  if (ticket > headerLoad(q, kQueueProduced))
+    return qfail(q, flagcxInvalidArgument, "%s: ticket %lld has not been handed out", who, (long long)ticket);
+  for (;;) {
+    if (headerLoad(q, kQueueConsumed) >= ticket) return flagcxSuccess;
+    const uint64_t state = headerLoad(q, kQueueState);
+    if (state != kQueueRunning) {
+      if (headerLoad(q, kQueueConsumed) >= ticket) return flagcxSuccess;
+      return qfail(q, state == kQueueTimedOut ? flagcxInternalError : flagcxInvalidUsage,
+                   "%s: the consumer is not running (state %lld) and entry %lld was not reached", who,
+                   (long long)state, (long long)ticket);
+    }
+    sched_yield();
+  }
+}
+
+flagcxResult_t flagcxLocalReduceFifoStop(flagcxLocalReduceFifo_t q) {
+  if (!q) return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(q->mu);
+  if (!q->launched) return flagcxSuccess;
+  if (!q->stopSent && headerLoad(q, kQueueState) == kQueueRunning) {
+    QueueEntry e;
+    memset(&e, 0, sizeof(e)); // k = 0
+    // a full ring drains by itself: entries ahead of the stop entry finish first
+    for (;;) {
+      if (headerLoad(q, kQueueState) != kQueueRunning) break;
+      if (q->produced - headerLoad(q, kQueueConsumed) < q->capacity) {
+        memcpy(q->hostEntries + q->produced % q->capacity, &e, sizeof(e));
+        q->produced++;
+        __atomic_store_n(q->header + kQueueProduced, q->produced, __ATOMIC_RELEASE);
+        q->stopSent = true;
+        break;
+      }
+      sched_yield();
+    }
+  }
+  const uint64_t want = q->produced;
+  flagcxResult_t r = joinConsumer(q);
+  if (r != flagcxSuccess) return r;
+  const uint64_t state = headerLoad(q, kQueueState);
+  if (state == kQueueTimedOut || headerLoad(q, kQueueConsumed) < want)
+    return qfail(q, flagcxInternalError,
+                 "flagcxLocalReduceFifoStop: the consumer gave up after its spin limit with %lld of %lld entries done",
+                 (long long)headerLoad(q, kQueueConsumed), (long long)want);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduceFifoDestroy(flagcxLocalReduceFifo_t q) {
+  if (!q) return flagcxSuccess;
+  flagcxResult_t r = flagcxLocalReduceFifoStop(q);
+  hipError_t e = hipStreamDestroy(q->stream);
+  hipError_t e2 = hipFree(q->devBlock);
+  hipError_t e3 = hipHostFree(q->header);
+  delete q;
+  if (e != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return flagcxUnhandledDeviceError;
+  return r;
+}
+
+const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t q) { return q ? q->lastError : ""; }
+
+flagcxResult_t flagcxLocalReduceFifoGetGrid(flagcxLocalReduceFifo_t q, unsigned *workgroups) {
+  if (!q || !workgroups) return flagcxInvalidArgument;
+  *workgroups = q->grid;
+  return flagcxSuccess;
+}
+
+} // extern "C"
+#pragma GCC visibility pop

@@ -41,6 +41,43 @@ ReduceLauncher reduceLauncherFor(int dtype);
 typedef int (*ReduceBatchLauncher)(const ReduceCall *, int);
 ReduceBatchLauncher reduceBatchLauncherFor(int dtype);
 
+// Host-producer / device-consumer reduce queue (reduce_queue_device.h,
+// host_reduce_fifo.cpp).  One entry as the resident consumer kernel reads it.
+struct alignas(128) QueueEntry {
+  uint64_t src[8];  // inputs in fold order
+  uint64_t dst;
+  uint64_t nvec;    // 16-byte vectors in the body
+  uint32_t head;    // elements before the body
+  uint32_t tail;    // elements after it
+  uint32_t k;       // number of inputs, 1..8; 0 = stop
+  uint32_t vector;  // 1: every source shares dst's address modulo 16
+  uint64_t pad[4];
+};
+static_assert(sizeof(QueueEntry) == 128, "queue entries are 16 words");
+
+// Words of the pinned host header, as in the reference's FIFO
+// ([capacity, consumed, produced, ...], flagcx/include/flagcx_kernel.h:75-77),
+// plus a state word.
+enum : int { kQueueCapacity = 0, kQueueConsumed = 1, kQueueProduced = 2, kQueueState = 3, kQueueHeaderWords = 16 };
+enum : uint64_t { kQueueIdle = 0, kQueueRunning = 1, kQueueStopped = 2, kQueueTimedOut = 3 };
+
+struct QueueKernelArgs {
+  uint64_t *hostHeader;          // pinned, device-visible
+  const QueueEntry *hostEntries; // pinned ring, `capacity` entries
+  QueueEntry *devEntries;        // device copy of the ring the workers read
+  uint64_t *devProduced;         // entries forwarded to the device ring; ~0 = abort
+  uint32_t *progress;            // per worker: entries finished (low 32 bits)
+  uint32_t capacity;
+  int64_t maxSpin;
+};
+
+// Launches the consumer for one element type: grid = min(occupancy, wavesPerCU) *
+// numCU one-wave workgroups, all resident.  Returns a hipError_t value.
+typedef int (*ReduceQueueLauncher)(int op, const QueueKernelArgs &, int wavesPerCU, int numCU, int lds,
+                                   unsigned maxGrid, hipStream_t, unsigned *grid);
+ReduceQueueLauncher reduceQueueLauncherFor(int dtype);
+long long asyncMaxSpin(); // async_kernels.hip
+
 // Byte movers (copy_kernels.hip); all return a hipError_t value.
 struct Copy2D {
   void *dst;

@@ -3,6 +3,7 @@
 // so the ten types build in parallel.
 #include "launch.h"
 #include "reduce_device.h"
+#include "reduce_queue_device.h"
 
 #ifndef FLAGCX_DT
 #error "compile with -DFLAGCX_DT=<flagcxDataType_t value>"
@@ -194,6 +195,43 @@ int FLAGCX_CAT(launchReduceBatch_, FLAGCX_DT)(const ReduceCall *calls, int n) {
     case kMax: return launchBatchOp<kMax>(calls, n);
     case kMin: return launchBatchOp<kMin>(calls, n);
     case kAvg: return launchBatchOp<kAvg>(calls, n);
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
+// The resident queue consumer.  Its grid must be resident all at once, so the
+// size comes from the occupancy query for this very kernel and LDS reservation.
+template <int OP>
+static int launchQueueOp(const QueueKernelArgs &q, int wavesPerCU, int numCU, int lds, unsigned maxGrid,
+                         hipStream_t stream, unsigned *grid) {
+  int fit = 0;
+  hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reduceQueueKernel<elem_t, OP>, 64, (size_t)lds);
+  if (e != hipSuccess) return (int)e;
+  if (wavesPerCU > 0 && fit > wavesPerCU) fit = wavesPerCU;
+  // LDS is handed out in 1280-byte granules on gfx950 (160 KiB per CU): count what
+  // really fits, a workgroup that never becomes resident would stall the queue
+  if (lds > 0) {
+    const int granules = (lds + 1279) / 1280;
+    const int byLds = (160 * 1024 / 1280) / granules;
+    if (fit > byLds) fit = byLds;
+  }
+  if (fit < 1) return (int)hipErrorLaunchOutOfResources;
+  uint64_t g = (uint64_t)fit * (uint64_t)numCU;
+  if (g > maxGrid) g = maxGrid;
+  if (g < 2) return (int)hipErrorLaunchOutOfResources;
+  *grid = (unsigned)g;
+  reduceQueueKernel<elem_t, OP><<<dim3((unsigned)g), dim3(64), lds, stream>>>(q);
+  return (int)hipGetLastError();
+}
+
+int FLAGCX_CAT(launchReduceQueue_, FLAGCX_DT)(int op, const QueueKernelArgs &q, int wavesPerCU, int numCU, int lds,
+                                              unsigned maxGrid, hipStream_t stream, unsigned *grid) {
+  switch (op) {
+    case kSum: return launchQueueOp<kSum>(q, wavesPerCU, numCU, lds, maxGrid, stream, grid);
+    case kProd: return launchQueueOp<kProd>(q, wavesPerCU, numCU, lds, maxGrid, stream, grid);
+    case kMax: return launchQueueOp<kMax>(q, wavesPerCU, numCU, lds, maxGrid, stream, grid);
+    case kMin: return launchQueueOp<kMin>(q, wavesPerCU, numCU, lds, maxGrid, stream, grid);
+    case kAvg: return launchQueueOp<kAvg>(q, wavesPerCU, numCU, lds, maxGrid, stream, grid);
     default: return (int)hipErrorInvalidValue;
   }
 }

@@ -1,0 +1,323 @@
+// reduce_queue_device.h - resident consumer of a host-produced queue of reduce
+// descriptors: the host-producer / device-consumer half that the reference
+// declares next to flagcxReduceTrigger and leaves commented out
+// (flagcx/include/flagcx_kernel.h:52-73,96-98).
+//
+// One launch stays on the GPU and folds every descriptor the host appends, so a
+// chunk is reduced when it arrives without a kernel launch per chunk.  The grid
+// is 1 leader + W workers, each a single wavefront, all resident at once:
+//   leader : polls `produced` in the pinned host header, copies new entries into a
+//            device ring, publishes the count the workers poll (device memory, so
+//            only one wavefront reads over PCIe), folds the workers' progress
+//            words into `consumed` in the host header.
+//   worker : for each forwarded entry takes the KiB tiles whose running global
+//            index is congruent to its number modulo W (the numbering runs on
+//            across entries, so entries of a few thousand tiles still spread
+//            evenly), in the same per-tile shape as the launch-per-call kernels.
+//
+// Coherence is per access, not per cache: a kernel that never ends gets no
+// launch-boundary invalidate or write-back, and cache-wide maintenance from
+// thousands of wavefronts costs tens of microseconds per entry.  So every data
+// load carries sc0 sc1 (re-fetched at system scope: inputs may have been written
+// by a copy engine or another stream since this kernel last touched the line),
+// every data store carries sc0 sc1 (written through), queue words are scoped
+// atomics, and "release" is waiting for the wavefront's own stores (s_waitcnt)
+// before the progress word is written.  Only entries whose sources need
+// unaligned global loads (no cache-policy bits there) fall back to a system-scope
+// acquire fence in front of the entry.
+//
+// Every wait is bounded by maxSpin polls: a host that stops producing, or a
+// worker that never becomes resident, ends in kQueueTimedOut, not in a hang
+// (the leader counts polls without new entries or progress and then tells the
+// workers to leave; a worker counts polls during which the leader's heartbeat
+// word did not move).  A stop entry (k = 0) drains the queue: workers exit when
+// they reach it.
+#pragma once
+
+#include "launch.h"
+#include "reduce_device.h"
+
+namespace flagcx_amd {
+
+constexpr int kCoherentLoadAux = kAuxSc0 | kAuxSc1 | kAuxNt;
+constexpr int kCoherentStoreAux = kAuxSc0 | kAuxSc1;
+
+__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ uint64_t agentLoad(const uint64_t *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void agentStore(uint64_t *p, uint64_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t systemLoad(const uint64_t *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void systemStore(uint64_t *p, uint64_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// This wavefront's earlier loads have returned and its earlier stores have been
+// acknowledged (gfx9 counts both in vmcnt); nothing moves across it at compile time.
+__device__ __forceinline__ void waitOwnMemory() {
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __builtin_amdgcn_s_waitcnt(0);
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
+__device__ __forceinline__ uint32_t waveMin32(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t o = __shfl_xor(v, off, 64);
+    v = o < v ? o : v;
+  }
+  return v;
+}
+
+// Word `word` of a value every lane holds for the queue word (lane & 15).
+__device__ __forceinline__ uint64_t laneWord(uint64_t v, int word) {
+  const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)v, word);
+  const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(v >> 32), word);
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// One element read / written at system scope (head and tail elements).
+template <int BYTES> struct UintOf;
+template <> struct UintOf<1> { typedef uint8_t type; };
+template <> struct UintOf<2> { typedef uint16_t type; };
+template <> struct UintOf<4> { typedef uint32_t type; };
+template <> struct UintOf<8> { typedef uint64_t type; };
+
+template <typename T>
+__device__ __forceinline__ T coherentLoad(uint64_t base, uint64_t i) {
+  typedef typename UintOf<sizeof(T)>::type U;
+  const U bits = __hip_atomic_load(reinterpret_cast<const U *>((uintptr_t)base) + i, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_SYSTEM);
+  T out;
+  __builtin_memcpy(&out, &bits, sizeof(T));
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ void coherentStore(uint64_t base, uint64_t i, T v) {
+  typedef typename UintOf<sizeof(T)>::type U;
+  U bits;
+  __builtin_memcpy(&bits, &v, sizeof(T));
+  __hip_atomic_store(reinterpret_cast<U *>((uintptr_t)base) + i, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__device__ inline void queueLeader(const QueueKernelArgs &q) {
+  const uint32_t nworkers = gridDim.x - 1;
+  const uint32_t lane = threadIdx.x;
+  uint64_t forwarded = 0, published = 0, stopAt = ~0ull, beat = 0;
+  int64_t spins = 0;
+  for (;;) {
+    agentStore(q.devProduced + 1, ++beat); // heartbeat: workers count polls only while this stands still
+    if (stopAt == ~0ull) {
+      const uint64_t produced = uniform64(systemLoad(q.hostHeader + kQueueProduced));
+      if (produced > forwarded) {
+        // four entries per round trip over PCIe: lane = 16 * entry + word
+        for (uint64_t base = forwarded; base < produced; base += 4) {
+          const uint64_t i = base + (lane >> 4);
+          const uint32_t word = lane & 15;
+          const bool valid = i < produced;
+          uint64_t w = 1;
+          if (valid) {
+            const uint64_t slot = i % q.capacity;
+            w = systemLoad(reinterpret_cast<const uint64_t *>(q.hostEntries + slot) + word);
+            agentStore(reinterpret_cast<uint64_t *>(q.devEntries + slot) + word, w);
+          }
+          // word 11 = k | vector << 32; k = 0 is the stop entry
+          const uint64_t stopMask = __ballot(valid && word == 11 && (uint32_t)w == 0);
+          uint64_t upto = base + 4 < produced ? base + 4 : produced;
+          if (stopMask) {
+            stopAt = base + ((uint64_t)(__ffsll((long long)stopMask) - 1) >> 4);
+            upto = stopAt + 1; // nothing after a stop entry is published
+          }
+          waitOwnMemory(); // the entries are in the device ring before the count says so
+          agentStore(q.devProduced, upto);
+          forwarded = upto;
+          if (stopMask) break;
+        }
+        spins = 0;
+      }
+    }
+    // min over the workers' 32-bit progress words, relative to what is published
+    const uint32_t base32 = (uint32_t)published;
+    uint32_t ahead = ~0u;
+    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)q.progress, 0, nworkers * 4u, kRsrcFlags);
+    for (uint32_t v0 = 0; v0 < nworkers; v0 += 1024) {
+      u32x4 p[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        p[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, (v0 + u * 256 + lane * 4) * 4u, 0, kAuxSc0 | kAuxSc1);
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const uint32_t d = p[u][c] - base32;
+          if (v0 + u * 256 + lane * 4 + c < nworkers && d < ahead) ahead = d;
+        }
+    }
+    ahead = __builtin_amdgcn_readfirstlane(waveMin32(ahead));
+    if (ahead != 0 && ahead != ~0u) {
+      // a worker writes its progress word only after its results were acknowledged
+      // by memory, so the count can go to the host as soon as it has been read
+      waitOwnMemory();
+      published += ahead;
+      systemStore(q.hostHeader + kQueueConsumed, published);
+      spins = 0;
+    }
+    if (stopAt != ~0ull && published > stopAt) {
+      waitOwnMemory();
+      systemStore(q.hostHeader + kQueueState, kQueueStopped);
+      return;
+    }
+    if (++spins > q.maxSpin) {
+      agentStore(q.devProduced, ~0ull); // workers leave at their next poll
+      systemStore(q.hostHeader + kQueueState, kQueueTimedOut);
+      return;
+    }
+    __builtin_amdgcn_s_sleep(8);
+  }
+}
+
+// This worker's KiB tiles of one entry, K inputs known at compile time.  ALIGNED:
+// every pointer agrees modulo 16 and tiles go through clipped buffer descriptors;
+// otherwise the destination's tiling with unaligned 16-byte loads.
+template <typename T, int OP, int K, bool ALIGNED>
+__device__ __forceinline__ void queueTiles(const uint64_t (&src)[8], uint64_t dst, uint64_t headBytes,
+                                           uint64_t bodyBytes, uint64_t first, uint64_t stride) {
+  const uint32_t voff = threadIdx.x * 16u;
+  const uint64_t ntiles = (bodyBytes + 1023) / 1024;
+  for (uint64_t t = first; t < ntiles; t += stride) {
+    const uint64_t off = headBytes + t * 1024;
+    const uint64_t left = bodyBytes - t * 1024;
+    const uint32_t span = left < 1024 ? (uint32_t)left : 1024u;
+    u32x4 in[K];
+    if (ALIGNED) {
+#pragma unroll
+      for (int j = 0; j < K; j++) {
+        __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)(src[j] + off), 0, span, kRsrcFlags);
+        in[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kCoherentLoadAux);
+      }
+      __amdgpu_buffer_rsrc_t rd =
+          __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)(dst + off), 0, span, kRsrcFlags);
+      __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, voff, 0, kCoherentStoreAux);
+    } else if (voff < span) {
+#pragma unroll
+      for (int j = 0; j < K; j++)
+        in[j] = __builtin_nontemporal_load((const u32x4_unaligned *)(uintptr_t)(src[j] + off + voff));
+      __amdgpu_buffer_rsrc_t rd =
+          __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)(dst + off), 0, span, kRsrcFlags);
+      __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, voff, 0, kCoherentStoreAux);
+    }
+  }
+}
+
+template <typename T, int OP, int K>
+__device__ __forceinline__ void queueEntry(const uint64_t (&src)[8], uint64_t dst, uint32_t head, uint32_t tail,
+                                           uint64_t nvec, bool aligned, uint64_t first, uint64_t stride) {
+  constexpr int N = 16 / sizeof(T);
+  const uint64_t headBytes = (uint64_t)head * sizeof(T);
+  if (aligned) {
+    queueTiles<T, OP, K, true>(src, dst, headBytes, nvec * 16, first, stride);
+  } else {
+    // plain global loads carry no scope bits: drop whatever this CU and L2 hold
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
+    queueTiles<T, OP, K, false>(src, dst, headBytes, nvec * 16, first, stride);
+  }
+  // head and tail elements: the worker that owns tile 0, one lane each
+  if (first == 0 && threadIdx.x < head + tail) {
+    const uint64_t i = threadIdx.x < head ? threadIdx.x : head + nvec * N + (threadIdx.x - head);
+    typedef Fold<T, OP> F;
+    typename F::acc_t acc = F::init(coherentLoad<T>(src[0], i));
+#pragma unroll
+    for (int j = 1; j < K; j++) acc = F::step(coherentLoad<T>(src[j], i), acc);
+    coherentStore<T>(dst, i, F::fin(acc, K));
+  }
+}
+
+template <typename T, int OP>
+__device__ inline void queueWorker(const QueueKernelArgs &q) {
+  const uint32_t nworkers = gridDim.x - 1;
+  const uint32_t worker = blockIdx.x - 1;
+  uint64_t done = 0; // entries this worker has finished
+  uint64_t lastBeat = 0;
+  uint32_t rot = 0;  // tiles handed out so far, modulo nworkers
+  for (;;) {
+    uint64_t produced;
+    int64_t spins = 0;
+    for (;;) {
+      produced = uniform64(agentLoad(q.devProduced));
+      if (produced > done) break; // the abort value ~0 ends the wait too
+      // an idle queue is the leader's to time out; a worker only gives up by
+      // itself when the leader's heartbeat has stopped for maxSpin polls
+      const uint64_t beat = uniform64(agentLoad(q.devProduced + 1));
+      if (beat != lastBeat) {
+        lastBeat = beat;
+        spins = 0;
+      }
+      if (++spins > q.maxSpin) return;
+      __builtin_amdgcn_s_sleep(4);
+    }
+    if (produced == ~0ull) return;
+    bool stop = false;
+    // lane l holds word l & 15 of the entry; the next entry is fetched while this
+    // one's tiles are in flight
+    uint64_t words =
+        agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + done % q.capacity) + (threadIdx.x & 15));
+    while (done < produced) {
+      const uint64_t cur = words;
+      if (done + 1 < produced)
+        words = agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (done + 1) % q.capacity) +
+                          (threadIdx.x & 15));
+      const uint64_t kv = laneWord(cur, 11);
+      const int k = (int)(uint32_t)kv;
+      done++;
+      if (k == 0) {
+        stop = true;
+        break;
+      }
+      const bool vector = (kv >> 32) != 0;
+      uint64_t src[8];
+#pragma unroll
+      for (int b = 0; b < 8; b++) src[b] = laneWord(cur, b);
+      const uint64_t dst = laneWord(cur, 8);
+      const uint64_t nvec = laneWord(cur, 9);
+      const uint64_t ht = laneWord(cur, 10);
+      const uint32_t head = (uint32_t)ht, tail = (uint32_t)(ht >> 32);
+      const uint64_t ntiles = (nvec * 16 + 1023) / 1024;
+      const uint32_t first = worker >= rot ? worker - rot : worker + nworkers - rot;
+      switch (k) {
+        case 1: queueEntry<T, OP, 1>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+        case 2: queueEntry<T, OP, 2>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+        case 3: queueEntry<T, OP, 3>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+        case 4: queueEntry<T, OP, 4>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+        case 5: queueEntry<T, OP, 5>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+        case 6: queueEntry<T, OP, 6>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+        case 7: queueEntry<T, OP, 7>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+        default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nworkers); break;
+      }
+      rot = (uint32_t)((rot + ntiles) % nworkers);
+    }
+    // this wavefront's results are acknowledged by memory before the count says so
+    waitOwnMemory();
+    if (threadIdx.x == 0)
+      __hip_atomic_store(q.progress + worker, (uint32_t)done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (stop) return;
+  }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(64) reduceQueueKernel(QueueKernelArgs q) {
+  if (blockIdx.x == 0)
+    queueLeader(q);
+  else
+    queueWorker<T, OP>(q);
+}
+
+} // namespace flagcx_amd

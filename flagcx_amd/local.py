@@ -126,6 +126,10 @@ EXPORTS = [
     "flagcxLocalGetDeviceAdaptor", "flagcxLocalDeviceAdaptorLayout",
     "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
     "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
+    "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
+    "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
+    "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
+    "flagcxLocalReduceFifoGetLastError",
 ]
 
 
@@ -188,6 +192,18 @@ def lib():
         L.flagcxLocalPlanExecute.argtypes = [vp, pp, pp, pp, i, i, sp]
         L.flagcxLocalPlanGetLastError.restype = C.c_char_p
         L.flagcxLocalPlanGetLastError.argtypes = [vp]
+        u64p = C.POINTER(C.c_uint64)
+        L.flagcxLocalReduceFifoCreate.argtypes = [C.POINTER(vp), i, i, i, i]
+        L.flagcxLocalReduceFifoDestroy.argtypes = [vp]
+        L.flagcxLocalReduceFifoStart.argtypes = [vp]
+        L.flagcxLocalReduceFifoStop.argtypes = [vp]
+        L.flagcxLocalReduceFifoEnqueue.argtypes = [vp, C.POINTER(ReduceTrigger), u64p]
+        L.flagcxLocalReduceFifoEnqueueReduce.argtypes = [vp, pp, i, vp, sz, u64p]
+        L.flagcxLocalReduceFifoQuery.argtypes = [vp, u64p, u64p, C.POINTER(i)]
+        L.flagcxLocalReduceFifoWait.argtypes = [vp, C.c_uint64]
+        L.flagcxLocalReduceFifoGetGrid.argtypes = [vp, C.POINTER(C.c_uint)]
+        L.flagcxLocalReduceFifoGetLastError.restype = C.c_char_p
+        L.flagcxLocalReduceFifoGetLastError.argtypes = [vp]
         L.flagcxLocalSetMaxSpinCount.restype = None
         L.flagcxLocalSetMaxSpinCount.argtypes = [C.c_int64]
         for name in ("deviceAsyncStore", "deviceAsyncLoad"):
@@ -397,6 +413,91 @@ class Ring:
         if self._h:
             lib().flagcxLocalRingDestroy(self._h)
             self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class ReduceFifo:
+    """Host-producer / device-consumer reduce queue (flagcxLocalReduceFifo*).
+
+    While it runs, do not synchronise the whole device (torch.cuda.synchronize, freeing
+    tensors): that returns only after stop().  Use it as a context manager so that an
+    exception between start and stop still stops the resident kernel.
+    """
+
+    def __init__(self, capacity, max_ranks, dtype, op):
+        self._h = C.c_void_p()
+        rc = lib().flagcxLocalReduceFifoCreate(C.byref(self._h), capacity, max_ranks, int(dtype), int(op))
+        if rc:
+            raise FlagcxError(rc, "flagcxLocalReduceFifoCreate")
+
+    def _check(self, rc):
+        if rc:
+            raise FlagcxError(rc, (lib().flagcxLocalReduceFifoGetLastError(self._h) or b"").decode())
+
+    def start(self):
+        self._check(lib().flagcxLocalReduceFifoStart(self._h))
+        return self
+
+    def stop(self):
+        self._check(lib().flagcxLocalReduceFifoStop(self._h))
+
+    def try_enqueue_reduce(self, src_ptrs, dst_ptr, count):
+        """Ticket, or None when the ring is full."""
+        t = C.c_uint64()
+        rc = lib().flagcxLocalReduceFifoEnqueueReduce(self._h, _ptr_array(src_ptrs), len(src_ptrs), dst_ptr, count,
+                                                      C.byref(t))
+        if rc == Result.InProgress:
+            return None
+        self._check(rc)
+        return t.value
+
+    def enqueue_reduce(self, src_ptrs, dst_ptr, count):
+        while True:
+            t = self.try_enqueue_reduce(src_ptrs, dst_ptr, count)
+            if t is not None:
+                return t
+
+    def enqueue(self, trigger):
+        t = C.c_uint64()
+        while True:
+            rc = lib().flagcxLocalReduceFifoEnqueue(self._h, C.byref(trigger), C.byref(t))
+            if rc != Result.InProgress:
+                break
+        self._check(rc)
+        return t.value
+
+    def query(self):
+        """(produced, consumed, state)"""
+        p, c, st = C.c_uint64(), C.c_uint64(), C.c_int()
+        self._check(lib().flagcxLocalReduceFifoQuery(self._h, C.byref(p), C.byref(c), C.byref(st)))
+        return p.value, c.value, st.value
+
+    def wait(self, ticket):
+        self._check(lib().flagcxLocalReduceFifoWait(self._h, ticket))
+
+    def grid(self):
+        g = C.c_uint()
+        self._check(lib().flagcxLocalReduceFifoGetGrid(self._h, C.byref(g)))
+        return g.value
+
+    def close(self):
+        if self._h:
+            lib().flagcxLocalReduceFifoDestroy(self._h)
+            self._h = C.c_void_p()
+
+    def __enter__(self):
+        return self.start()
+
+    def __exit__(self, *exc):
+        try:
+            lib().flagcxLocalReduceFifoStop(self._h)
+        finally:
+            return False
 
     def __del__(self):
         try:

@@ -1,0 +1,169 @@
+// fifo_perf.cpp - C++ timing driver for the host-producer / device-consumer reduce
+// queue (flagcxLocalReduceFifo*), beside the launch-per-chunk and batched forms of
+// the same work:
+//
+//   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
+//
+// A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
+// staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
+// chunk.  Times are host wall clock from the first enqueue (or launch) to the
+// moment the last chunk is known to be done; GB/s = (k+1)*bytes/time.
+// Also: latency of ONE small entry, enqueue -> Wait, against launch -> stream sync.
+#include "../../include/flagcx_amd.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#define CK(x)                                                                  \
+  do {                                                                         \
+    hipError_t e_ = (x);                                                       \
+    if (e_ != hipSuccess) {                                                    \
+      fprintf(stderr, "HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+      return 1;                                                                \
+    }                                                                          \
+  } while (0)
+#define FX(x)                                                                  \
+  do {                                                                         \
+    flagcxResult_t r_ = (x);                                                   \
+    if (r_ != flagcxSuccess) {                                                 \
+      fprintf(stderr, "flagcx error %d at %s:%d: %s | %s\n", (int)r_, __FILE__, __LINE__, flagcxLocalGetLastError(), \
+              fifo ? flagcxLocalReduceFifoGetLastError(fifo) : "");            \
+      if (fifo) flagcxLocalReduceFifoDestroy(fifo);                            \
+      return 1;                                                                \
+    }                                                                          \
+  } while (0)
+
+struct flagcxStream {
+  hipStream_t base;
+};
+
+static double nowUs() {
+  return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+static double median(std::vector<double> v) {
+  std::sort(v.begin(), v.end());
+  return v[v.size() / 2];
+}
+
+int main(int argc, char **argv) {
+  int k = 8, dtype = flagcxHalf, op = flagcxAvg, nchunks = 32, warmup = 5, iters = 20;
+  size_t chunkBytes = FLAGCX_LOCAL_CHUNKSIZE;
+  long long spin = 1ll << 22;
+  for (int i = 1; i + 1 < argc; i += 2) {
+    const char *f = argv[i], *v = argv[i + 1];
+    if (!strcmp(f, "-k")) k = atoi(v);
+    else if (!strcmp(f, "-t")) dtype = atoi(v);
+    else if (!strcmp(f, "-o")) op = atoi(v);
+    else if (!strcmp(f, "-c")) chunkBytes = strtoull(v, 0, 0);
+    else if (!strcmp(f, "-m")) nchunks = atoi(v);
+    else if (!strcmp(f, "-w")) warmup = atoi(v);
+    else if (!strcmp(f, "-n")) iters = atoi(v);
+    else if (!strcmp(f, "-s")) spin = atoll(v);
+  }
+  flagcxLocalReduceFifo_t fifo = nullptr;
+  const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
+  if (!ts || k < 1 || k > 8 || nchunks < 1 || chunkBytes % ts) return 2;
+  FX(flagcxLocalInit());
+  flagcxLocalSetMaxSpinCount(spin); // an idle consumer leaves after this many polls
+  const size_t shardBytes = chunkBytes * (size_t)nchunks;
+  const size_t chunkCount = chunkBytes / ts;
+  std::vector<void *> src(k);
+  void *dst = nullptr;
+  for (int j = 0; j < k; j++) {
+    CK(hipMalloc(&src[j], shardBytes));
+    CK(hipMemset(src[j], 0, shardBytes)); // zeros are valid in every type; timing does not depend on values
+  }
+  CK(hipMalloc(&dst, shardBytes));
+  flagcxStream st;
+  CK(hipStreamCreateWithFlags(&st.base, hipStreamNonBlocking));
+  CK(hipDeviceSynchronize());
+  const double algo = (k + 1.0) * (double)shardBytes;
+  printf("# k=%d dtype=%d op=%d chunk=%zu B x %d chunks (%.0f MiB per input), warmup=%d iters=%d\n", k, dtype, op,
+         chunkBytes, nchunks, shardBytes / 1048576.0, warmup, iters);
+
+  std::vector<std::vector<const void *>> chunkSrc(nchunks, std::vector<const void *>(k));
+  std::vector<flagcxLocalReduceDesc> descs(nchunks);
+  for (int c = 0; c < nchunks; c++) {
+    for (int j = 0; j < k; j++) chunkSrc[c][j] = (const char *)src[j] + (size_t)c * chunkBytes;
+    descs[c].sendbuffs = chunkSrc[c].data();
+    descs[c].recvbuff = (char *)dst + (size_t)c * chunkBytes;
+    descs[c].count = chunkCount;
+  }
+
+  // (1) one launch per chunk
+  std::vector<double> t;
+  for (int it = 0; it < warmup + iters; it++) {
+    const double t0 = nowUs();
+    for (int c = 0; c < nchunks; c++)
+      FX(flagcxLocalReduce(chunkSrc[c].data(), k, descs[c].recvbuff, chunkCount, (flagcxDataType_t)dtype,
+                           (flagcxRedOp_t)op, &st));
+    CK(hipStreamSynchronize(st.base));
+    if (it >= warmup) t.push_back(nowUs() - t0);
+  }
+  printf("%-46s %10.1f us  %8.1f GB/s\n", "one launch per chunk, then stream sync", median(t), algo / median(t) / 1e3);
+
+  // (2) all chunks known up front: one batch call
+  t.clear();
+  for (int it = 0; it < warmup + iters; it++) {
+    const double t0 = nowUs();
+    FX(flagcxLocalReduceBatch(descs.data(), nchunks, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op, &st));
+    CK(hipStreamSynchronize(st.base));
+    if (it >= warmup) t.push_back(nowUs() - t0);
+  }
+  printf("%-46s %10.1f us  %8.1f GB/s\n", "one batch call (all chunks present), sync", median(t), algo / median(t) / 1e3);
+
+  // (3) the resident consumer: enqueue chunk by chunk, wait for the last ticket
+  FX(flagcxLocalReduceFifoCreate(&fifo, 64, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op));
+  FX(flagcxLocalReduceFifoStart(fifo));
+  unsigned grid = 0;
+  FX(flagcxLocalReduceFifoGetGrid(fifo, &grid));
+  t.clear();
+  for (int it = 0; it < warmup + iters; it++) {
+    const double t0 = nowUs();
+    uint64_t ticket = 0;
+    for (int c = 0; c < nchunks; c++) {
+      flagcxResult_t r;
+      while ((r = flagcxLocalReduceFifoEnqueueReduce(fifo, chunkSrc[c].data(), k, descs[c].recvbuff, chunkCount,
+                                                     &ticket)) == flagcxInProgress) {
+      }
+      FX(r);
+    }
+    FX(flagcxLocalReduceFifoWait(fifo, ticket));
+    if (it >= warmup) t.push_back(nowUs() - t0);
+  }
+  printf("%-46s %10.1f us  %8.1f GB/s  (%u resident wavefronts)\n", "resident consumer, enqueue per chunk, Wait",
+         median(t), algo / median(t) / 1e3, grid);
+
+  // (4) latency of one small entry (4 KiB per input)
+  const size_t smallCount = 4096 / ts;
+  t.clear();
+  for (int it = 0; it < 200; it++) {
+    uint64_t ticket = 0;
+    const double t0 = nowUs();
+    FX(flagcxLocalReduceFifoEnqueueReduce(fifo, chunkSrc[0].data(), k, dst, smallCount, &ticket));
+    FX(flagcxLocalReduceFifoWait(fifo, ticket));
+    t.push_back(nowUs() - t0);
+  }
+  const double fifoLat = median(t);
+  FX(flagcxLocalReduceFifoStop(fifo));
+  t.clear();
+  for (int it = 0; it < 200; it++) {
+    const double t0 = nowUs();
+    FX(flagcxLocalReduce(chunkSrc[0].data(), k, dst, smallCount, (flagcxDataType_t)dtype, (flagcxRedOp_t)op, &st));
+    CK(hipStreamSynchronize(st.base));
+    t.push_back(nowUs() - t0);
+  }
+  printf("4 KiB entry: enqueue -> Wait %.2f us; launch -> stream sync %.2f us\n", fifoLat, median(t));
+  FX(flagcxLocalReduceFifoDestroy(fifo));
+  fifo = nullptr;
+  for (int j = 0; j < k; j++) CK(hipFree(src[j]));
+  CK(hipFree(dst));
+  return 0;
+}

@@ -344,6 +344,68 @@ flagcxResult_t flagcxLocalP2pDemo(const void *sendbuff, void *recvbuff, size_t c
                                   void *fifoBuffer, flagcxStream_t stream);
 
 /* ------------------------------------------------------------------------- */
+/* Host-producer / device-consumer reduce queue                                */
+/* ------------------------------------------------------------------------- */
+/* The other direction of the kernel FIFO, which the reference declares for
+ * flagcxReduceTrigger and leaves commented out
+ * (`enqueue(flagcxReduceTrigger)` on the host, `dequeue` on the device,
+ * flagcx/include/flagcx_kernel.h:96-98): the host appends reduce descriptors to a
+ * pinned ring [capacity, consumed, produced, ...] and ONE resident kernel folds
+ * them as they arrive, so a 4 MiB chunk costs no kernel launch.  The queue owns a
+ * non-blocking stream for that kernel, as the kernel proxy owns its stream
+ * (flagcx/core/proxy.cc:1094-1097).
+ *
+ * A queue is created for one element type and one op; entries carry 1..maxRanks
+ * (at most 8) inputs.  Entries run in order; entries in flight together must not
+ * depend on one another unless the producer waits for the earlier ticket first.
+ * The producer appends an entry only when its inputs are complete in device
+ * memory (an event or stream it has synchronised with), and reads results after
+ * Wait(ticket) or Stop.  Create / Start / Stop / Destroy allocate or synchronise
+ * (setup time); Enqueue, Query and Wait touch pinned host memory only.
+ *
+ * While the consumer is resident it holds a share of every CU: launches that
+ * reserve LDS (this library's 2..8-input reductions) queue behind it until Stop,
+ * and anything that synchronises the whole device (hipDeviceSynchronize, hipFree)
+ * returns only after Stop or after the consumer's idle limit.  The consumer gives
+ * up, state 3, after FLAGCX_FUNC_MAX_SPIN_COUNT polls without new entries or
+ * progress (flagcxLocalSetMaxSpinCount; default 2^27, minutes). */
+typedef struct flagcxLocalReduceFifo *flagcxLocalReduceFifo_t;
+#define FLAGCX_LOCAL_REDUCE_FIFO_IDLE 0
+#define FLAGCX_LOCAL_REDUCE_FIFO_RUNNING 1
+#define FLAGCX_LOCAL_REDUCE_FIFO_STOPPED 2
+#define FLAGCX_LOCAL_REDUCE_FIFO_TIMED_OUT 3
+
+flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int capacity, int maxRanks,
+                                           flagcxDataType_t datatype, flagcxRedOp_t op);
+/* Stop (if running), then free everything. */
+flagcxResult_t flagcxLocalReduceFifoDestroy(flagcxLocalReduceFifo_t fifo);
+/* Launches the consumer; counters restart at zero.  A stopped or timed-out queue
+ * can be started again. */
+flagcxResult_t flagcxLocalReduceFifoStart(flagcxLocalReduceFifo_t fifo);
+/* Appends a stop entry behind everything enqueued so far and waits until the
+ * consumer has finished those entries and left the GPU. */
+flagcxResult_t flagcxLocalReduceFifoStop(flagcxLocalReduceFifo_t fifo);
+/* Host `enqueue(flagcxReduceTrigger)`: addr3 = OP(addr1, addr2) over `count`
+ * elements, as flagcxLocalReduceTriggers; the trigger's datatype and redop must be
+ * the queue's.  *ticket (may be NULL) is the value `consumed` reaches when this
+ * entry is done.  flagcxInProgress: the ring is full, try again. */
+flagcxResult_t flagcxLocalReduceFifoEnqueue(flagcxLocalReduceFifo_t fifo, const flagcxLocalReduceTrigger *trigger,
+                                            uint64_t *ticket);
+/* The N-way form: recvbuff = fold of sendbuffs[0..nranks) in array order, as
+ * flagcxLocalReduce, nranks <= maxRanks. */
+flagcxResult_t flagcxLocalReduceFifoEnqueueReduce(flagcxLocalReduceFifo_t fifo, const void *const *sendbuffs,
+                                                  int nranks, void *recvbuff, size_t count, uint64_t *ticket);
+/* Counters and state (any pointer may be NULL); never blocks. */
+flagcxResult_t flagcxLocalReduceFifoQuery(flagcxLocalReduceFifo_t fifo, uint64_t *produced, uint64_t *consumed,
+                                          int *state);
+/* Spins on the host until consumed >= ticket.  flagcxInvalidArgument if the ticket
+ * has not been handed out; an error if the consumer exits first. */
+flagcxResult_t flagcxLocalReduceFifoWait(flagcxLocalReduceFifo_t fifo, uint64_t ticket);
+/* Workgroups (one wavefront each) of the running consumer: 1 leader + workers. */
+flagcxResult_t flagcxLocalReduceFifoGetGrid(flagcxLocalReduceFifo_t fifo, unsigned *workgroups);
+const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t fifo);
+
+/* ------------------------------------------------------------------------- */
 /* Staging ring (the pipeline either side of the reduce)                       */
 /* ------------------------------------------------------------------------- */
 /* The 16 x 4 MiB staging ring of the reference's proxies

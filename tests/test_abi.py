@@ -151,6 +151,25 @@ def test_batch_and_trigger_entry_points_validate():
     assert C.sizeof(local.ReduceTrigger) == 32
 
 
+def test_reduce_fifo_entry_points_validate_without_a_device():
+    L = local.lib()
+    inv = int(local.Result.InvalidArgument)
+    h = C.c_void_p()
+    assert L.flagcxLocalReduceFifoCreate(None, 16, 8, 7, 0) == inv
+    assert L.flagcxLocalReduceFifoCreate(C.byref(h), 16, 8, 10, 0) == inv      # dtype
+    assert L.flagcxLocalReduceFifoCreate(C.byref(h), 16, 8, 7, 5) == inv       # op
+    assert L.flagcxLocalReduceFifoCreate(C.byref(h), 0, 8, 7, 0) == inv        # capacity
+    assert L.flagcxLocalReduceFifoCreate(C.byref(h), 16, 9, 7, 0) == inv       # more than 8 inputs
+    assert not h.value
+    assert L.flagcxLocalReduceFifoStart(None) == inv
+    assert L.flagcxLocalReduceFifoEnqueue(None, None, None) == inv
+    assert L.flagcxLocalReduceFifoEnqueueReduce(None, None, 2, None, 1, None) == inv
+    assert L.flagcxLocalReduceFifoQuery(None, None, None, None) == inv
+    assert L.flagcxLocalReduceFifoWait(None, 1) == inv
+    assert L.flagcxLocalReduceFifoStop(None) == inv
+    assert L.flagcxLocalReduceFifoDestroy(None) == 0
+
+
 def test_error_strings():
     L = local.lib()
     for code in range(0, 11):

@@ -1,0 +1,275 @@
+"""GPU tests of the host-producer / device-consumer reduce queue (flagcxLocalReduceFifo*),
+through the C ABI, against the CPU oracle.  Same bar as the launch-per-call reduce:
+bit equality with the oracle; where an arithmetic result is NaN any payload passes.
+
+Every test bounds the consumer's idle limit first, so a mistake ends in a timed-out
+queue and a failed assertion, not in a resident kernel that waits for minutes.
+"""
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from tests.util import DT_NAME, OP_NAME, dev_empty, from_dev, is_float, make_inputs, same, to_dev
+
+pytestmark = pytest.mark.gpu
+
+RUNNING, STOPPED, TIMED_OUT = 1, 2, 3
+
+
+@pytest.fixture(scope="module")
+def L():
+    import torch
+    assert torch.cuda.is_available()
+    from flagcx_amd import local
+    assert local.lib().flagcxLocalInit() == 0
+    local.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+    yield local
+    local.lib().flagcxLocalSetMaxSpinCount(-1)
+
+
+def nan_ok(dtype, op):
+    return is_float(dtype) and op in (O.SUM, O.PROD, O.AVG)
+
+
+def expect(srcs, dt, op):
+    rc, want = O.reduce([np.ascontiguousarray(s) for s in srcs], dt, op)
+    assert rc == 0
+    return want
+
+
+CASES = [
+    (O.BF16, O.SUM, 8), (O.FP16, O.AVG, 8), (O.FP32, O.SUM, 2), (O.INT32, O.MAX, 4), (O.INT32, O.MIN, 4),
+    (O.FP64, O.PROD, 3), (O.INT8, O.MIN, 5), (O.UINT8, O.SUM, 7), (O.INT64, O.SUM, 6), (O.BF16, O.MAX, 8),
+    (O.FP16, O.MIN, 2), (O.UINT64, O.MAX, 1), (O.FP32, O.AVG, 3), (O.UINT32, O.PROD, 2),
+]
+
+
+@pytest.mark.parametrize("dt,op,k", CASES, ids=lambda v: str(v))
+def test_fifo_reduce_matches_oracle(L, dt, op, k):
+    """Several entries of different, ragged sizes in one run of the consumer."""
+    import torch
+    counts = [1, 7, 1023, 4097, (1 << 18) + 3, 64 * 1024]
+    ins = [make_inputs(dt, k, n, seed=100 + i, op=op) for i, n in enumerate(counts)]
+    devs = [[to_dev(a) for a in group] for group in ins]
+    outs = [dev_empty(n, ins[0][0].dtype.itemsize, fill=0x55) for n in counts]
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(16, k, dt, op)
+    try:
+        with q:
+            assert q.grid() >= 2
+            tickets = [q.enqueue_reduce([d.data_ptr() for d in devs[i]], outs[i].data_ptr(), counts[i])
+                       for i in range(len(counts))]
+            assert tickets == list(range(1, len(counts) + 1))
+            q.wait(tickets[-1])
+            assert q.query()[:2] == (len(counts), len(counts))
+        assert q.query()[2] == STOPPED
+    finally:
+        q.close()
+    for i, n in enumerate(counts):
+        got = from_dev(outs[i], ins[i][0].dtype)
+        assert same(got, expect(ins[i], dt, op), nan_class=nan_ok(dt, op), dtype=dt), (DT_NAME[dt], OP_NAME[op], n)
+
+
+@pytest.mark.parametrize("dt,op,k", [(O.BF16, O.SUM, 8), (O.FP32, O.SUM, 3), (O.INT8, O.MAX, 4), (O.FP64, O.MIN, 2)],
+                         ids=lambda v: str(v))
+def test_fifo_misaligned_and_in_place(L, dt, op, k):
+    """Element-aligned pointers: a shared offset (head/tail peel), sources at other
+    offsets modulo 16 (unaligned loads), and recvbuff == sendbuffs[0]."""
+    import torch
+    n = 50_000
+    isz = np.dtype(O.NP_OF[dt]).itemsize
+    pad = 16 // isz
+    ins = make_inputs(dt, k, n + 2 * pad, seed=7, op=op)
+    devs = [to_dev(a) for a in ins]
+    out_a = dev_empty(n + 2 * pad, isz, fill=0)
+    out_b = dev_empty(n + 2 * pad, isz, fill=0)
+    torch.cuda.synchronize()
+    # a: every pointer shifted by one element; b: source j shifted by j % pad elements, dst by 1
+    offs_b = [(j + 2) % pad if pad > 1 else 0 for j in range(k)]
+    inplace = devs[0].clone()
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(8, k, dt, op)
+    try:
+        with q:
+            q.enqueue_reduce([d.data_ptr() + isz for d in devs], out_a.data_ptr() + isz, n)
+            q.enqueue_reduce([d.data_ptr() + offs_b[j] * isz for j, d in enumerate(devs)], out_b.data_ptr() + isz, n)
+            q.enqueue_reduce([inplace.data_ptr()] + [d.data_ptr() for d in devs[1:]], inplace.data_ptr(), n)
+    finally:
+        q.close()
+    npdt = ins[0].dtype
+    got_a = from_dev(out_a, npdt)
+    assert same(got_a[1:n + 1], expect([a[1:n + 1] for a in ins], dt, op), nan_class=nan_ok(dt, op), dtype=dt)
+    assert not got_a[0].tobytes().strip(b"\0") and not got_a[n + 1:].tobytes().strip(b"\0")  # guards untouched
+    got_b = from_dev(out_b, npdt)
+    want_b = expect([a[offs_b[j]:offs_b[j] + n] for j, a in enumerate(ins)], dt, op)
+    assert same(got_b[1:n + 1], want_b, nan_class=nan_ok(dt, op), dtype=dt)
+    assert not got_b[0].tobytes().strip(b"\0") and not got_b[n + 1:].tobytes().strip(b"\0")
+    got_c = from_dev(inplace, npdt)
+    assert same(got_c[:n], expect([a[:n] for a in ins], dt, op), nan_class=nan_ok(dt, op), dtype=dt)
+    assert same(got_c[n:], ins[0][n:])
+
+
+def test_fifo_triggers_chain(L):
+    """Binary triggers in the reference's 256-bit layout: addr3 = OP(addr1, addr2).
+    A k-way sum as a chain through one accumulator, each link waiting for the last."""
+    import torch
+    dt, op, k, n = O.FP32, O.SUM, 5, 300_001
+    ins = make_inputs(dt, k, n, seed=11)
+    devs = [to_dev(a) for a in ins]
+    acc = dev_empty(n, 4, fill=0)
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(4, 2, dt, op)
+    try:
+        with q:
+            # acc = in1 + in0, then acc = in_j + acc
+            t = q.enqueue(L.ReduceTrigger.make(devs[1].data_ptr(), devs[0].data_ptr(), acc.data_ptr(), n, dt, op))
+            for j in range(2, k):
+                q.wait(t)
+                t = q.enqueue(L.ReduceTrigger.make(devs[j].data_ptr(), acc.data_ptr(), acc.data_ptr(), n, dt, op))
+            q.wait(t)
+            # results are visible to a host copy while the consumer is still resident
+            got_live = from_dev(acc, np.float32)
+            bad = L.ReduceTrigger.make(devs[0].data_ptr(), devs[1].data_ptr(), acc.data_ptr(), n, O.FP64, op)
+            with pytest.raises(L.FlagcxError):
+                q.enqueue(bad)
+    finally:
+        q.close()
+    want = expect(ins, dt, op)
+    assert same(got_live, want, nan_class=True, dtype=dt)
+    assert same(from_dev(acc, np.float32), want, nan_class=True, dtype=dt)
+
+
+def test_fifo_sees_inputs_rewritten_while_resident(L):
+    """The same small buffers (they would stay in cache) are rewritten between entries,
+    by a host-to-device copy and by a copy kernel on another stream, while the consumer
+    stays resident: every entry must fold the new contents, and its result must be
+    what a host copy and another stream's kernel read afterwards."""
+    import torch
+    dt, op, k, n = O.INT32, O.SUM, 4, 16 * 1024
+    rounds = 12
+    rng = np.random.default_rng(3)
+    host = [[rng.integers(-2**31, 2**31 - 1, n, dtype=np.int32) for _ in range(k)] for _ in range(rounds)]
+    staged = [[torch.from_numpy(a).cuda() for a in group] for group in host]   # sources of the copy kernel
+    pinned = [[torch.from_numpy(a).pin_memory() for a in group] for group in host]
+    devs = [torch.zeros(n, dtype=torch.int32, device="cuda") for _ in range(k)]
+    out = torch.zeros(n, dtype=torch.int32, device="cuda")
+    echo = torch.zeros(n, dtype=torch.int32, device="cuda")
+    side = torch.cuda.Stream()
+    side_ref = L.Stream(side.cuda_stream)
+    torch.cuda.synchronize()
+    got_host, got_echo = [], []
+    q = L.ReduceFifo(8, k, dt, op)
+    try:
+        with q:
+            for r in range(rounds):
+                for j in range(k):
+                    if r % 2 == 0:
+                        with torch.cuda.stream(side):
+                            devs[j].copy_(pinned[r][j], non_blocking=True)      # copy engine
+                    else:
+                        L.memcpy(devs[j].data_ptr(), staged[r][j].data_ptr(), n * 4, stream=side_ref)  # kernel
+                side.synchronize()
+                q.wait(q.enqueue_reduce([d.data_ptr() for d in devs], out.data_ptr(), n))
+                L.memcpy(echo.data_ptr(), out.data_ptr(), n * 4, stream=side_ref)
+                side.synchronize()
+                got_echo.append(echo.cpu().numpy().copy())
+                got_host.append(out.cpu().numpy().copy())
+    finally:
+        q.close()
+    for r in range(rounds):
+        want = expect(host[r], dt, op)
+        assert same(got_host[r], want), r
+        assert same(got_echo[r], want), r
+
+
+def test_fifo_ring_wraps_and_restarts(L):
+    """More entries than slots (the producer sees 'full' and retries), then a second
+    start on the same queue with counters back at zero."""
+    import torch
+    dt, op, k, n = O.INT32, O.SUM, 3, 70_001
+    rounds = 37
+    ins = [make_inputs(dt, k, n, seed=300 + r) for r in range(4)]
+    devs = [[to_dev(a) for a in g] for g in ins]
+    outs = [dev_empty(n, 4, fill=0) for _ in range(rounds)]
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(4, k, dt, op)
+    try:
+        for attempt in range(2):
+            with q:
+                full_seen = 0
+                for r in range(rounds):
+                    while True:
+                        t = q.try_enqueue_reduce([d.data_ptr() for d in devs[r % 4]], outs[r].data_ptr(), n)
+                        if t is not None:
+                            break
+                        full_seen += 1
+                    assert t == r + 1
+                    p, c, st = q.query()
+                    assert p - c <= 4 and st == RUNNING
+            p, c, st = q.query()
+            assert (p, c, st) == (rounds + 1, rounds + 1, STOPPED)  # + the stop entry
+            for r in range(rounds):
+                assert same(from_dev(outs[r], np.int32), expect(ins[r % 4], dt, op)), (attempt, r)
+                outs[r].zero_()
+            torch.cuda.synchronize()
+    finally:
+        q.close()
+
+
+def test_fifo_consumer_gives_up_when_idle(L):
+    """No entry ever arrives: the consumer leaves by itself after its spin limit,
+    the queue reports it, and a restart works.  Every wavefront exits normally."""
+    import time
+    import torch
+    dt, op = O.FP32, O.SUM
+    ins = make_inputs(dt, 2, 5000, seed=5)
+    devs = [to_dev(a) for a in ins]
+    out = dev_empty(5000, 4, fill=0)
+    torch.cuda.synchronize()
+    L.lib().flagcxLocalSetMaxSpinCount(2000)
+    q = L.ReduceFifo(4, 2, dt, op)
+    try:
+        q.start()
+        deadline = time.time() + 60
+        while q.query()[2] == RUNNING and time.time() < deadline:
+            time.sleep(0.01)
+        assert q.query()[2] == TIMED_OUT
+        with pytest.raises(L.FlagcxError):
+            q.enqueue_reduce([d.data_ptr() for d in devs], out.data_ptr(), 5000)
+        with pytest.raises(L.FlagcxError):
+            q.stop()
+        L.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+        with q:
+            q.enqueue_reduce([d.data_ptr() for d in devs], out.data_ptr(), 5000)
+        assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
+    finally:
+        L.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+        q.close()
+
+
+def test_fifo_chunked_shard_matches_single_launch(L):
+    """A reduce-scatter shard cut into 4 MiB chunks and fed chunk by chunk gives the
+    bytes of one launch over the whole shard (fp16 avg, 8 inputs)."""
+    import torch
+    dt, op, k = O.FP16, O.AVG, 8
+    chunk = 2 * 1024 * 1024  # elements = 4 MiB
+    nchunks = 8
+    n = chunk * nchunks
+    g = torch.Generator(device="cuda").manual_seed(1)
+    devs = [(torch.randn(n, generator=g, device="cuda") * 0.01).to(torch.float16) for _ in range(k)]
+    whole = torch.empty(n, dtype=torch.float16, device="cuda")
+    piecewise = torch.zeros(n, dtype=torch.float16, device="cuda")
+    L.reduce(devs, whole, op, dtype=dt)
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(16, k, dt, op)
+    try:
+        with q:
+            for c in range(nchunks):
+                q.enqueue_reduce([d.data_ptr() + c * chunk * 2 for d in devs], piecewise.data_ptr() + c * chunk * 2,
+                                 chunk)
+    finally:
+        q.close()
+    assert torch.equal(whole.view(torch.int16), piecewise.view(torch.int16))
+    sample = slice(0, 4096)
+    want = expect([d[sample].view(torch.int16).cpu().numpy().view(np.float16) for d in devs], dt, op)
+    assert same(piecewise[sample].view(torch.int16).cpu().numpy().view(np.float16), want, nan_class=True, dtype=dt)
