@@ -37,6 +37,7 @@ struct flagcxLocalReduceFifo {
   unsigned maxGrid = 0;
   unsigned grid = 0;
   int maxRanks = 0, dtype = 0, op = 0;
+  int wavesPerCU = 8;               // resident one-wave workgroups per CU
   size_t typeSize = 0;
   hipStream_t stream = nullptr;
   uint64_t produced = 0;            // host copy of header[kQueueProduced]
@@ -145,6 +146,11 @@ flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int ca
   q->dtype = dt;
   q->op = rop;
   q->typeSize = ts;
+  // Measured on MI355X (128 x 4 MiB chunks per input): few inputs want more
+  // wavefronts in flight, many inputs fewer; never more than half a CU's slots,
+  // so that residency does not depend on the last slot being free.
+  static const int kWaves[9] = {16, 16, 12, 12, 8, 8, 8, 8, 8};
+  q->wavesPerCU = kWaves[maxRanks];
   const DeviceInfo &info = deviceInfo();
   q->maxGrid = (unsigned)info.numCU * 16u;
   const size_t hostBytes = kQueueHeaderWords * sizeof(uint64_t) + (size_t)capacity * sizeof(QueueEntry);
@@ -196,10 +202,7 @@ flagcxResult_t flagcxLocalReduceFifoStart(flagcxLocalReduceFifo_t q) {
   a.maxSpin = asyncMaxSpin();
   // LDS is reserved only to spread the resident wavefronts evenly over the CUs, in
   // whole 1280-byte allocation granules so that exactly `waves` fit per CU
-  // (at most 16: half of a CU's wavefront slots, so that residency never depends
-  // on the last slot being free)
-  int waves = wavesPerCUFor(q->maxRanks);
-  if (waves <= 0 || waves > 16) waves = 16;
+  const int waves = q->wavesPerCU;
   const int lds = (deviceInfo().ldsPerCU / waves) / 1280 * 1280;
   const int err = reduceQueueLauncherFor(q->dtype)(q->op, a, waves, deviceInfo().numCU, lds, q->maxGrid, q->stream,
                                                    &q->grid);
@@ -320,6 +323,16 @@ flagcxResult_t flagcxLocalReduceFifoDestroy(flagcxLocalReduceFifo_t q) {
   delete q;
   if (e != hipSuccess || e2 != hipSuccess || e3 != hipSuccess) return flagcxUnhandledDeviceError;
   return r;
+}
+
+flagcxResult_t flagcxLocalReduceFifoSetWaves(flagcxLocalReduceFifo_t q, int wavesPerCU) {
+  if (!q) return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(q->mu);
+  if (wavesPerCU < 1 || wavesPerCU > 16)
+    return qfail(q, flagcxInvalidArgument, "flagcxLocalReduceFifoSetWaves: %d outside [1, 16]", wavesPerCU);
+  if (q->launched) return qfail(q, flagcxInvalidUsage, "flagcxLocalReduceFifoSetWaves: the consumer is running");
+  q->wavesPerCU = wavesPerCU;
+  return flagcxSuccess;
 }
 
 const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t q) { return q ? q->lastError : ""; }

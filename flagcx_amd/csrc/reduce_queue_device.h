@@ -303,6 +303,13 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
         default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nworkers); break;
       }
       rot = (uint32_t)((rot + ntiles) % nworkers);
+      // in a long run of entries let the count move every eighth entry, so that
+      // the producer's ring drains while the run is still going
+      if ((done & 7) == 0 && done < produced) {
+        waitOwnMemory();
+        if (threadIdx.x == 0)
+          __hip_atomic_store(q.progress + worker, (uint32_t)done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
     // this wavefront's results are acknowledged by memory before the count says so
     waitOwnMemory();

@@ -129,6 +129,7 @@ EXPORTS = [
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
+    "flagcxLocalReduceFifoSetWaves",
     "flagcxLocalReduceFifoGetLastError",
 ]
 
@@ -202,6 +203,7 @@ def lib():
         L.flagcxLocalReduceFifoQuery.argtypes = [vp, u64p, u64p, C.POINTER(i)]
         L.flagcxLocalReduceFifoWait.argtypes = [vp, C.c_uint64]
         L.flagcxLocalReduceFifoGetGrid.argtypes = [vp, C.POINTER(C.c_uint)]
+        L.flagcxLocalReduceFifoSetWaves.argtypes = [vp, i]
         L.flagcxLocalReduceFifoGetLastError.restype = C.c_char_p
         L.flagcxLocalReduceFifoGetLastError.argtypes = [vp]
         L.flagcxLocalSetMaxSpinCount.restype = None
@@ -479,6 +481,9 @@ class ReduceFifo:
 
     def wait(self, ticket):
         self._check(lib().flagcxLocalReduceFifoWait(self._h, ticket))
+
+    def set_waves(self, waves_per_cu):
+        self._check(lib().flagcxLocalReduceFifoSetWaves(self._h, waves_per_cu))
 
     def grid(self):
         g = C.c_uint()

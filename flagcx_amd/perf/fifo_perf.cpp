@@ -3,6 +3,7 @@
 // the same work:
 //
 //   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
+//             [-W wavesPerCU] [-s idleSpinLimit]
 //
 // A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
 // staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
@@ -56,6 +57,7 @@ int main(int argc, char **argv) {
   int k = 8, dtype = flagcxHalf, op = flagcxAvg, nchunks = 32, warmup = 5, iters = 20;
   size_t chunkBytes = FLAGCX_LOCAL_CHUNKSIZE;
   long long spin = 1ll << 22;
+  int tuneWaves = -1;
   for (int i = 1; i + 1 < argc; i += 2) {
     const char *f = argv[i], *v = argv[i + 1];
     if (!strcmp(f, "-k")) k = atoi(v);
@@ -66,6 +68,7 @@ int main(int argc, char **argv) {
     else if (!strcmp(f, "-w")) warmup = atoi(v);
     else if (!strcmp(f, "-n")) iters = atoi(v);
     else if (!strcmp(f, "-s")) spin = atoll(v);
+    else if (!strcmp(f, "-W")) tuneWaves = atoi(v);
   }
   flagcxLocalReduceFifo_t fifo = nullptr;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
@@ -121,6 +124,7 @@ int main(int argc, char **argv) {
 
   // (3) the resident consumer: enqueue chunk by chunk, wait for the last ticket
   FX(flagcxLocalReduceFifoCreate(&fifo, 64, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op));
+  if (tuneWaves > 0) FX(flagcxLocalReduceFifoSetWaves(fifo, tuneWaves));
   FX(flagcxLocalReduceFifoStart(fifo));
   unsigned grid = 0;
   FX(flagcxLocalReduceFifoGetGrid(fifo, &grid));

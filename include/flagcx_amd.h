@@ -401,6 +401,9 @@ flagcxResult_t flagcxLocalReduceFifoQuery(flagcxLocalReduceFifo_t fifo, uint64_t
 /* Spins on the host until consumed >= ticket.  flagcxInvalidArgument if the ticket
  * has not been handed out; an error if the consumer exits first. */
 flagcxResult_t flagcxLocalReduceFifoWait(flagcxLocalReduceFifo_t fifo, uint64_t ticket);
+/* Resident wavefronts per CU of the next Start (1..16; the default depends on
+ * maxRanks).  Not while the consumer runs. */
+flagcxResult_t flagcxLocalReduceFifoSetWaves(flagcxLocalReduceFifo_t fifo, int wavesPerCU);
 /* Workgroups (one wavefront each) of the running consumer: 1 leader + workers. */
 flagcxResult_t flagcxLocalReduceFifoGetGrid(flagcxLocalReduceFifo_t fifo, unsigned *workgroups);
 const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t fifo);
