@@ -200,10 +200,12 @@ flagcxResult_t flagcxLocalReduceFifoStart(flagcxLocalReduceFifo_t q) {
   a.progress = q->progress;
   a.capacity = q->capacity;
   a.maxSpin = asyncMaxSpin();
-  // LDS is reserved only to spread the resident wavefronts evenly over the CUs, in
-  // whole 1280-byte allocation granules so that exactly `waves` fit per CU
+  // LDS is reserved only to spread the resident wavefronts over the CUs (at most
+  // `waves` + 2 fit on one), in whole 1280-byte allocation granules.  A fifth of
+  // every CU's LDS stays free, so that other launches that need LDS (this library's
+  // own reductions on other streams) still make progress next to the consumer.
   const int waves = q->wavesPerCU;
-  const int lds = (deviceInfo().ldsPerCU / waves) / 1280 * 1280;
+  const int lds = ((deviceInfo().ldsPerCU - 32 * 1024) / waves) / 1280 * 1280;
   const int err = reduceQueueLauncherFor(q->dtype)(q->op, a, waves, deviceInfo().numCU, lds, q->maxGrid, q->stream,
                                                    &q->grid);
   if (err) {

@@ -363,8 +363,8 @@ flagcxResult_t flagcxLocalP2pDemo(const void *sendbuff, void *recvbuff, size_t c
  * Wait(ticket) or Stop.  Create / Start / Stop / Destroy allocate or synchronise
  * (setup time); Enqueue, Query and Wait touch pinned host memory only.
  *
- * While the consumer is resident it holds a share of every CU: launches that
- * reserve LDS (this library's 2..8-input reductions) queue behind it until Stop,
+ * While the consumer is resident it holds up to half of every CU's wavefront
+ * slots and four fifths of its LDS: other launches run next to it, more slowly,
  * and anything that synchronises the whole device (hipDeviceSynchronize, hipFree)
  * returns only after Stop or after the consumer's idle limit.  The consumer gives
  * up, state 3, after FLAGCX_FUNC_MAX_SPIN_COUNT polls without new entries or

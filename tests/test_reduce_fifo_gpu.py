@@ -182,6 +182,35 @@ def test_fifo_sees_inputs_rewritten_while_resident(L):
         assert same(got_echo[r], want), r
 
 
+def test_other_launches_run_next_to_the_resident_consumer(L):
+    """An ordinary 8-input reduce (which reserves LDS) and a copy on another stream
+    finish while the consumer stays resident and keeps serving entries."""
+    import torch
+    dt, op, k, n = O.BF16, O.SUM, 8, 1 << 20
+    ins = make_inputs(dt, k, n, seed=21)
+    devs = [to_dev(a) for a in ins]
+    out_q = dev_empty(n, 2, fill=0)
+    out_l = dev_empty(n, 2, fill=0)
+    out_c = dev_empty(n, 2, fill=0)
+    side = torch.cuda.Stream()
+    st = L.Stream(side.cuda_stream)
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(8, k, dt, op)
+    try:
+        with q:
+            L.reduce(devs, out_l, op, dtype=dt, stream=st)
+            L.memcpy(out_c.data_ptr(), out_l.data_ptr(), n * 2, stream=st)
+            side.synchronize()
+            assert q.query()[2] == RUNNING
+            q.wait(q.enqueue_reduce([d.data_ptr() for d in devs], out_q.data_ptr(), n))
+            assert q.query()[2] == RUNNING
+    finally:
+        q.close()
+    want = expect(ins, dt, op)
+    for got in (out_q, out_l, out_c):
+        assert same(from_dev(got, np.uint16), want, nan_class=True, dtype=dt)
+
+
 def test_fifo_ring_wraps_and_restarts(L):
     """More entries than slots (the producer sees 'full' and retries), then a second
     start on the same queue with counters back at zero."""

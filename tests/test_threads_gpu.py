@@ -1,0 +1,87 @@
+"""Re-entrancy of the C ABI: the reference enters its device layer from user threads,
+from the per-communicator proxy thread on its own stream (flagcx/core/proxy.cc:365-378,
+flagcx/core/p2p.cc:86-91) and from the kernel-proxy thread (proxy.cc:1074-1099), so
+every entry point must work from several threads at once, on streams made elsewhere."""
+import threading
+
+import numpy as np
+import pytest
+
+from oracle import cpu_oracle as O
+from tests.util import dev_empty, from_dev, make_inputs, same, to_dev
+
+
+@pytest.mark.gpu
+def test_concurrent_callers_on_their_own_streams():
+    import torch
+    from flagcx_amd import local as L
+    assert L.lib().flagcxLocalInit() == 0
+    nthreads, rounds = 6, 40
+    cases = [(O.BF16, O.SUM, 8), (O.FP32, O.SUM, 2), (O.INT32, O.MAX, 4), (O.FP16, O.AVG, 3), (O.INT64, O.MIN, 5),
+             (O.UINT8, O.PROD, 2)]
+    n = 200_003
+    work = []
+    for t in range(nthreads):
+        dt, op, k = cases[t]
+        ins = make_inputs(dt, k, n, seed=40 + t, op=op)
+        work.append((dt, op, ins, [to_dev(a) for a in ins], dev_empty(n, ins[0].dtype.itemsize, fill=0),
+                     dev_empty(n, ins[0].dtype.itemsize, fill=0)))
+    # streams are created here, on the main thread, and used from the workers
+    streams = [torch.cuda.Stream() for _ in range(nthreads)]
+    torch.cuda.synchronize()
+    errors = []
+    barrier = threading.Barrier(nthreads)
+
+    def run(t):
+        try:
+            dt, op, ins, devs, out, packed = work[t]
+            st = L.Stream(streams[t].cuda_stream)
+            barrier.wait()
+            for r in range(rounds):
+                L.reduce(devs, out, op, dtype=dt, stream=st)
+                L.memcpy(packed.data_ptr(), out.data_ptr(), n * ins[0].dtype.itemsize, stream=st)
+                if r % 8 == 0:
+                    # a deliberate error on this thread must not show up on the others
+                    rc = L.lib().flagcxLocalReduce(None, 2, None, 16, int(dt), int(op), None)
+                    assert rc == int(L.Result.InvalidArgument)
+                    assert b"flagcxLocalReduce" in L.lib().flagcxLocalGetLastError()
+            streams[t].synchronize()
+        except Exception as e:  # collected and re-raised on the main thread
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=run, args=(t,)) for t in range(nthreads)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(120)
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for t in range(nthreads):
+        dt, op, ins, devs, out, packed = work[t]
+        rc, want = O.reduce(ins, dt, op)
+        assert rc == 0
+        nan = dt in (O.BF16, O.FP16, O.FP32)
+        assert same(from_dev(out, ins[0].dtype), want, nan_class=nan, dtype=dt), t
+        assert same(from_dev(packed, ins[0].dtype), want, nan_class=nan, dtype=dt), t
+
+
+def test_last_error_is_per_thread():
+    from flagcx_amd import local as L
+    lib = L.lib()
+    seen = {}
+
+    def bad():
+        lib.flagcxLocalReduce(None, 99, None, 16, 7, 0, None)
+        seen["bad"] = lib.flagcxLocalGetLastError()
+
+    def clean():
+        seen["clean"] = lib.flagcxLocalGetLastError()
+
+    a = threading.Thread(target=bad)
+    a.start()
+    a.join()
+    b = threading.Thread(target=clean)
+    b.start()
+    b.join()
+    assert b"sendbuffs is NULL" in seen["bad"]
+    assert seen["clean"] == b""
