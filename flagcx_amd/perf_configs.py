@@ -86,6 +86,19 @@ def main():
     ms = timed(lambda: L.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks))
     report("C3 fp16 avg shard, 32 chunks as one batch call", nb, ms)
 
+    # the 32 chunk launches captured once into a HIP graph and replayed
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        L.reduce_scatter(send, 3, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        L.reduce_scatter(send, 3, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE)
+    ms = timed(graph.replay)
+    report("C3 fp16 avg shard, 32 chunk launches as one HIP graph", nb, ms)
+    del graph
+
     # the same shard with the 7 peers' slices staged through a 16 x 4 MiB ring on a second stream
     ring_mem = torch.empty(L.CHUNKSIZE * 16 * (nranks - 1), dtype=torch.uint8, device="cuda")
     ring = L.Ring(ring_mem, nranks - 1)
