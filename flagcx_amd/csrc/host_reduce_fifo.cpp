@@ -41,6 +41,7 @@ struct flagcxLocalReduceFifo {
   size_t typeSize = 0;
   hipStream_t stream = nullptr;
   uint64_t produced = 0;            // host copy of header[kQueueProduced]
+  uint64_t lastAfterAll = 0;        // index of the youngest entry marked kQueueFlagAfterAll
   bool launched = false;            // a consumer has been launched and not yet joined
   bool stopSent = false;
   std::mutex mu;                    // producers may be several threads
@@ -63,15 +64,38 @@ inline uint64_t headerLoad(const flagcxLocalReduceFifo *q, int word) {
   return __atomic_load_n(q->header + word, __ATOMIC_ACQUIRE);
 }
 
-inline bool overlaps(uintptr_t x, uintptr_t y, uint64_t bytes) { return x < y + bytes && y < x + bytes; }
+inline bool overlaps(uintptr_t x, uintptr_t y, uint64_t xbytes, uint64_t ybytes) {
+  return x < y + ybytes && y < x + xbytes;
+}
 
 // Appends one validated entry; the caller holds the mutex.
-flagcxResult_t appendEntry(flagcxLocalReduceFifo *q, const QueueEntry &e, uint64_t *ticket, const char *who) {
+flagcxResult_t appendEntry(flagcxLocalReduceFifo *q, const QueueEntry &in, uint64_t *ticket, const char *who) {
   if (!q->launched || q->stopSent) return qfail(q, flagcxInvalidUsage, "%s: the queue is not running", who);
   const uint64_t state = headerLoad(q, kQueueState);
   if (state != kQueueRunning)
     return qfail(q, flagcxInternalError, "%s: the consumer has exited (state %lld)", who, (long long)state);
-  if (q->produced - headerLoad(q, kQueueConsumed) >= q->capacity) return flagcxInProgress; // full: retry
+  const uint64_t consumed = headerLoad(q, kQueueConsumed);
+  if (q->produced - consumed >= q->capacity) return flagcxInProgress; // full: retry
+  // Entries are folded concurrently.  One that reads or overwrites what an entry
+  // still in flight writes, or overwrites what it reads, is marked to start after
+  // everything before it; entries older than the last such mark are finished by
+  // the time anything behind the mark starts, so only younger ones are compared.
+  QueueEntry e = in;
+  const size_t ts = q->typeSize;
+  auto bytesOf = [ts](const QueueEntry &x) { return ((uint64_t)x.head + x.tail) * ts + x.nvec * 16; };
+  const uint64_t eb = bytesOf(e);
+  for (uint64_t j = consumed > q->lastAfterAll ? consumed : q->lastAfterAll; j < q->produced; j++) {
+    const QueueEntry &o = q->hostEntries[j % q->capacity];
+    const uint64_t ob = bytesOf(o);
+    bool hit = overlaps((uintptr_t)e.dst, (uintptr_t)o.dst, eb, ob);
+    for (uint32_t a = 0; !hit && a < e.k; a++) hit = overlaps((uintptr_t)e.src[a], (uintptr_t)o.dst, eb, ob);
+    for (uint32_t a = 0; !hit && a < o.k; a++) hit = overlaps((uintptr_t)e.dst, (uintptr_t)o.src[a], eb, ob);
+    if (hit) {
+      e.flags |= kQueueFlagAfterAll;
+      q->lastAfterAll = q->produced;
+      break;
+    }
+  }
   memcpy(q->hostEntries + q->produced % q->capacity, &e, sizeof(e));
   q->produced++;
   __atomic_store_n(q->header + kQueueProduced, q->produced, __ATOMIC_RELEASE);
@@ -91,14 +115,14 @@ flagcxResult_t buildEntry(flagcxLocalReduceFifo *q, const void *const *srcs, int
   const uint64_t bytes = count * ts;
   memset(&e, 0, sizeof(e));
   const uintptr_t mis = (uintptr_t)dst & 15u;
-  e.vector = 1;
+  e.flags = kQueueFlagAligned;
   for (int j = 0; j < k; j++) {
     const uintptr_t s = (uintptr_t)srcs[j];
     if (!s) return qfail(q, flagcxInvalidArgument, "%s: sendbuffs[%d] is NULL", who, j);
     if (s % ts) return qfail(q, flagcxInvalidArgument, "%s: sendbuffs[%d] not aligned to its element size", who, j);
-    if (s != (uintptr_t)dst && overlaps(s, (uintptr_t)dst, bytes))
+    if (s != (uintptr_t)dst && overlaps(s, (uintptr_t)dst, bytes, bytes))
       return qfail(q, flagcxInvalidArgument, "%s: recvbuff partially overlaps sendbuffs[%d]", who, j);
-    if ((s & 15u) != mis) e.vector = 0;
+    if ((s & 15u) != mis) e.flags &= ~(uint32_t)kQueueFlagAligned;
     e.src[j] = (uint64_t)s;
   }
   e.dst = (uint64_t)(uintptr_t)dst;
@@ -186,6 +210,7 @@ flagcxResult_t flagcxLocalReduceFifoStart(flagcxLocalReduceFifo_t q) {
     if (r != flagcxSuccess) return r;
   }
   q->produced = 0;
+  q->lastAfterAll = 0;
   q->header[kQueueConsumed] = 0;
   q->header[kQueueProduced] = 0;
   __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueRunning, __ATOMIC_RELEASE);

@@ -50,7 +50,7 @@ struct alignas(128) QueueEntry {
   uint32_t head;    // elements before the body
   uint32_t tail;    // elements after it
   uint32_t k;       // number of inputs, 1..8; 0 = stop
-  uint32_t vector;  // 1: every source shares dst's address modulo 16
+  uint32_t flags;   // kQueueFlag*
   uint64_t pad[4];
 };
 static_assert(sizeof(QueueEntry) == 128, "queue entries are 16 words");
@@ -59,6 +59,10 @@ static_assert(sizeof(QueueEntry) == 128, "queue entries are 16 words");
 // ([capacity, consumed, produced, ...], flagcx/include/flagcx_kernel.h:75-77),
 // plus a state word.
 enum : int { kQueueCapacity = 0, kQueueConsumed = 1, kQueueProduced = 2, kQueueState = 3, kQueueHeaderWords = 16 };
+// Entry flags: every source shares dst's address modulo 16; the entry reads or
+// overwrites what an entry still in flight writes or reads, so it must start after
+// everything before it has finished.
+enum : uint32_t { kQueueFlagAligned = 1, kQueueFlagAfterAll = 2 };
 enum : uint64_t { kQueueIdle = 0, kQueueRunning = 1, kQueueStopped = 2, kQueueTimedOut = 3 };
 
 struct QueueKernelArgs {

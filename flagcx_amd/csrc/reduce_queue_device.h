@@ -117,31 +117,49 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
     agentStore(q.devProduced + 1, ++beat); // heartbeat: workers count polls only while this stands still
     if (stopAt == ~0ull) {
       const uint64_t produced = uniform64(systemLoad(q.hostHeader + kQueueProduced));
-      if (produced > forwarded) {
-        // four entries per round trip over PCIe: lane = 16 * entry + word
-        for (uint64_t base = forwarded; base < produced; base += 4) {
-          const uint64_t i = base + (lane >> 4);
-          const uint32_t word = lane & 15;
-          const bool valid = i < produced;
-          uint64_t w = 1;
-          if (valid) {
-            const uint64_t slot = i % q.capacity;
-            w = systemLoad(reinterpret_cast<const uint64_t *>(q.hostEntries + slot) + word);
-            agentStore(reinterpret_cast<uint64_t *>(q.devEntries + slot) + word, w);
-          }
-          // word 11 = k | vector << 32; k = 0 is the stop entry
-          const uint64_t stopMask = __ballot(valid && word == 11 && (uint32_t)w == 0);
-          uint64_t upto = base + 4 < produced ? base + 4 : produced;
-          if (stopMask) {
-            stopAt = base + ((uint64_t)(__ffsll((long long)stopMask) - 1) >> 4);
-            upto = stopAt + 1; // nothing after a stop entry is published
-          }
-          waitOwnMemory(); // the entries are in the device ring before the count says so
-          agentStore(q.devProduced, upto);
-          forwarded = upto;
-          if (stopMask) break;
+      // four entries per round trip over PCIe: lane = 16 * entry + word
+      while (forwarded < produced) {
+        const uint64_t i = forwarded + (lane >> 4);
+        const uint32_t word = lane & 15;
+        const bool valid = i < produced;
+        uint64_t w = 1;
+        if (valid) {
+          const uint64_t slot = i % q.capacity;
+          w = systemLoad(reinterpret_cast<const uint64_t *>(q.hostEntries + slot) + word);
+          agentStore(reinterpret_cast<uint64_t *>(q.devEntries + slot) + word, w);
         }
+        // word 11 = k | flags << 32; k = 0 is the stop entry; flag bit 1: this entry
+        // depends on an earlier one and starts only when everything before it is done
+        const bool isCtl = valid && word == 11;
+        const uint64_t stopMask = __ballot(isCtl && (uint32_t)w == 0);
+        const uint64_t waitMask = __ballot(isCtl && ((w >> 32) & kQueueFlagAfterAll) != 0);
+        uint64_t upto = forwarded + 4 < produced ? forwarded + 4 : produced;
+        bool blocked = false;
+        if (waitMask) {
+          const uint64_t at = forwarded + ((uint64_t)(__ffsll((long long)waitMask) - 1) >> 4);
+          if (at > forwarded) {
+            upto = at; // what precedes it goes out now, the entry itself in a later round
+          } else if (published < at) {
+            blocked = true; // its predecessors are still in flight
+          } else {
+            upto = at + 1;
+          }
+        }
+        if (blocked) break;
+        bool stopping = false;
+        if (stopMask) {
+          const uint64_t at = forwarded + ((uint64_t)(__ffsll((long long)stopMask) - 1) >> 4);
+          if (at < upto) {
+            stopAt = at;
+            upto = at + 1; // nothing after a stop entry is published
+            stopping = true;
+          }
+        }
+        waitOwnMemory(); // the entries are in the device ring before the count says so
+        agentStore(q.devProduced, upto);
+        forwarded = upto;
         spins = 0;
+        if (stopping) break;
       }
     }
     // min over the workers' 32-bit progress words, relative to what is published
@@ -282,7 +300,7 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
         stop = true;
         break;
       }
-      const bool vector = (kv >> 32) != 0;
+      const bool vector = ((kv >> 32) & kQueueFlagAligned) != 0;
       uint64_t src[8];
 #pragma unroll
       for (int b = 0; b < 8; b++) src[b] = laneWord(cur, b);

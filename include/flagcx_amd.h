@@ -356,8 +356,10 @@ flagcxResult_t flagcxLocalP2pDemo(const void *sendbuff, void *recvbuff, size_t c
  * (flagcx/core/proxy.cc:1094-1097).
  *
  * A queue is created for one element type and one op; entries carry 1..maxRanks
- * (at most 8) inputs.  Entries run in order; entries in flight together must not
- * depend on one another unless the producer waits for the earlier ticket first.
+ * (at most 8) inputs.  The result is that of running the entries one after
+ * another: independent entries are folded concurrently, and an entry that reads or
+ * overwrites what an earlier entry still in flight writes (or overwrites what it
+ * reads) is held back until everything before it has finished.
  * The producer appends an entry only when its inputs are complete in device
  * memory (an event or stream it has synchronised with), and reads results after
  * Wait(ticket) or Stop.  Create / Start / Stop / Destroy allocate or synchronise

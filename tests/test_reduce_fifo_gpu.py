@@ -111,7 +111,7 @@ def test_fifo_misaligned_and_in_place(L, dt, op, k):
 
 def test_fifo_triggers_chain(L):
     """Binary triggers in the reference's 256-bit layout: addr3 = OP(addr1, addr2).
-    A k-way sum as a chain through one accumulator, each link waiting for the last."""
+    A k-way sum as a chain through one accumulator."""
     import torch
     dt, op, k, n = O.FP32, O.SUM, 5, 300_001
     ins = make_inputs(dt, k, n, seed=11)
@@ -122,9 +122,9 @@ def test_fifo_triggers_chain(L):
     try:
         with q:
             # acc = in1 + in0, then acc = in_j + acc
+            # (no waits in between: the queue itself orders an entry behind the one it depends on)
             t = q.enqueue(L.ReduceTrigger.make(devs[1].data_ptr(), devs[0].data_ptr(), acc.data_ptr(), n, dt, op))
             for j in range(2, k):
-                q.wait(t)
                 t = q.enqueue(L.ReduceTrigger.make(devs[j].data_ptr(), acc.data_ptr(), acc.data_ptr(), n, dt, op))
             q.wait(t)
             # results are visible to a host copy while the consumer is still resident
@@ -209,6 +209,45 @@ def test_other_launches_run_next_to_the_resident_consumer(L):
     want = expect(ins, dt, op)
     for got in (out_q, out_l, out_c):
         assert same(from_dev(got, np.uint16), want, nan_class=True, dtype=dt)
+
+
+def test_fifo_orders_dependent_entries(L):
+    """Entries are folded concurrently unless one touches what another still in flight
+    reads or writes; then the result must be that of running them one after another.
+    Read-after-write, write-after-read and write-after-write, between independent ones."""
+    import torch
+    dt, op, n = O.INT32, O.SUM, 1_500_001
+    rng = np.random.default_rng(9)
+    h = {name: rng.integers(-2**31, 2**31 - 1, n, dtype=np.int32) for name in "abcdefg"}
+    d = {name: to_dev(v) for name, v in h.items()}
+    outs = {name: dev_empty(n, 4, fill=0) for name in ("p", "q", "r", "s")}
+    torch.cuda.synchronize()
+    P = lambda name: (d[name] if name in d else outs[name]).data_ptr()
+    program = [                      # (dst, srcs)
+        ("p", ["a", "b"]),           # p = a + b
+        ("a", ["c", "d"]),           # overwrites a while p may still be reading it
+        ("q", ["p", "a", "e"]),      # reads both results
+        ("r", ["f", "g"]),           # independent
+        ("q", ["q", "r"]),           # in place on q, needs q and r
+        ("s", ["e", "f"]),           # independent
+        ("s", ["g", "g"]),           # overwrites s
+    ]
+    q = L.ReduceFifo(4, 3, dt, op)
+    try:
+        with q:
+            for _ in range(3):       # several times over, through a ring of 4 slots
+                for dst, srcs in program:
+                    t = q.enqueue_reduce([P(x) for x in srcs], P(dst), n)
+            q.wait(t)
+    finally:
+        q.close()
+    env = {k_: v.copy() for k_, v in h.items()}
+    for _ in range(3):
+        for dst, srcs in program:
+            env[dst] = expect([env[x] for x in srcs], dt, op)
+    for name in ("p", "q", "r", "s"):
+        assert same(from_dev(outs[name], np.int32), env[name]), name
+    assert same(from_dev(d["a"], np.int32), env["a"])
 
 
 def test_fifo_ring_wraps_and_restarts(L):
