@@ -362,6 +362,15 @@ flagcxResult_t flagcxLocalReduceFifoSetWaves(flagcxLocalReduceFifo_t q, int wave
   return flagcxSuccess;
 }
 
+flagcxResult_t flagcxLocalReduceFifoGetType(flagcxLocalReduceFifo_t q, flagcxDataType_t *datatype, flagcxRedOp_t *op,
+                                            int *maxRanks) {
+  if (!q) return flagcxInvalidArgument;
+  if (datatype) *datatype = (flagcxDataType_t)q->dtype;
+  if (op) *op = (flagcxRedOp_t)q->op;
+  if (maxRanks) *maxRanks = q->maxRanks;
+  return flagcxSuccess;
+}
+
 const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t q) { return q ? q->lastError : ""; }
 
 flagcxResult_t flagcxLocalReduceFifoGetGrid(flagcxLocalReduceFifo_t q, unsigned *workgroups) {

@@ -157,5 +157,66 @@ flagcxResult_t flagcxLocalRingReduceScatter(flagcxLocalRing *r, const void *cons
   return flagcxSuccess;
 }
 
+// The same shard with the host in the role of the reference's proxy thread, which
+// never makes one stream wait for another: it issues a step's copy, records an
+// event, polls it with eventQuery and only then hands the step on
+// (flagcx/core/p2p.cc:75-107,170-205).  Here "hands on" is an entry in the resident
+// reduce queue, and a slot is free again when that entry's ticket is consumed.
+// Blocks until the shard is complete.
+flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing *r, flagcxLocalReduceFifo_t fifo,
+                                                const void *const *sendbuffs, int nranks, int rank,
+                                                void *recvbuff, size_t recvcount, flagcxStream_t copyStream) {
+  if (!r || !fifo || !sendbuffs || !copyStream) return flagcxInvalidArgument;
+  if (nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS || rank < 0 || rank >= nranks) return flagcxInvalidArgument;
+  if (nranks - 1 > r->npeers) return flagcxInvalidArgument;
+  flagcxDataType_t datatype;
+  flagcxRedOp_t op;
+  int maxRanks = 0;
+  RCHECK(flagcxLocalReduceFifoGetType(fifo, &datatype, &op, &maxRanks));
+  if (nranks > maxRanks) return flagcxInvalidArgument;
+  const size_t ts = flagcxLocalGetDataTypeSize(datatype);
+  if (!ts || (r->chunkBytes % ts)) return flagcxInvalidArgument;
+  if (recvcount == 0) return flagcxSuccess;
+  hipStream_t ps = hipOf(copyStream);
+  const size_t size = recvcount * ts;
+  const size_t nsteps = (size + r->chunkBytes - 1) / r->chunkBytes;
+  const size_t depth = (size_t)r->steps;
+  std::vector<uint64_t> ticket(depth, 0); // per slot: ticket of the entry that reads it
+  const void *peerSrc[FLAGCX_LOCAL_MAX_RANKS];
+  const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
+  size_t copied = 0, handed = 0; // steps whose copy is issued / whose reduce is enqueued
+  uint64_t lastTicket = 0, consumed = 0;
+  while (handed < nsteps) {
+    RCHECK(flagcxLocalReduceFifoQuery(fifo, nullptr, &consumed, nullptr));
+    // issue copies into free slots (sendHead side)
+    while (copied < nsteps && (copied < depth || (copied - depth < handed && consumed >= ticket[copied % depth]))) {
+      const size_t off = copied * r->chunkBytes;
+      const size_t n = size - off < r->chunkBytes ? size - off : r->chunkBytes;
+      for (int j = 0; j < nranks - 1; j++)
+        peerSrc[j] = (const char *)sendbuffs[(rank + 1 + j) % nranks] + (size_t)rank * size + off;
+      if (nranks > 1) RCHECK(flagcxLocalPackList(slotOf(r, copied, 0), peerSrc, nranks - 1, n, copyStream));
+      HCHECK(hipEventRecord(r->filled[copied % depth], ps));
+      copied++;
+    }
+    // hand on, in order, every step whose copy has completed (recvTail side)
+    while (handed < copied) {
+      const hipError_t q = hipEventQuery(r->filled[handed % depth]);
+      if (q == hipErrorNotReady) break;
+      if (q != hipSuccess) return flagcxUnhandledDeviceError;
+      const size_t off = handed * r->chunkBytes;
+      const size_t n = size - off < r->chunkBytes ? size - off : r->chunkBytes;
+      for (int j = 0; j < nranks - 1; j++) ordered[j] = slotOf(r, handed, 0) + (size_t)j * n;
+      ordered[nranks - 1] = (const char *)sendbuffs[rank] + (size_t)rank * size + off;
+      const flagcxResult_t e =
+          flagcxLocalReduceFifoEnqueueReduce(fifo, ordered, nranks, (char *)recvbuff + off, n / ts, &lastTicket);
+      if (e == flagcxInProgress) break; // queue full: its entries drain by themselves
+      if (e != flagcxSuccess) return e;
+      ticket[handed % depth] = lastTicket;
+      handed++;
+    }
+  }
+  return flagcxLocalReduceFifoWait(fifo, lastTicket);
+}
+
 } // extern "C"
 #pragma GCC visibility pop

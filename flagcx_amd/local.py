@@ -129,7 +129,7 @@ EXPORTS = [
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
-    "flagcxLocalReduceFifoSetWaves",
+    "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
     "flagcxLocalReduceFifoGetLastError",
 ]
 
@@ -204,6 +204,8 @@ def lib():
         L.flagcxLocalReduceFifoWait.argtypes = [vp, C.c_uint64]
         L.flagcxLocalReduceFifoGetGrid.argtypes = [vp, C.POINTER(C.c_uint)]
         L.flagcxLocalReduceFifoSetWaves.argtypes = [vp, i]
+        L.flagcxLocalReduceFifoGetType.argtypes = [vp, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
+        L.flagcxLocalRingReduceScatterFifo.argtypes = [vp, vp, pp, i, i, vp, sz, sp]
         L.flagcxLocalReduceFifoGetLastError.restype = C.c_char_p
         L.flagcxLocalReduceFifoGetLastError.argtypes = [vp]
         L.flagcxLocalSetMaxSpinCount.restype = None
@@ -410,6 +412,14 @@ class Ring:
         check(lib().flagcxLocalRingReduceScatter(self._h, _ptr_array([s.data_ptr() for s in sendbuffs]),
                                                  len(sendbuffs), rank, recv.data_ptr(), recv.numel(), int(dt),
                                                  int(op), C.byref(copy_stream), C.byref(stream)))
+
+    def reduce_scatter_fifo(self, fifo, sendbuffs, rank, recv, copy_stream):
+        """Proxy-style: staging copies on copy_stream, reduces through the running ReduceFifo; blocks."""
+        rc = lib().flagcxLocalRingReduceScatterFifo(self._h, fifo._h, _ptr_array([s.data_ptr() for s in sendbuffs]),
+                                                    len(sendbuffs), rank, recv.data_ptr(), recv.numel(),
+                                                    C.byref(copy_stream))
+        if rc:
+            raise FlagcxError(rc, (lib().flagcxLocalReduceFifoGetLastError(fifo._h) or b"").decode())
 
     def close(self):
         if self._h:

@@ -108,6 +108,22 @@ def main():
     # staging moves 2 x 7/8 of the inputs on top of the reduce's 9 x shard
     report("C3 shard through the staging ring (2 streams)", nb, ms,
            "HBM bytes incl. staging: %d" % (nb + 2 * (nranks - 1) * shard * 2))
+    # proxy-style: copies on one stream, polled events, reduces through the resident consumer (host wall clock)
+    import time
+    L.lib().flagcxLocalSetMaxSpinCount(1 << 22)
+    fifo = L.ReduceFifo(64, nranks, L.DataType.Float16, L.RedOp.Avg)
+    torch.cuda.synchronize()
+    with fifo:
+        for _ in range(5):
+            ring.reduce_scatter_fifo(fifo, send, 3, recv, cs)
+        t0 = time.perf_counter()
+        for _ in range(20):
+            ring.reduce_scatter_fifo(fifo, send, 3, recv, cs)
+        ms = (time.perf_counter() - t0) * 1e3 / 20
+    fifo.close()
+    L.lib().flagcxLocalSetMaxSpinCount(-1)
+    report("C3 shard through the ring + reduce queue (polled)", nb, ms,
+           "HBM bytes incl. staging: %d" % (nb + 2 * (nranks - 1) * shard * 2))
     ring.close()
     del ring_mem
 

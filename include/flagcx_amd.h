@@ -406,6 +406,9 @@ flagcxResult_t flagcxLocalReduceFifoWait(flagcxLocalReduceFifo_t fifo, uint64_t 
 /* Resident wavefronts per CU of the next Start (1..16; the default depends on
  * maxRanks).  Not while the consumer runs. */
 flagcxResult_t flagcxLocalReduceFifoSetWaves(flagcxLocalReduceFifo_t fifo, int wavesPerCU);
+/* What the queue was created for (any pointer may be NULL). */
+flagcxResult_t flagcxLocalReduceFifoGetType(flagcxLocalReduceFifo_t fifo, flagcxDataType_t *datatype,
+                                            flagcxRedOp_t *op, int *maxRanks);
 /* Workgroups (one wavefront each) of the running consumer: 1 leader + workers. */
 flagcxResult_t flagcxLocalReduceFifoGetGrid(flagcxLocalReduceFifo_t fifo, unsigned *workgroups);
 const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t fifo);
@@ -439,6 +442,16 @@ flagcxResult_t flagcxLocalRingReduceScatter(flagcxLocalRing_t ring, const void *
                                             int nranks, int rank, void *recvbuff, size_t recvcount,
                                             flagcxDataType_t datatype, flagcxRedOp_t op,
                                             flagcxStream_t copyStream, flagcxStream_t stream);
+/* The same shard driven the way the reference's proxy thread drives its steps
+ * (flagcx/core/p2p.cc:75-107,170-205): the caller's thread issues each step's
+ * staging copy on copyStream, records an event, polls it (eventQuery) and then
+ * hands the step to a running reduce queue; a slot is reused when that entry's
+ * ticket is consumed.  No stream waits for another and no reduce is launched.
+ * Type and op are the queue's; nranks <= its maxRanks.  Inputs must be complete
+ * in copyStream's order.  Blocks until recvbuff is complete. */
+flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing_t ring, flagcxLocalReduceFifo_t fifo,
+                                                const void *const *sendbuffs, int nranks, int rank,
+                                                void *recvbuff, size_t recvcount, flagcxStream_t copyStream);
 
 /* ------------------------------------------------------------------------- */
 /* C2C plan replay on one GPU                                                  */

@@ -74,6 +74,49 @@ def test_ring_reduce_scatter_equals_direct(L, dt, op, nranks, rcount, chunk, ste
     ring.close()
 
 
+@pytest.mark.parametrize("dt,op,nranks,rcount,chunk,steps", [
+    (O.FP32, O.SUM, 4, 10000, 4096, 4),          # many wraps of a small ring, ragged last chunk
+    (O.BF16, O.SUM, 8, 1 << 20, 1 << 18, 16),
+    (O.FP16, O.AVG, 8, (1 << 21) + 24, 0, 0),     # default 16 x 4 MiB ring
+    (O.INT32, O.MAX, 2, 5000, 4096, 2),
+    (O.INT64, O.MIN, 3, 70001, 8192, 3),
+])
+def test_ring_reduce_scatter_through_the_reduce_queue(L, dt, op, nranks, rcount, chunk, steps):
+    """Proxy-style progress: copies on one stream, polled events, reduces through the
+    resident consumer; same bytes as the direct call, for the first and the last rank,
+    twice over on one ring and one running queue (slots and tickets are reused)."""
+    import torch
+    ts = O.type_size(dt)
+    send_h = make_inputs(dt, nranks, nranks * rcount, seed=23 + dt, op=op)
+    send = [to_dev(h) for h in send_h]
+    ring_mem = torch.empty((steps or 16) * (nranks - 1) * (chunk or L.CHUNKSIZE), dtype=torch.uint8, device="cuda")
+    ring = L.Ring(ring_mem, nranks - 1, chunk, steps)
+    ta, tb, sa, sb = streams(L)
+    direct = {rank: dev_empty(rcount, ts) for rank in (0, nranks - 1)}
+    staged = {rank: dev_empty(rcount, ts, fill=0) for rank in (0, nranks - 1)}
+    for rank in direct:
+        L.reduce_scatter(send, rank, direct[rank], op, dtype=dt)
+    torch.cuda.synchronize()
+    L.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+    q = L.ReduceFifo(8, nranks, dt, op)
+    try:
+        with q:
+            for rep in range(2):
+                for rank in staged:
+                    ring.reduce_scatter_fifo(q, send, rank, staged[rank], sa)
+                    assert q.query()[2] == 1
+    finally:
+        q.close()
+        L.lib().flagcxLocalSetMaxSpinCount(-1)
+    torch.cuda.synchronize()
+    for rank in staged:
+        assert torch.equal(direct[rank], staged[rank]), rank
+        rc, want = O.reduce_scatter_rank(send_h, rank, rcount, dt, op)
+        nan_ok = dt in (O.FP16, O.BF16, O.FP32) and op in (O.SUM, O.AVG)
+        assert same(from_dev(staged[rank], send_h[0].dtype), want, nan_class=nan_ok, dtype=dt)
+    ring.close()
+
+
 def test_ring_rejects_bad_arguments(L):
     import torch
     mem = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
