@@ -42,8 +42,9 @@ struct flagcxLocalReduceFifo {
   hipStream_t stream = nullptr;
   uint64_t produced = 0;            // host copy of header[kQueueProduced]
   uint64_t lastAfterAll = 0;        // index of the youngest entry marked kQueueFlagAfterAll
-  bool launched = false;            // a consumer has been launched and not yet joined
+  bool started = false;             // between Start and Stop
   bool stopSent = false;
+  int64_t linger = 64;              // idle polls of the leader before the consumer parks (0: never)
   std::mutex mu;                    // producers may be several threads
   char lastError[256] = "";
 };
@@ -64,15 +65,65 @@ inline uint64_t headerLoad(const flagcxLocalReduceFifo *q, int word) {
   return __atomic_load_n(q->header + word, __ATOMIC_ACQUIRE);
 }
 
+inline uint64_t producedLoad(const flagcxLocalReduceFifo *q) {
+  return headerLoad(q, kQueueProduced) & ~kQueueParkedBit;
+}
+
+inline bool alive(uint64_t state) { return state == kQueueRunning || state == kQueueParked; }
+
 inline bool overlaps(uintptr_t x, uintptr_t y, uint64_t xbytes, uint64_t ybytes) {
   return x < y + ybytes && y < x + xbytes;
 }
 
+// Launches a consumer that takes over at entry `base` (everything before it is
+// finished).  The caller holds the mutex.
+flagcxResult_t launchConsumer(flagcxLocalReduceFifo *q, uint64_t base, const char *who) {
+  __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueRunning, __ATOMIC_RELEASE);
+  const size_t clearBytes = 128 + (size_t)q->maxGrid * sizeof(uint64_t);
+  hipError_t e = hipMemsetAsync(q->devProduced, 0, clearBytes, q->stream);
+  if (e != hipSuccess) return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString(e));
+  QueueKernelArgs a;
+  a.hostHeader = q->header;
+  a.hostEntries = q->hostEntries;
+  a.devEntries = q->devEntries;
+  a.devProduced = q->devProduced;
+  a.progress = q->progress;
+  a.capacity = q->capacity;
+  a.maxSpin = asyncMaxSpin();
+  a.base = base;
+  a.linger = q->linger;
+  // LDS is reserved only to spread the resident wavefronts over the CUs (at most
+  // `waves` + 2 fit on one), in whole 1280-byte allocation granules.  A fifth of
+  // every CU's LDS stays free, so that other launches that need LDS (this library's
+  // own reductions on other streams) still make progress next to the consumer.
+  const int waves = q->wavesPerCU;
+  const int lds = ((deviceInfo().ldsPerCU - 32 * 1024) / waves) / 1280 * 1280;
+  const int err = reduceQueueLauncherFor(q->dtype)(q->op, a, waves, deviceInfo().numCU, lds, q->maxGrid, q->stream,
+                                                   &q->grid);
+  if (err) {
+    __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueIdle, __ATOMIC_RELEASE);
+    return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString((hipError_t)err));
+  }
+  return flagcxSuccess;
+}
+
+// Publishes the entry already written at index q->produced.  If the consumer had
+// parked (the bit comes back with the old count), the bit is cleared and a new
+// consumer is launched from this entry on.  The caller holds the mutex.
+flagcxResult_t publishEntry(flagcxLocalReduceFifo *q, const char *who, bool *wasParked) {
+  const uint64_t old = __atomic_fetch_add(q->header + kQueueProduced, 1, __ATOMIC_ACQ_REL);
+  q->produced++;
+  *wasParked = (old & kQueueParkedBit) != 0;
+  if (!*wasParked) return flagcxSuccess;
+  __atomic_fetch_and(q->header + kQueueProduced, ~kQueueParkedBit, __ATOMIC_ACQ_REL);
+  return flagcxSuccess;
+}
+
 // Appends one validated entry; the caller holds the mutex.
 flagcxResult_t appendEntry(flagcxLocalReduceFifo *q, const QueueEntry &in, uint64_t *ticket, const char *who) {
-  if (!q->launched || q->stopSent) return qfail(q, flagcxInvalidUsage, "%s: the queue is not running", who);
+  if (!q->started || q->stopSent) return qfail(q, flagcxInvalidUsage, "%s: the queue is not running", who);
   const uint64_t state = headerLoad(q, kQueueState);
-  if (state != kQueueRunning)
+  if (!alive(state))
     return qfail(q, flagcxInternalError, "%s: the consumer has exited (state %lld)", who, (long long)state);
   const uint64_t consumed = headerLoad(q, kQueueConsumed);
   if (q->produced - consumed >= q->capacity) return flagcxInProgress; // full: retry
@@ -97,10 +148,12 @@ flagcxResult_t appendEntry(flagcxLocalReduceFifo *q, const QueueEntry &in, uint6
     }
   }
   memcpy(q->hostEntries + q->produced % q->capacity, &e, sizeof(e));
-  q->produced++;
-  __atomic_store_n(q->header + kQueueProduced, q->produced, __ATOMIC_RELEASE);
+  const uint64_t index = q->produced;
+  bool wasParked;
+  flagcxResult_t r = publishEntry(q, who, &wasParked);
+  if (r == flagcxSuccess && wasParked) r = launchConsumer(q, index, who);
   if (ticket) *ticket = q->produced;
-  return flagcxSuccess;
+  return r;
 }
 
 flagcxResult_t buildEntry(flagcxLocalReduceFifo *q, const void *const *srcs, int k, void *dst, uint64_t count,
@@ -137,12 +190,9 @@ flagcxResult_t buildEntry(flagcxLocalReduceFifo *q, const void *const *srcs, int
   return flagcxSuccess;
 }
 
-// Waits for the consumer kernel to leave the GPU and forgets it.
+// Waits until no consumer kernel is on the GPU.
 flagcxResult_t joinConsumer(flagcxLocalReduceFifo *q) {
-  if (!q->launched) return flagcxSuccess;
   const hipError_t e = hipStreamSynchronize(q->stream);
-  q->launched = false;
-  q->stopSent = false;
   return e == hipSuccess ? flagcxSuccess
                          : qfail(q, flagcxUnhandledDeviceError, "flagcxLocalReduceFifo: %s", hipGetErrorString(e));
 }
@@ -204,40 +254,19 @@ flagcxResult_t flagcxLocalReduceFifoStart(flagcxLocalReduceFifo_t q) {
   if (!q) return flagcxInvalidArgument;
   std::lock_guard<std::mutex> lock(q->mu);
   const char *who = "flagcxLocalReduceFifoStart";
-  if (q->launched) {
-    if (headerLoad(q, kQueueState) == kQueueRunning) return qfail(q, flagcxInvalidUsage, "%s: already running", who);
-    flagcxResult_t r = joinConsumer(q); // the previous consumer stopped or timed out
-    if (r != flagcxSuccess) return r;
+  if (q->started) {
+    if (alive(headerLoad(q, kQueueState))) return qfail(q, flagcxInvalidUsage, "%s: already running", who);
+    q->started = false; // the previous consumer timed out
   }
+  flagcxResult_t r = joinConsumer(q);
+  if (r != flagcxSuccess) return r;
   q->produced = 0;
   q->lastAfterAll = 0;
   q->header[kQueueConsumed] = 0;
-  q->header[kQueueProduced] = 0;
-  __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueRunning, __ATOMIC_RELEASE);
-  const size_t clearBytes = 128 + (size_t)q->maxGrid * sizeof(uint64_t);
-  hipError_t e = hipMemsetAsync(q->devProduced, 0, clearBytes, q->stream);
-  if (e != hipSuccess) return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString(e));
-  QueueKernelArgs a;
-  a.hostHeader = q->header;
-  a.hostEntries = q->hostEntries;
-  a.devEntries = q->devEntries;
-  a.devProduced = q->devProduced;
-  a.progress = q->progress;
-  a.capacity = q->capacity;
-  a.maxSpin = asyncMaxSpin();
-  // LDS is reserved only to spread the resident wavefronts over the CUs (at most
-  // `waves` + 2 fit on one), in whole 1280-byte allocation granules.  A fifth of
-  // every CU's LDS stays free, so that other launches that need LDS (this library's
-  // own reductions on other streams) still make progress next to the consumer.
-  const int waves = q->wavesPerCU;
-  const int lds = ((deviceInfo().ldsPerCU - 32 * 1024) / waves) / 1280 * 1280;
-  const int err = reduceQueueLauncherFor(q->dtype)(q->op, a, waves, deviceInfo().numCU, lds, q->maxGrid, q->stream,
-                                                   &q->grid);
-  if (err) {
-    __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueIdle, __ATOMIC_RELEASE);
-    return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString((hipError_t)err));
-  }
-  q->launched = true;
+  __atomic_store_n(q->header + kQueueProduced, (uint64_t)0, __ATOMIC_RELEASE);
+  r = launchConsumer(q, 0, who);
+  if (r != flagcxSuccess) return r;
+  q->started = true;
   q->stopSent = false;
   return flagcxSuccess;
 }
@@ -287,7 +316,7 @@ flagcxResult_t flagcxLocalReduceFifoQuery(flagcxLocalReduceFifo_t q, uint64_t *p
                                           int *state) {
   if (!q) return flagcxInvalidArgument;
   if (consumed) *consumed = headerLoad(q, kQueueConsumed);
-  if (produced) *produced = headerLoad(q, kQueueProduced);
+  if (produced) *produced = producedLoad(q);
   if (state) *state = (int)headerLoad(q, kQueueState);
   return flagcxSuccess;
 }
@@ -295,12 +324,12 @@ flagcxResult_t flagcxLocalReduceFifoQuery(flagcxLocalReduceFifo_t q, uint64_t *p
 flagcxResult_t flagcxLocalReduceFifoWait(flagcxLocalReduceFifo_t q, uint64_t ticket) {
   if (!q) return flagcxInvalidArgument;
   const char *who = "flagcxLocalReduceFifoWait";
-  if (ticket > headerLoad(q, kQueueProduced))
+  if (ticket > producedLoad(q))
     return qfail(q, flagcxInvalidArgument, "%s: ticket %lld has not been handed out", who, (long long)ticket);
   for (;;) {
     if (headerLoad(q, kQueueConsumed) >= ticket) return flagcxSuccess;
     const uint64_t state = headerLoad(q, kQueueState);
-    if (state != kQueueRunning) {
+    if (!alive(state)) {
       if (headerLoad(q, kQueueConsumed) >= ticket) return flagcxSuccess;
       return qfail(q, state == kQueueTimedOut ? flagcxInternalError : flagcxInvalidUsage,
                    "%s: the consumer is not running (state %lld) and entry %lld was not reached", who,
@@ -313,18 +342,26 @@ flagcxResult_t flagcxLocalReduceFifoWait(flagcxLocalReduceFifo_t q, uint64_t tic
 flagcxResult_t flagcxLocalReduceFifoStop(flagcxLocalReduceFifo_t q) {
   if (!q) return flagcxInvalidArgument;
   std::lock_guard<std::mutex> lock(q->mu);
-  if (!q->launched) return flagcxSuccess;
-  if (!q->stopSent && headerLoad(q, kQueueState) == kQueueRunning) {
+  if (!q->started) return flagcxSuccess;
+  const char *who = "flagcxLocalReduceFifoStop";
+  if (!q->stopSent && alive(headerLoad(q, kQueueState))) {
     QueueEntry e;
     memset(&e, 0, sizeof(e)); // k = 0
     // a full ring drains by itself: entries ahead of the stop entry finish first
     for (;;) {
-      if (headerLoad(q, kQueueState) != kQueueRunning) break;
+      if (!alive(headerLoad(q, kQueueState))) break;
       if (q->produced - headerLoad(q, kQueueConsumed) < q->capacity) {
         memcpy(q->hostEntries + q->produced % q->capacity, &e, sizeof(e));
-        q->produced++;
-        __atomic_store_n(q->header + kQueueProduced, q->produced, __ATOMIC_RELEASE);
+        bool wasParked;
+        (void)publishEntry(q, who, &wasParked);
         q->stopSent = true;
+        if (wasParked) {
+          // no consumer is left to read the stop entry, and nothing was outstanding
+          __atomic_store_n(q->header + kQueueConsumed, q->produced, __ATOMIC_RELEASE);
+          flagcxResult_t r = joinConsumer(q); // the parked kernel's last stores are done
+          if (r != flagcxSuccess) return r;
+          __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueStopped, __ATOMIC_RELEASE);
+        }
         break;
       }
       sched_yield();
@@ -332,11 +369,13 @@ flagcxResult_t flagcxLocalReduceFifoStop(flagcxLocalReduceFifo_t q) {
   }
   const uint64_t want = q->produced;
   flagcxResult_t r = joinConsumer(q);
+  q->started = false;
+  q->stopSent = false;
   if (r != flagcxSuccess) return r;
   const uint64_t state = headerLoad(q, kQueueState);
   if (state == kQueueTimedOut || headerLoad(q, kQueueConsumed) < want)
     return qfail(q, flagcxInternalError,
-                 "flagcxLocalReduceFifoStop: the consumer gave up after its spin limit with %lld of %lld entries done",
+                 "%s: the consumer gave up after its spin limit with %lld of %lld entries done", who,
                  (long long)headerLoad(q, kQueueConsumed), (long long)want);
   return flagcxSuccess;
 }
@@ -357,8 +396,17 @@ flagcxResult_t flagcxLocalReduceFifoSetWaves(flagcxLocalReduceFifo_t q, int wave
   std::lock_guard<std::mutex> lock(q->mu);
   if (wavesPerCU < 1 || wavesPerCU > 16)
     return qfail(q, flagcxInvalidArgument, "flagcxLocalReduceFifoSetWaves: %d outside [1, 16]", wavesPerCU);
-  if (q->launched) return qfail(q, flagcxInvalidUsage, "flagcxLocalReduceFifoSetWaves: the consumer is running");
+  if (q->started) return qfail(q, flagcxInvalidUsage, "flagcxLocalReduceFifoSetWaves: the queue is started");
   q->wavesPerCU = wavesPerCU;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduceFifoSetLinger(flagcxLocalReduceFifo_t q, int64_t polls) {
+  if (!q) return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(q->mu);
+  if (polls < 0) return qfail(q, flagcxInvalidArgument, "flagcxLocalReduceFifoSetLinger: negative");
+  if (q->started) return qfail(q, flagcxInvalidUsage, "flagcxLocalReduceFifoSetLinger: the queue is started");
+  q->linger = polls;
   return flagcxSuccess;
 }
 

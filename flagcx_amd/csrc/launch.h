@@ -63,7 +63,12 @@ enum : int { kQueueCapacity = 0, kQueueConsumed = 1, kQueueProduced = 2, kQueueS
 // overwrites what an entry still in flight writes or reads, so it must start after
 // everything before it has finished.
 enum : uint32_t { kQueueFlagAligned = 1, kQueueFlagAfterAll = 2 };
-enum : uint64_t { kQueueIdle = 0, kQueueRunning = 1, kQueueStopped = 2, kQueueTimedOut = 3 };
+enum : uint64_t { kQueueIdle = 0, kQueueRunning = 1, kQueueStopped = 2, kQueueTimedOut = 3, kQueueParked = 4 };
+// Top bit of the `produced` word: set by the consumer (compare-and-swap against an
+// unchanged count) when it leaves an idle queue, seen and cleared by the producer's
+// next fetch-and-add, which then launches a new consumer.  One word, so exactly one
+// side wins when an entry arrives while the consumer is leaving.
+constexpr uint64_t kQueueParkedBit = 1ull << 63;
 
 struct QueueKernelArgs {
   uint64_t *hostHeader;          // pinned, device-visible
@@ -73,6 +78,8 @@ struct QueueKernelArgs {
   uint32_t *progress;            // per worker: entries finished (low 32 bits)
   uint32_t capacity;
   int64_t maxSpin;
+  uint64_t base;                 // entries finished before this launch; device counts are relative to it
+  int64_t linger;                // idle polls before the consumer parks; 0 = stay until stopped
 };
 
 // Launches the consumer for one element type: grid = min(occupancy, wavesPerCU) *

@@ -31,7 +31,9 @@
 // (the leader counts polls without new entries or progress and then tells the
 // workers to leave; a worker counts polls during which the leader's heartbeat
 // word did not move).  A stop entry (k = 0) drains the queue: workers exit when
-// they reach it.
+// they reach it.  A queue with nothing outstanding for `linger` polls parks: the
+// kernel ends, so streams that share its hardware queue are held up only while
+// there is work, and the producer's next entry launches it again.
 #pragma once
 
 #include "launch.h"
@@ -111,12 +113,14 @@ __device__ __forceinline__ void coherentStore(uint64_t base, uint64_t i, T v) {
 __device__ inline void queueLeader(const QueueKernelArgs &q) {
   const uint32_t nworkers = gridDim.x - 1;
   const uint32_t lane = threadIdx.x;
-  uint64_t forwarded = 0, published = 0, stopAt = ~0ull, beat = 0;
-  int64_t spins = 0;
+  // host counts are absolute, the device words (devProduced, progress) relative to q.base
+  uint64_t forwarded = q.base, published = q.base, stopAt = ~0ull, beat = 0, produced = q.base;
+  int64_t spins = 0, idle = 0;
+  if (lane == 0) systemStore(q.hostHeader + kQueueState, kQueueRunning);
   for (;;) {
     agentStore(q.devProduced + 1, ++beat); // heartbeat: workers count polls only while this stands still
     if (stopAt == ~0ull) {
-      const uint64_t produced = uniform64(systemLoad(q.hostHeader + kQueueProduced));
+      produced = uniform64(systemLoad(q.hostHeader + kQueueProduced)) & ~kQueueParkedBit;
       // four entries per round trip over PCIe: lane = 16 * entry + word
       while (forwarded < produced) {
         const uint64_t i = forwarded + (lane >> 4);
@@ -156,14 +160,14 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
           }
         }
         waitOwnMemory(); // the entries are in the device ring before the count says so
-        agentStore(q.devProduced, upto);
+        agentStore(q.devProduced, upto - q.base);
         forwarded = upto;
         spins = 0;
         if (stopping) break;
       }
     }
     // min over the workers' 32-bit progress words, relative to what is published
-    const uint32_t base32 = (uint32_t)published;
+    const uint32_t base32 = (uint32_t)(published - q.base);
     uint32_t ahead = ~0u;
     __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)q.progress, 0, nworkers * 4u, kRsrcFlags);
     for (uint32_t v0 = 0; v0 < nworkers; v0 += 1024) {
@@ -192,6 +196,30 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
       waitOwnMemory();
       systemStore(q.hostHeader + kQueueState, kQueueStopped);
       return;
+    }
+    // Nothing outstanding for q.linger polls: leave the GPU to others.  The park bit
+    // goes into the `produced` word itself, only if the count is still the one seen;
+    // the producer's next fetch-and-add finds the bit and launches a new consumer.
+    if (q.linger > 0 && stopAt == ~0ull && forwarded == produced && published == forwarded) {
+      if (++idle > q.linger) {
+        uint32_t parked = 0;
+        if (lane == 0) {
+          uint64_t expected = forwarded;
+          parked = __hip_atomic_compare_exchange_strong(q.hostHeader + kQueueProduced, &expected,
+                                                        forwarded | kQueueParkedBit, __ATOMIC_ACQ_REL,
+                                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM)
+                       ? 1u
+                       : 0u;
+        }
+        if (__builtin_amdgcn_readfirstlane(parked)) {
+          agentStore(q.devProduced, ~0ull); // workers leave at their next poll
+          systemStore(q.hostHeader + kQueueState, kQueueParked);
+          return;
+        }
+        idle = 0; // an entry arrived in between
+      }
+    } else {
+      idle = 0;
     }
     if (++spins > q.maxSpin) {
       agentStore(q.devProduced, ~0ull); // workers leave at their next poll
@@ -263,7 +291,7 @@ template <typename T, int OP>
 __device__ inline void queueWorker(const QueueKernelArgs &q) {
   const uint32_t nworkers = gridDim.x - 1;
   const uint32_t worker = blockIdx.x - 1;
-  uint64_t done = 0; // entries this worker has finished
+  uint64_t done = 0; // entries this worker has finished since this launch (entry index = q.base + done)
   uint64_t lastBeat = 0;
   uint32_t rot = 0;  // tiles handed out so far, modulo nworkers
   for (;;) {
@@ -287,11 +315,11 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
     // lane l holds word l & 15 of the entry; the next entry is fetched while this
     // one's tiles are in flight
     uint64_t words =
-        agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + done % q.capacity) + (threadIdx.x & 15));
+        agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (q.base + done) % q.capacity) + (threadIdx.x & 15));
     while (done < produced) {
       const uint64_t cur = words;
       if (done + 1 < produced)
-        words = agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (done + 1) % q.capacity) +
+        words = agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (q.base + done + 1) % q.capacity) +
                           (threadIdx.x & 15));
       const uint64_t kv = laneWord(cur, 11);
       const int k = (int)(uint32_t)kv;

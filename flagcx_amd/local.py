@@ -129,7 +129,7 @@ EXPORTS = [
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
-    "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
+    "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoSetLinger", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
     "flagcxLocalReduceFifoGetLastError",
 ]
 
@@ -204,6 +204,7 @@ def lib():
         L.flagcxLocalReduceFifoWait.argtypes = [vp, C.c_uint64]
         L.flagcxLocalReduceFifoGetGrid.argtypes = [vp, C.POINTER(C.c_uint)]
         L.flagcxLocalReduceFifoSetWaves.argtypes = [vp, i]
+        L.flagcxLocalReduceFifoSetLinger.argtypes = [vp, C.c_int64]
         L.flagcxLocalReduceFifoGetType.argtypes = [vp, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
         L.flagcxLocalRingReduceScatterFifo.argtypes = [vp, vp, pp, i, i, vp, sz, sp]
         L.flagcxLocalReduceFifoGetLastError.restype = C.c_char_p
@@ -436,9 +437,9 @@ class Ring:
 class ReduceFifo:
     """Host-producer / device-consumer reduce queue (flagcxLocalReduceFifo*).
 
-    While it runs, do not synchronise the whole device (torch.cuda.synchronize, freeing
-    tensors): that returns only after stop().  Use it as a context manager so that an
-    exception between start and stop still stops the resident kernel.
+    The consumer kernel is on the GPU while entries are outstanding and for a short linger
+    after; then it parks and the next entry launches it again.  Use the object as a context
+    manager so that an exception between start and stop still stops it.
     """
 
     def __init__(self, capacity, max_ranks, dtype, op):
@@ -491,6 +492,9 @@ class ReduceFifo:
 
     def wait(self, ticket):
         self._check(lib().flagcxLocalReduceFifoWait(self._h, ticket))
+
+    def set_linger(self, polls):
+        self._check(lib().flagcxLocalReduceFifoSetLinger(self._h, polls))
 
     def set_waves(self, waves_per_cu):
         self._check(lib().flagcxLocalReduceFifoSetWaves(self._h, waves_per_cu))

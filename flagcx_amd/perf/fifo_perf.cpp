@@ -3,7 +3,7 @@
 // the same work:
 //
 //   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
-//             [-W wavesPerCU] [-s idleSpinLimit]
+//             [-W wavesPerCU] [-L lingerPolls] [-s spinLimit]
 //
 // A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
 // staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
@@ -19,6 +19,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <thread>
 #include <vector>
 
 #define CK(x)                                                                  \
@@ -58,6 +59,7 @@ int main(int argc, char **argv) {
   size_t chunkBytes = FLAGCX_LOCAL_CHUNKSIZE;
   long long spin = 1ll << 22;
   int tuneWaves = -1;
+  long long linger = -1;
   for (int i = 1; i + 1 < argc; i += 2) {
     const char *f = argv[i], *v = argv[i + 1];
     if (!strcmp(f, "-k")) k = atoi(v);
@@ -69,6 +71,7 @@ int main(int argc, char **argv) {
     else if (!strcmp(f, "-n")) iters = atoi(v);
     else if (!strcmp(f, "-s")) spin = atoll(v);
     else if (!strcmp(f, "-W")) tuneWaves = atoi(v);
+    else if (!strcmp(f, "-L")) linger = atoll(v);
   }
   flagcxLocalReduceFifo_t fifo = nullptr;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
@@ -125,6 +128,7 @@ int main(int argc, char **argv) {
   // (3) the resident consumer: enqueue chunk by chunk, wait for the last ticket
   FX(flagcxLocalReduceFifoCreate(&fifo, 64, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op));
   if (tuneWaves > 0) FX(flagcxLocalReduceFifoSetWaves(fifo, tuneWaves));
+  if (linger >= 0) FX(flagcxLocalReduceFifoSetLinger(fifo, linger));
   FX(flagcxLocalReduceFifoStart(fifo));
   unsigned grid = 0;
   FX(flagcxLocalReduceFifoGetGrid(fifo, &grid));
@@ -156,6 +160,22 @@ int main(int argc, char **argv) {
     t.push_back(nowUs() - t0);
   }
   const double fifoLat = median(t);
+  // the same entry after the consumer has parked (the enqueue launches it again)
+  t.clear();
+  for (int it = 0; it < 20; it++) {
+    int state = 0;
+    for (int spin = 0; spin < 2000 && state != FLAGCX_LOCAL_REDUCE_FIFO_PARKED; spin++) {
+      FX(flagcxLocalReduceFifoQuery(fifo, nullptr, nullptr, &state));
+      std::this_thread::sleep_for(std::chrono::microseconds(50));
+    }
+    if (state != FLAGCX_LOCAL_REDUCE_FIFO_PARKED) break; // parking is off (-L 0)
+    uint64_t ticket = 0;
+    const double t0 = nowUs();
+    FX(flagcxLocalReduceFifoEnqueueReduce(fifo, chunkSrc[0].data(), k, dst, smallCount, &ticket));
+    FX(flagcxLocalReduceFifoWait(fifo, ticket));
+    t.push_back(nowUs() - t0);
+  }
+  const double parkedLat = t.empty() ? 0.0 : median(t);
   FX(flagcxLocalReduceFifoStop(fifo));
   t.clear();
   for (int it = 0; it < 200; it++) {
@@ -164,7 +184,8 @@ int main(int argc, char **argv) {
     CK(hipStreamSynchronize(st.base));
     t.push_back(nowUs() - t0);
   }
-  printf("4 KiB entry: enqueue -> Wait %.2f us; launch -> stream sync %.2f us\n", fifoLat, median(t));
+  printf("4 KiB entry: enqueue -> Wait %.2f us (consumer on the GPU), %.2f us (parked, launched again); "
+         "launch -> stream sync %.2f us\n", fifoLat, parkedLat, median(t));
   FX(flagcxLocalReduceFifoDestroy(fifo));
   fifo = nullptr;
   for (int j = 0; j < k; j++) CK(hipFree(src[j]));

@@ -365,17 +365,24 @@ flagcxResult_t flagcxLocalP2pDemo(const void *sendbuff, void *recvbuff, size_t c
  * Wait(ticket) or Stop.  Create / Start / Stop / Destroy allocate or synchronise
  * (setup time); Enqueue, Query and Wait touch pinned host memory only.
  *
- * While the consumer is resident it holds up to half of every CU's wavefront
+ * While the consumer is on the GPU it holds up to half of every CU's wavefront
  * slots and four fifths of its LDS: other launches run next to it, more slowly,
- * and anything that synchronises the whole device (hipDeviceSynchronize, hipFree)
- * returns only after Stop or after the consumer's idle limit.  The consumer gives
- * up, state 3, after FLAGCX_FUNC_MAX_SPIN_COUNT polls without new entries or
- * progress (flagcxLocalSetMaxSpinCount; default 2^27, minutes). */
+ * except those on streams that the runtime has mapped to the same hardware queue,
+ * which wait like behind any other kernel.  So the consumer does not outstay its
+ * work: after `linger` polls (about 3 us each, default 64) with nothing
+ * outstanding it parks, i.e. the kernel ends, and the next Enqueue launches it
+ * again (about 20 us more for that entry).  Device-wide synchronisation
+ * (hipDeviceSynchronize, hipFree) therefore returns once the queue has drained
+ * and lingered.  With linger 0 the consumer stays until Stop.  If entries are
+ * outstanding and nothing moves for FLAGCX_FUNC_MAX_SPIN_COUNT polls
+ * (flagcxLocalSetMaxSpinCount; default 2^27, minutes) the consumer gives up,
+ * state 3. */
 typedef struct flagcxLocalReduceFifo *flagcxLocalReduceFifo_t;
 #define FLAGCX_LOCAL_REDUCE_FIFO_IDLE 0
 #define FLAGCX_LOCAL_REDUCE_FIFO_RUNNING 1
 #define FLAGCX_LOCAL_REDUCE_FIFO_STOPPED 2
 #define FLAGCX_LOCAL_REDUCE_FIFO_TIMED_OUT 3
+#define FLAGCX_LOCAL_REDUCE_FIFO_PARKED 4 /* started, idle, off the GPU until the next entry */
 
 flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int capacity, int maxRanks,
                                            flagcxDataType_t datatype, flagcxRedOp_t op);
@@ -404,11 +411,13 @@ flagcxResult_t flagcxLocalReduceFifoQuery(flagcxLocalReduceFifo_t fifo, uint64_t
  * has not been handed out; an error if the consumer exits first. */
 flagcxResult_t flagcxLocalReduceFifoWait(flagcxLocalReduceFifo_t fifo, uint64_t ticket);
 /* Resident wavefronts per CU of the next Start (1..16; the default depends on
- * maxRanks).  Not while the consumer runs. */
+ * maxRanks).  Not between Start and Stop. */
 flagcxResult_t flagcxLocalReduceFifoSetWaves(flagcxLocalReduceFifo_t fifo, int wavesPerCU);
 /* What the queue was created for (any pointer may be NULL). */
 flagcxResult_t flagcxLocalReduceFifoGetType(flagcxLocalReduceFifo_t fifo, flagcxDataType_t *datatype,
                                             flagcxRedOp_t *op, int *maxRanks);
+/* Idle polls before the consumer parks (0: never).  Not between Start and Stop. */
+flagcxResult_t flagcxLocalReduceFifoSetLinger(flagcxLocalReduceFifo_t fifo, int64_t polls);
 /* Workgroups (one wavefront each) of the running consumer: 1 leader + workers. */
 flagcxResult_t flagcxLocalReduceFifoGetGrid(flagcxLocalReduceFifo_t fifo, unsigned *workgroups);
 const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t fifo);

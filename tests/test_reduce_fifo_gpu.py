@@ -13,7 +13,8 @@ from tests.util import DT_NAME, OP_NAME, dev_empty, from_dev, is_float, make_inp
 
 pytestmark = pytest.mark.gpu
 
-RUNNING, STOPPED, TIMED_OUT = 1, 2, 3
+RUNNING, STOPPED, TIMED_OUT, PARKED = 1, 2, 3, 4
+ALIVE = (RUNNING, PARKED)
 
 
 @pytest.fixture(scope="module")
@@ -201,9 +202,9 @@ def test_other_launches_run_next_to_the_resident_consumer(L):
             L.reduce(devs, out_l, op, dtype=dt, stream=st)
             L.memcpy(out_c.data_ptr(), out_l.data_ptr(), n * 2, stream=st)
             side.synchronize()
-            assert q.query()[2] == RUNNING
+            assert q.query()[2] in ALIVE
             q.wait(q.enqueue_reduce([d.data_ptr() for d in devs], out_q.data_ptr(), n))
-            assert q.query()[2] == RUNNING
+            assert q.query()[2] in ALIVE
     finally:
         q.close()
     want = expect(ins, dt, op)
@@ -273,7 +274,7 @@ def test_fifo_ring_wraps_and_restarts(L):
                         full_seen += 1
                     assert t == r + 1
                     p, c, st = q.query()
-                    assert p - c <= 4 and st == RUNNING
+                    assert p - c <= 4 and st in ALIVE
             p, c, st = q.query()
             assert (p, c, st) == (rounds + 1, rounds + 1, STOPPED)  # + the stop entry
             for r in range(rounds):
@@ -285,8 +286,9 @@ def test_fifo_ring_wraps_and_restarts(L):
 
 
 def test_fifo_consumer_gives_up_when_idle(L):
-    """No entry ever arrives: the consumer leaves by itself after its spin limit,
-    the queue reports it, and a restart works.  Every wavefront exits normally."""
+    """With parking switched off and a tiny spin limit, a consumer that never gets an
+    entry leaves by itself, the queue reports it, and a restart works.  Every
+    wavefront exits normally."""
     import time
     import torch
     dt, op = O.FP32, O.SUM
@@ -296,6 +298,7 @@ def test_fifo_consumer_gives_up_when_idle(L):
     torch.cuda.synchronize()
     L.lib().flagcxLocalSetMaxSpinCount(2000)
     q = L.ReduceFifo(4, 2, dt, op)
+    q.set_linger(0)
     try:
         q.start()
         deadline = time.time() + 60
@@ -312,6 +315,48 @@ def test_fifo_consumer_gives_up_when_idle(L):
         assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
     finally:
         L.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+        q.close()
+
+
+def test_fifo_parks_when_idle_and_comes_back(L):
+    """Nothing outstanding for `linger` polls: the kernel ends (a device-wide
+    synchronisation returns), the queue stays usable, and the next entry launches the
+    consumer again with the counters carried on.  Several idle gaps, a stop while
+    parked, and a restart."""
+    import time
+    import torch
+    dt, op, k, n = O.BF16, O.SUM, 8, 300_000
+    ins = [make_inputs(dt, k, n, seed=60 + r) for r in range(3)]
+    devs = [[to_dev(a) for a in g] for g in ins]
+    outs = [dev_empty(n, 2, fill=0) for _ in range(6)]
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(4, k, dt, op)
+    q.set_linger(16)
+    try:
+        q.start()
+        tickets = []
+        for r in range(6):
+            tickets.append(q.enqueue_reduce([d.data_ptr() for d in devs[r % 3]], outs[r].data_ptr(), n))
+            q.wait(tickets[-1])
+            if r % 2 == 1:
+                deadline = time.time() + 30
+                while q.query()[2] != PARKED and time.time() < deadline:
+                    time.sleep(0.001)
+                assert q.query()[2] == PARKED
+                torch.cuda.synchronize()          # returns: no kernel is left on the GPU
+                p, c, _ = q.query()
+                assert p == c == r + 1
+        assert tickets == [1, 2, 3, 4, 5, 6]
+        q.stop()                                  # parked at this point
+        assert q.query() == (7, 7, STOPPED)
+        for r in range(6):
+            assert same(from_dev(outs[r], np.uint16), expect(ins[r % 3], dt, op), nan_class=True, dtype=dt), r
+            outs[r].zero_()
+        torch.cuda.synchronize()
+        with q:                                   # counters start again at zero
+            assert q.enqueue_reduce([d.data_ptr() for d in devs[0]], outs[0].data_ptr(), n) == 1
+        assert same(from_dev(outs[0], np.uint16), expect(ins[0], dt, op), nan_class=True, dtype=dt)
+    finally:
         q.close()
 
 

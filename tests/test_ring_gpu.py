@@ -104,7 +104,7 @@ def test_ring_reduce_scatter_through_the_reduce_queue(L, dt, op, nranks, rcount,
             for rep in range(2):
                 for rank in staged:
                     ring.reduce_scatter_fifo(q, send, rank, staged[rank], sa)
-                    assert q.query()[2] == 1
+                    assert q.query()[2] in (1, 4)
     finally:
         q.close()
         L.lib().flagcxLocalSetMaxSpinCount(-1)
