@@ -44,6 +44,7 @@ struct flagcxLocalReduceFifo {
   uint64_t lastAfterAll = 0;        // index of the youngest entry marked kQueueFlagAfterAll
   bool started = false;             // between Start and Stop
   bool stopSent = false;
+  uint64_t windowBytes = 256ull << 20; // traffic of the entries in work together
   int64_t linger = 64;              // idle polls of the leader before the consumer parks (0: never)
   std::mutex mu;                    // producers may be several threads
   char lastError[256] = "";
@@ -92,6 +93,7 @@ flagcxResult_t launchConsumer(flagcxLocalReduceFifo *q, uint64_t base, const cha
   a.maxSpin = asyncMaxSpin();
   a.base = base;
   a.linger = q->linger;
+  a.windowBytes = q->windowBytes;
   // LDS is reserved only to spread the resident wavefronts over the CUs (at most
   // `waves` + 2 fit on one), in whole 1280-byte allocation granules.  A fifth of
   // every CU's LDS stays free, so that other launches that need LDS (this library's
@@ -407,6 +409,15 @@ flagcxResult_t flagcxLocalReduceFifoSetLinger(flagcxLocalReduceFifo_t q, int64_t
   if (polls < 0) return qfail(q, flagcxInvalidArgument, "flagcxLocalReduceFifoSetLinger: negative");
   if (q->started) return qfail(q, flagcxInvalidUsage, "flagcxLocalReduceFifoSetLinger: the queue is started");
   q->linger = polls;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduceFifoSetWindow(flagcxLocalReduceFifo_t q, size_t bytes) {
+  if (!q) return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(q->mu);
+  if (bytes == 0) return qfail(q, flagcxInvalidArgument, "flagcxLocalReduceFifoSetWindow: zero");
+  if (q->started) return qfail(q, flagcxInvalidUsage, "flagcxLocalReduceFifoSetWindow: the queue is started");
+  q->windowBytes = bytes;
   return flagcxSuccess;
 }
 

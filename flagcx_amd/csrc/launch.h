@@ -51,7 +51,8 @@ struct alignas(128) QueueEntry {
   uint32_t tail;    // elements after it
   uint32_t k;       // number of inputs, 1..8; 0 = stop
   uint32_t flags;   // kQueueFlag*
-  uint64_t pad[4];
+  uint64_t traffic; // device copy only: (k + 1) * body bytes, written by the consumer's leader
+  uint64_t pad[3];
 };
 static_assert(sizeof(QueueEntry) == 128, "queue entries are 16 words");
 
@@ -80,6 +81,7 @@ struct QueueKernelArgs {
   int64_t maxSpin;
   uint64_t base;                 // entries finished before this launch; device counts are relative to it
   int64_t linger;                // idle polls before the consumer parks; 0 = stay until stopped
+  uint64_t windowBytes;          // traffic of the entries the workers may have in work together
 };
 
 // Launches the consumer for one element type: grid = min(occupancy, wavesPerCU) *

@@ -115,6 +115,7 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
   const uint32_t lane = threadIdx.x;
   // host counts are absolute, the device words (devProduced, progress) relative to q.base
   uint64_t forwarded = q.base, published = q.base, stopAt = ~0ull, beat = 0, produced = q.base;
+  uint64_t inWork = 0; // traffic of the entries handed out and not yet finished by every worker
   int64_t spins = 0, idle = 0;
   if (lane == 0) systemStore(q.hostHeader + kQueueState, kQueueRunning);
   for (;;) {
@@ -138,7 +139,30 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
         const uint64_t stopMask = __ballot(isCtl && (uint32_t)w == 0);
         const uint64_t waitMask = __ballot(isCtl && ((w >> 32) & kQueueFlagAfterAll) != 0);
         uint64_t upto = forwarded + 4 < produced ? forwarded + 4 : produced;
-        bool blocked = false;
+        // Workers that run far apart lose the DRAM pages and the last-level cache
+        // that neighbouring tiles share: hand out entries only while the traffic of
+        // the unfinished ones stays inside a window (two entries may always be in work,
+        // so that large entries follow one another without a gap).
+        // An entry's traffic, (k + 1) * body bytes, is kept in word 12 of its copy in
+        // the device ring for the day it retires.
+        uint64_t traffic[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          traffic[e] = laneWord(w, 16 * e + 9) * 16 * ((uint64_t)(uint32_t)laneWord(w, 16 * e + 11) + 1);
+        if (valid && word == 12) {
+          const uint32_t e = lane >> 4;
+          agentStore(reinterpret_cast<uint64_t *>(q.devEntries + i % q.capacity) + 12,
+                     e == 0 ? traffic[0] : e == 1 ? traffic[1] : e == 2 ? traffic[2] : traffic[3]);
+        }
+        uint64_t fits = forwarded, sum = inWork;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (fits == forwarded + e && fits < upto && (fits - published < 2 || sum + traffic[e] <= q.windowBytes)) {
+            sum += traffic[e];
+            fits++;
+          }
+        upto = fits;
+        bool blocked = upto <= forwarded;
         if (waitMask) {
           const uint64_t at = forwarded + ((uint64_t)(__ffsll((long long)waitMask) - 1) >> 4);
           if (at > forwarded) {
@@ -161,6 +185,9 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
         }
         waitOwnMemory(); // the entries are in the device ring before the count says so
         agentStore(q.devProduced, upto - q.base);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (forwarded + e < upto) inWork += traffic[e];
         forwarded = upto;
         spins = 0;
         if (stopping) break;
@@ -188,6 +215,11 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
       // a worker writes its progress word only after its results were acknowledged
       // by memory, so the count can go to the host as soon as it has been read
       waitOwnMemory();
+      for (uint32_t r = 0; r < ahead; r++) {
+        const uint64_t gone =
+            uniform64(agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (published + r) % q.capacity) + 12));
+        inWork = inWork > gone ? inWork - gone : 0;
+      }
       published += ahead;
       systemStore(q.hostHeader + kQueueConsumed, published);
       spins = 0;
@@ -349,9 +381,9 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
         default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nworkers); break;
       }
       rot = (uint32_t)((rot + ntiles) % nworkers);
-      // in a long run of entries let the count move every eighth entry, so that
-      // the producer's ring drains while the run is still going
-      if ((done & 7) == 0 && done < produced) {
+      // in a long run of entries let the count move every fourth entry, so that the
+      // leader's window and the producer's ring move while the run is still going
+      if ((done & 3) == 0 && done < produced) {
         waitOwnMemory();
         if (threadIdx.x == 0)
           __hip_atomic_store(q.progress + worker, (uint32_t)done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -129,7 +129,7 @@ EXPORTS = [
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
-    "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoSetLinger", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
+    "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoSetLinger", "flagcxLocalReduceFifoSetWindow", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
     "flagcxLocalReduceFifoGetLastError",
 ]
 
@@ -205,6 +205,7 @@ def lib():
         L.flagcxLocalReduceFifoGetGrid.argtypes = [vp, C.POINTER(C.c_uint)]
         L.flagcxLocalReduceFifoSetWaves.argtypes = [vp, i]
         L.flagcxLocalReduceFifoSetLinger.argtypes = [vp, C.c_int64]
+        L.flagcxLocalReduceFifoSetWindow.argtypes = [vp, sz]
         L.flagcxLocalReduceFifoGetType.argtypes = [vp, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
         L.flagcxLocalRingReduceScatterFifo.argtypes = [vp, vp, pp, i, i, vp, sz, sp]
         L.flagcxLocalReduceFifoGetLastError.restype = C.c_char_p
@@ -492,6 +493,9 @@ class ReduceFifo:
 
     def wait(self, ticket):
         self._check(lib().flagcxLocalReduceFifoWait(self._h, ticket))
+
+    def set_window(self, nbytes):
+        self._check(lib().flagcxLocalReduceFifoSetWindow(self._h, nbytes))
 
     def set_linger(self, polls):
         self._check(lib().flagcxLocalReduceFifoSetLinger(self._h, polls))

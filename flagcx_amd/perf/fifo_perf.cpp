@@ -3,7 +3,8 @@
 // the same work:
 //
 //   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
-//             [-W wavesPerCU] [-L lingerPolls] [-s spinLimit]
+//             [-W wavesPerCU] [-L lingerPolls] [-s spinLimit] [-q ringCapacity]
+//             [-D windowBytes]
 //
 // A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
 // staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
@@ -60,6 +61,8 @@ int main(int argc, char **argv) {
   long long spin = 1ll << 22;
   int tuneWaves = -1;
   long long linger = -1;
+  int capacity = 64;
+  size_t window = 0;
   for (int i = 1; i + 1 < argc; i += 2) {
     const char *f = argv[i], *v = argv[i + 1];
     if (!strcmp(f, "-k")) k = atoi(v);
@@ -72,6 +75,8 @@ int main(int argc, char **argv) {
     else if (!strcmp(f, "-s")) spin = atoll(v);
     else if (!strcmp(f, "-W")) tuneWaves = atoi(v);
     else if (!strcmp(f, "-L")) linger = atoll(v);
+    else if (!strcmp(f, "-q")) capacity = atoi(v);
+    else if (!strcmp(f, "-D")) window = strtoull(v, 0, 0);
   }
   flagcxLocalReduceFifo_t fifo = nullptr;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
@@ -126,9 +131,10 @@ int main(int argc, char **argv) {
   printf("%-46s %10.1f us  %8.1f GB/s\n", "one batch call (all chunks present), sync", median(t), algo / median(t) / 1e3);
 
   // (3) the resident consumer: enqueue chunk by chunk, wait for the last ticket
-  FX(flagcxLocalReduceFifoCreate(&fifo, 64, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op));
+  FX(flagcxLocalReduceFifoCreate(&fifo, capacity, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op));
   if (tuneWaves > 0) FX(flagcxLocalReduceFifoSetWaves(fifo, tuneWaves));
   if (linger >= 0) FX(flagcxLocalReduceFifoSetLinger(fifo, linger));
+  if (window > 0) FX(flagcxLocalReduceFifoSetWindow(fifo, window));
   FX(flagcxLocalReduceFifoStart(fifo));
   unsigned grid = 0;
   FX(flagcxLocalReduceFifoGetGrid(fifo, &grid));

@@ -416,6 +416,11 @@ flagcxResult_t flagcxLocalReduceFifoSetWaves(flagcxLocalReduceFifo_t fifo, int w
 /* What the queue was created for (any pointer may be NULL). */
 flagcxResult_t flagcxLocalReduceFifoGetType(flagcxLocalReduceFifo_t fifo, flagcxDataType_t *datatype,
                                             flagcxRedOp_t *op, int *maxRanks);
+/* Traffic, (nranks + 1) * bytes per entry, of the entries the consumer works on
+ * together beyond the oldest unfinished one (default 256 MiB, measured best: a
+ * narrow window keeps the wavefronts on neighbouring tiles and inside the
+ * last-level cache; two entries may always be in work).  Not between Start and Stop. */
+flagcxResult_t flagcxLocalReduceFifoSetWindow(flagcxLocalReduceFifo_t fifo, size_t bytes);
 /* Idle polls before the consumer parks (0: never).  Not between Start and Stop. */
 flagcxResult_t flagcxLocalReduceFifoSetLinger(flagcxLocalReduceFifo_t fifo, int64_t polls);
 /* Workgroups (one wavefront each) of the running consumer: 1 leader + workers. */

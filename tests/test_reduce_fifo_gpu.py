@@ -251,6 +251,43 @@ def test_fifo_orders_dependent_entries(L):
     assert same(from_dev(d["a"], np.int32), env["a"])
 
 
+def test_fifo_several_producer_threads(L):
+    """Four host threads append to one queue at once (a one-slot-per-thread ring, so they
+    also meet 'full'); every entry is folded exactly once into its own output."""
+    import threading
+    import torch
+    dt, op, k, n = O.FP32, O.SUM, 2, 40_003
+    nthreads, per = 4, 25
+    ins = [make_inputs(dt, k, n, seed=500 + t) for t in range(nthreads)]
+    devs = [[to_dev(a) for a in g] for g in ins]
+    outs = [[dev_empty(n, 4, fill=0) for _ in range(per)] for _ in range(nthreads)]
+    torch.cuda.synchronize()
+    errors, last = [], [0] * nthreads
+    q = L.ReduceFifo(4, k, dt, op)
+    try:
+        with q:
+            def produce(t):
+                try:
+                    for i in range(per):
+                        last[t] = q.enqueue_reduce([d.data_ptr() for d in devs[t]], outs[t][i].data_ptr(), n)
+                except Exception as e:
+                    errors.append(repr(e))
+            threads = [threading.Thread(target=produce, args=(t,)) for t in range(nthreads)]
+            for th in threads:
+                th.start()
+            for th in threads:
+                th.join(60)
+            assert not errors, errors
+            q.wait(max(last))
+            assert q.query()[:2] == (nthreads * per, nthreads * per)
+    finally:
+        q.close()
+    for t in range(nthreads):
+        want = expect(ins[t], dt, op)
+        for i in range(per):
+            assert same(from_dev(outs[t][i], np.float32), want, nan_class=True, dtype=dt), (t, i)
+
+
 def test_fifo_ring_wraps_and_restarts(L):
     """More entries than slots (the producer sees 'full' and retries), then a second
     start on the same queue with counters back at zero."""
