@@ -235,28 +235,32 @@ struct FillParams {
   uint32_t pattern;
 };
 
-// Up to two byte ranges in one launch (blockIdx.y picks the range).
-template <int U>
-__global__ void __launch_bounds__(64) fillWaveKernel(FillParams p) {
-  constexpr uint32_t kTileBytes = 64u * U * 16u;
+// Up to two byte ranges in one launch (blockIdx.y picks the range).  Unlike the
+// kernels that read, a pure store stream runs best from workgroups of four
+// wavefronts, each wavefront storing one consecutive KiB (4 GiB on MI355X:
+// 90 % of the HBM peak, against 60 % from one-wavefront workgroups of one KiB and
+// 81 % from one-wavefront workgroups of four).
+constexpr int kFillWaves = 4;
+__global__ void __launch_bounds__(64 * kFillWaves) fillWaveKernel(FillParams p) {
+  constexpr uint32_t kTileBytes = 1024u;
   const int r = blockIdx.y;
   char *base = p.ptr[r] + p.head[r];
   const uint64_t body = p.body[r];
   const uint64_t ntiles = (body + kTileBytes - 1) / kTileBytes;
-  const uint32_t voff = threadIdx.x * 16u;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t voff = lane * 16u;
   const u32x4 v = {p.pattern, p.pattern, p.pattern, p.pattern};
-  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+  for (uint64_t t = (uint64_t)blockIdx.x * kFillWaves + wave; t < ntiles; t += (uint64_t)gridDim.x * kFillWaves) {
     const uint64_t off = t * kTileBytes;
     const uint64_t left = body - off;
     const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
     __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void *)(base + off), 0, span, kRsrcFlags);
-#pragma unroll
-    for (int u = 0; u < U; u++) __builtin_amdgcn_raw_buffer_store_b128(v, rd, voff + u * 1024u, 0, kStoreAux);
+    __builtin_amdgcn_raw_buffer_store_b128(v, rd, voff, 0, kStoreAux);
   }
-  if (blockIdx.x == gridDim.x - 1) {
+  if (blockIdx.x == gridDim.x - 1 && wave == 0) {
     const uint64_t edge = p.head[r] + p.tail[r];
-    if (threadIdx.x < edge) {
-      const uint64_t i = threadIdx.x < p.head[r] ? threadIdx.x : p.head[r] + body + (threadIdx.x - p.head[r]);
+    if (lane < edge) {
+      const uint64_t i = lane < p.head[r] ? lane : p.head[r] + body + (lane - p.head[r]);
       p.ptr[r][i] = (char)(p.pattern & 0xffu);
     }
   }
@@ -282,12 +286,11 @@ int launchFill(void *p0, uint64_t n0, void *p1, uint64_t n1, int value, hipStrea
   if (nr == 0) return (int)hipSuccess;
   const uint32_t b = (uint32_t)(value & 0xff);
   p.pattern = b | (b << 8) | (b << 16) | (b << 24);
-  constexpr int U = 4;
-  constexpr uint64_t tileBytes = 64ull * U * 16ull;
-  uint64_t gx = (maxBody + tileBytes - 1) / tileBytes;
+  constexpr uint64_t groupBytes = 1024ull * kFillWaves;
+  uint64_t gx = (maxBody + groupBytes - 1) / groupBytes;
   if (gx < 1) gx = 1;
   if (gx > kMaxGridX) gx = kMaxGridX;
-  fillWaveKernel<U><<<dim3((unsigned)gx, (unsigned)nr), dim3(64), 0, stream>>>(p);
+  fillWaveKernel<<<dim3((unsigned)gx, (unsigned)nr), dim3(64 * kFillWaves), 0, stream>>>(p);
   return (int)hipGetLastError();
 }
 

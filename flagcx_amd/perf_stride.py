@@ -19,7 +19,7 @@ from flagcx_amd import local as L
 MiB = 1 << 20
 STRIDES = [128 * MiB, 128 * MiB + 4096, 128 * MiB + 65536, 129 * MiB + 4096, 256 * MiB, 512 * MiB,
            1024 * MiB, 1024 * MiB + 4096, 1024 * MiB + 65536, 1025 * MiB, 1026 * MiB + 8192, 1057 * MiB + 12288]
-CAPS = [8, 10, 12, 14, 16, 20, 24, 0]
+CAPS = [8, 10, 12, 14, 16, 18, 21, 25, 0]   # caps that whole LDS granules can express
 
 
 def main():
