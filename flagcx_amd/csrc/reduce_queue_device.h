@@ -79,6 +79,12 @@ __device__ __forceinline__ uint32_t waveMin32(uint32_t v) {
   return v;
 }
 
+__device__ __forceinline__ uint64_t waveSum64(uint64_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
 // Word `word` of a value every lane holds for the queue word (lane & 15).
 __device__ __forceinline__ uint64_t laneWord(uint64_t v, int word) {
   const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)v, word);
@@ -166,7 +172,7 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
         if (waitMask) {
           const uint64_t at = forwarded + ((uint64_t)(__ffsll((long long)waitMask) - 1) >> 4);
           if (at > forwarded) {
-            upto = at; // what precedes it goes out now, the entry itself in a later round
+            if (upto > at) upto = at; // what precedes it goes out now, the entry itself in a later round
           } else if (published < at) {
             blocked = true; // its predecessors are still in flight
           } else {
@@ -215,13 +221,18 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
       // a worker writes its progress word only after its results were acknowledged
       // by memory, so the count can go to the host as soon as it has been read
       waitOwnMemory();
-      for (uint32_t r = 0; r < ahead; r++) {
-        const uint64_t gone =
-            uniform64(agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (published + r) % q.capacity) + 12));
-        inWork = inWork > gone ? inWork - gone : 0;
+      systemStore(q.hostHeader + kQueueConsumed, published + ahead);
+      // the finished entries leave the traffic window (one lane per entry)
+      uint64_t gone = 0;
+      for (uint32_t r0 = 0; r0 < ahead; r0 += 64) {
+        uint64_t mine = 0;
+        if (r0 + lane < ahead)
+          mine = agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (published + r0 + lane) % q.capacity) + 12);
+        gone += waveSum64(mine);
       }
+      gone = uniform64(gone);
+      inWork = inWork > gone ? inWork - gone : 0;
       published += ahead;
-      systemStore(q.hostHeader + kQueueConsumed, published);
       spins = 0;
     }
     if (stopAt != ~0ull && published > stopAt) {
