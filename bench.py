@@ -37,7 +37,7 @@ ALGO_BYTES = (K + 1) * N_ELEM * 2   # k reads + 1 write
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/reduce8_bf16_sum_256MiB_pmc.txt), scaled by a copy kernel of known size.
-MEASURED_TRAFFIC_BYTES = 2415727813
+MEASURED_TRAFFIC_BYTES = 2415853564
 
 
 def log(*a):
@@ -72,6 +72,8 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=32 * 1024 * 1024,
                     help="elements per input the CPU baseline reduces")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--allocator-layout", action="store_true",
+                    help="inputs and output as separate torch allocations instead of placed in one")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also run N flagcxLocalMemcpy launches of 256 MiB (a copy of known size "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -89,13 +91,27 @@ def main():
     torch.cuda.set_device(0)
     L.check(L.lib().flagcxLocalInit())
 
+    # The 8 input buffers and the output live in one allocation, at the addresses
+    # flagcxLocalPlaceBuffers gives: equal offsets into them fall into different HBM
+    # channel groups, which is how a caller that owns the ranks' staging buffers would
+    # lay them out.  --allocator-layout takes nine separate torch allocations instead
+    # (258 MiB apart on this allocator: all in one channel group).
+    nbytes = N_ELEM * 2
+    if args.allocator_layout:
+        bufs = [torch.empty(N_ELEM, dtype=torch.bfloat16, device="cuda") for _ in range(K + 1)]
+        layout = "nine separate torch allocations"
+    else:
+        pool_bytes = (K + 1) * (nbytes + 128 * 1024)
+        pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+        addrs = L.place_buffers(pool.data_ptr(), pool_bytes, nbytes, K + 1)
+        bufs = [pool[a - pool.data_ptr(): a - pool.data_ptr() + nbytes].view(torch.bfloat16) for a in addrs]
+        layout = "one allocation, buffers placed by flagcxLocalPlaceBuffers"
     # seeded synthetic inputs: N(0,1) per input from seeds 0..7, rounded to bf16
-    inputs = []
+    inputs = bufs[:K]
+    out = bufs[K]
     for seed in range(K):
         g = torch.Generator(device="cuda").manual_seed(seed)
-        x = torch.randn(N_ELEM, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
-        inputs.append(x)
-    out = torch.empty(N_ELEM, dtype=torch.bfloat16, device="cuda")
+        inputs[seed].copy_(torch.randn(N_ELEM, generator=g, device="cuda", dtype=torch.float32))
     torch.cuda.synchronize()
 
     def step():
@@ -178,7 +194,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "8-input bf16 sum reduce, fp32 accumulation, 256 MiB per input buffer "
                                "(128Mi elements), N(0,1) from seeds 0..7",
-                   "nranks": K, "elements": N_ELEM, "bytes_per_step": ALGO_BYTES, "accumulate": "fp32"},
+                   "nranks": K, "elements": N_ELEM, "bytes_per_step": ALGO_BYTES, "accumulate": "fp32",
+                   "buffers": layout},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,

@@ -26,9 +26,11 @@ struct DeviceInfo {
 };
 const DeviceInfo &deviceInfo();
 
-// Resident single-wave workgroups per CU for a k-input reduce (k = 0: copies).
-int wavesPerCUFor(int k);
+// Resident single-wave workgroups per CU for a k-input reduce (k = 0: copies);
+// `spread`: the inputs' addresses fall into different HBM channel groups.
+int wavesPerCUFor(int k, bool spread = true);
 void setWavesPerCU(int k, int waves);
+bool inputsSpread(const void *const *src, int k);
 
 // LDS bytes to reserve per workgroup so that at most `waves` one-wave workgroups
 // fit on a CU.  0 when no cap is wanted.

@@ -82,7 +82,7 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   uint64_t tiles = (s.nvec * 16 + tileBytes - 1) / tileBytes;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  const int lds = ldsReservation(wavesPerCUFor(K));
+  const int lds = ldsReservation(wavesPerCUFor(K, inputsSpread(c.src, K)));
   reduceWaveKernel<elem_t, OP, K, U><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
   return (int)hipGetLastError();
 }
@@ -100,7 +100,7 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  const int lds = ldsReservation(wavesPerCUFor(c.k > 8 ? 8 : c.k));
+  const int lds = ldsReservation(wavesPerCUFor(c.k > 8 ? 8 : c.k, inputsSpread(c.src, c.k)));
   if (s.vector)
     reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
   else
@@ -146,7 +146,7 @@ static int launchBatchFixed(const ReduceCall *calls, const Split *splits, int n)
       if (tiles > maxTiles) maxTiles = tiles;
     }
     if (maxTiles > kMaxGrid) maxTiles = kMaxGrid;
-    const int lds = ldsReservation(wavesPerCUFor(K));
+    const int lds = ldsReservation(wavesPerCUFor(K, inputsSpread(calls[base].src, K)));
     reduceBatchKernel<elem_t, OP, K, U>
         <<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, calls[0].stream>>>(bp);
     const int err = (int)hipGetLastError();

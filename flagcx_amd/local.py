@@ -114,7 +114,7 @@ class CopyArgs(C.Structure):         # flagcxLocalCopyArgs
 
 EXPORTS = [
     "flagcxLocalGetDataTypeSize", "flagcxLocalInit", "flagcxLocalGetErrorString", "flagcxLocalGetLastError",
-    "flagcxLocalTune", "flagcxLocalGetTune", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
+    "flagcxLocalTune", "flagcxLocalGetTune", "flagcxLocalPlaceBuffers", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
     "flagcxLocalAllReduce", "flagcxLocalRingChunkTable", "flagcxLocalMemcpy", "flagcxLocalMemset",
     "flagcxLocalRefresh", "flagcxLocalPack", "flagcxLocalUnpack", "flagcxLocalPackList",
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
@@ -155,6 +155,7 @@ def lib():
         L.flagcxLocalGetErrorString.argtypes = [i]
         L.flagcxLocalGetLastError.restype = C.c_char_p
         L.flagcxLocalTune.argtypes = [i, i]
+        L.flagcxLocalPlaceBuffers.argtypes = [vp, sz, sz, i, pp]
         L.flagcxLocalGetTune.argtypes = [i, C.POINTER(i)]
         L.flagcxLocalReduce.argtypes = [pp, i, vp, sz, i, i, sp]
         L.flagcxLocalReduceScatter.argtypes = [pp, i, i, vp, sz, i, i, sp]
@@ -260,6 +261,13 @@ def _sref(stream):
 
 def _ptr_array(ptrs):
     return (C.c_void_p * len(ptrs))(*ptrs)
+
+
+def place_buffers(pool_ptr, pool_bytes, nbytes, n):
+    """Addresses for n buffers of nbytes inside the pool, in different HBM channel groups."""
+    out = (C.c_void_p * n)()
+    check(lib().flagcxLocalPlaceBuffers(pool_ptr, pool_bytes, nbytes, n, out))
+    return [int(p) for p in out]
 
 
 def reduce(srcs, dst, op, dtype=None, count=None, stream="current"):

@@ -5,9 +5,9 @@ cap on resident wavefronts per CU (flagcxLocalTune):
 
 The inputs are slices of one allocation, `stride` bytes apart (128 MiB .. 1 GiB plus
 small offsets), so their addresses alias differently in the HBM channel hash.  For
-each stride the table gives percent of the 8 TB/s peak for several caps; the last
-line gives, per cap, the worst and best stride - the shipped default is the cap
-whose worst case is best.
+each stride the table gives percent of the 8 TB/s peak for several caps and for the
+library's own per-launch choice ("auto"); the last line gives the worst and best
+stride per column.
 """
 import argparse
 import sys
@@ -19,7 +19,7 @@ from flagcx_amd import local as L
 MiB = 1 << 20
 STRIDES = [128 * MiB, 128 * MiB + 4096, 128 * MiB + 65536, 129 * MiB + 4096, 256 * MiB, 512 * MiB,
            1024 * MiB, 1024 * MiB + 4096, 1024 * MiB + 65536, 1025 * MiB, 1026 * MiB + 8192, 1057 * MiB + 12288]
-CAPS = [8, 10, 12, 14, 16, 18, 21, 25, 0]   # caps that whole LDS granules can express
+CAPS = [8, 10, 12, 14, 16, 18, 21, 25, 0, -1]   # caps that whole LDS granules can express; -1 = the library's choice
 
 
 def main():
@@ -43,7 +43,7 @@ def main():
     big.view(torch.int16 if esz == 2 else torch.int32).random_(0, 1000)
     out = torch.empty(n, dtype=tdt, device="cuda")
     print("k=%d %s, %d MiB per input; percent of 8 TB/s, (k+1)*bytes/time" % (k, args.dtype, args.mib))
-    print("%14s " % "stride" + " ".join("%7s" % ("cap %d" % c if c else "no cap") for c in CAPS))
+    print("%14s " % "stride" + " ".join("%7s" % ("cap %d" % c if c > 0 else "no cap" if c == 0 else "auto") for c in CAPS))
     worst = {c: 100.0 for c in CAPS}
     best = {c: 0.0 for c in CAPS}
     for st in STRIDES:
@@ -67,7 +67,7 @@ def main():
             row.append("%7.1f" % pct)
         print("%14d " % st + " ".join(row), flush=True)
     L.check(L.lib().flagcxLocalTune(k, default_cap))
-    print("shipped cap for k=%d: %d" % (k, default_cap))
+    print("setting found for k=%d: %d (-1 = chosen per launch from the inputs' addresses)" % (k, default_cap))
     print("%14s " % "worst..best" + " ".join("%3.0f..%-3.0f" % (worst[c], best[c]) for c in CAPS))
     return 0
 

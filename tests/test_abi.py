@@ -112,6 +112,7 @@ def test_other_entry_points_reject_bad_arguments():
     assert L.flagcxLocalPackList(a, ptrs, 2, 16, st) == inv                     # dst overlaps a source
     assert L.flagcxLocalTune(9, 8) == inv
     assert L.flagcxLocalTune(8, 8) == 0
+    assert L.flagcxLocalTune(8, -1) == 0   # back to the per-launch choice
     # zero sizes succeed without a launch
     assert L.flagcxLocalMemcpy(b, a, 0, st) == 0
     assert L.flagcxLocalPack(b, a, 0, 64, 64, st) == 0
@@ -168,6 +169,30 @@ def test_reduce_fifo_entry_points_validate_without_a_device():
     assert L.flagcxLocalReduceFifoWait(None, 1) == inv
     assert L.flagcxLocalReduceFifoStop(None) == inv
     assert L.flagcxLocalReduceFifoDestroy(None) == 0
+
+
+def test_place_buffers_spreads_over_channel_groups():
+    """Host-only helper: addresses inside the pool, in order, KiB aligned, every buffer in a
+    channel group of its own, eight consecutive ones differing in the low three hash bits."""
+    group = lambda a: ((a >> 10) ^ (a >> 18) ^ (a >> 25)) & 31
+    for base, nbytes, n in ((0x7f1234567001, 256 << 20, 9), (0x10000000, 4 << 20, 8), (0x4ff751600000, 1000, 32),
+                            (0x20000400, 1 << 30, 2)):
+        pool_bytes = n * (nbytes + 64 * 1024) + 1024
+        addrs = local.place_buffers(base, pool_bytes, nbytes, n)
+        assert len(addrs) == n and all(a % 1024 == 0 for a in addrs)
+        assert addrs[0] >= base and addrs[-1] + nbytes <= base + pool_bytes
+        assert all(addrs[i] + nbytes <= addrs[i + 1] for i in range(n - 1))
+        assert all(addrs[i + 1] - addrs[i] - nbytes <= 64 * 1024 + 1024 for i in range(n - 1))
+        assert len({group(a) for a in addrs}) == n
+        for i in range(0, n - 7, 8):
+            assert sorted(group(a) & 7 for a in addrs[i:i + 8]) == list(range(8))
+    L = local.lib()
+    out = (C.c_void_p * 4)()
+    inv = int(local.Result.InvalidArgument)
+    assert L.flagcxLocalPlaceBuffers(0x1000, 4096, 4096, 4, out) == inv          # pool too small
+    assert L.flagcxLocalPlaceBuffers(None, 1 << 20, 16, 4, out) == inv
+    assert L.flagcxLocalPlaceBuffers(0x1000, 1 << 20, 16, 33, out) == inv
+    assert L.flagcxLocalPlaceBuffers(0x1000, 1 << 20, 16, 4, None) == inv
 
 
 def test_error_strings():
