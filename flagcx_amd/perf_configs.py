@@ -7,7 +7,8 @@
       launch, and 32 launches of 4 MiB chunks (the staging ring's step size)
   C4  4-input int32 max and min, 512 MiB per buffer
 5 warm-up + 20 timed iterations (test/perf/tools.cc:81-86), HIP events, back-to-back
-launches per iteration.  GB/s = (k+1) * n * size / time.  --cpu also times the CPU
+launches per iteration.  GB/s = (k+1) * n * size / time.  The ranks' buffers of C3 and
+the buffers of C4 sit in one allocation each, at the addresses flagcxLocalPlaceBuffers gives.  --cpu also times the CPU
 oracle (test infrastructure, imported only under this flag) on bounded samples.
 """
 import argparse
@@ -33,6 +34,18 @@ def timed(fn, warmup=5, iters=20):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / iters   # ms
+
+
+def placed(count, nelem, dtype):
+    """`count` tensors of nelem elements inside one allocation, at the addresses
+    flagcxLocalPlaceBuffers gives (different HBM channel groups); the pool is returned
+    too so that it stays alive."""
+    esz = torch.empty(0, dtype=dtype).element_size()
+    nbytes = nelem * esz
+    pool_bytes = count * (nbytes + 128 * 1024)
+    pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    base = pool.data_ptr()
+    return [pool[a - base: a - base + nbytes].view(dtype) for a in L.place_buffers(base, pool_bytes, nbytes, count)], pool
 
 
 def main():
@@ -64,13 +77,11 @@ def main():
     # C3
     nranks, per_rank = 8, 512 * MiB
     shard = per_rank // nranks
-    send = []
+    send, send_pool = placed(nranks, per_rank, torch.float16)   # the ranks' buffers, in different channel groups
     for r in range(nranks):
         g = torch.Generator(device="cuda").manual_seed(100 + r)
-        buf = torch.empty(per_rank, dtype=torch.float16, device="cuda")
         for s in range(nranks):
-            buf[s * shard:(s + 1) * shard] = (torch.randn(shard, generator=g, device="cuda") * 0.01).to(torch.float16)
-        send.append(buf)
+            send[r][s * shard:(s + 1) * shard] = (torch.randn(shard, generator=g, device="cuda") * 0.01).to(torch.float16)
     recv = torch.empty(shard, dtype=torch.float16, device="cuda")
     nb = 9 * shard * 2
     ms = timed(lambda: L.reduce_scatter(send, 3, recv, L.RedOp.Avg))
@@ -132,13 +143,15 @@ def main():
             L.reduce_scatter(send, rk, recv, L.RedOp.Avg)
     ms = timed(all_shards, warmup=2, iters=5)
     report("C3 all 8 shards (8 fused launches, 1 GiB out)", 8 * nb, ms)
-    del send, recv
+    del send, recv, send_pool
 
     # C4
     n = 128 * MiB
     g = torch.Generator(device="cuda").manual_seed(3)
-    ins = [torch.randint(-2**31, 2**31 - 1, (n,), generator=g, device="cuda", dtype=torch.int32) for _ in range(4)]
-    out = torch.empty(n, dtype=torch.int32, device="cuda")
+    bufs, c4_pool = placed(5, n, torch.int32)
+    ins, out = bufs[:4], bufs[4]
+    for t in ins:
+        t.copy_(torch.randint(-2**31, 2**31 - 1, (n,), generator=g, device="cuda", dtype=torch.int32))
     for op, nm in ((L.RedOp.Max, "max"), (L.RedOp.Min, "min")):
         ms = timed(lambda: L.reduce(ins, out, op))
         report("C4 4x int32 %s 512 MiB" % nm, 5 * n * 4, ms)
