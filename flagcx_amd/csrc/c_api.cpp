@@ -59,7 +59,7 @@ const DeviceInfo &deviceInfo() {
 // different channel groups, `aliased` when they collide (K = 8: 87-88 % of peak at
 // 8 when spread; 78-82 % at 8 but 81-83 % at 16 when aliased).  Up to four inputs
 // one value serves both.
-static const int kWavesSpread[9] = {0, 0, 25, 14, 11, 10, 10, 10, 8};
+static const int kWavesSpread[9] = {0, 0, 25, 14, 11, 10, 9, 8, 8};
 static const int kWavesAliased[9] = {0, 0, 25, 14, 11, 10, 18, 16, 16};
 // explicit settings (flagcxLocalTune); -1 = choose from the tables above
 static std::atomic<int> gWaves[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
