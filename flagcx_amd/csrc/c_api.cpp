@@ -56,11 +56,12 @@ const DeviceInfo &deviceInfo() {
 // unless the K loads of a wavefront all land in the same channel group, in which
 // case their latencies add up and more wavefronts are needed to cover them.  So
 // there are two columns: `spread` when the inputs' addresses fall into (nearly) K
-// different channel groups, `aliased` when they collide (K = 8: 87-88 % of peak at
-// 8 when spread; 78-82 % at 8 but 81-83 % at 16 when aliased).  Up to four inputs
-// one value serves both.
+// different channel groups, `aliased` when they collide; aliased launches also pace
+// their loads (reduce_device.h), which wants more wavefronts still (K = 8: 87-88 %
+// of peak at 8 when spread; aliased 78-82 % at 8, 81-83 % at 16, 85-86 % paced at
+// 18).  Up to four inputs one value serves both.
 static const int kWavesSpread[9] = {0, 0, 25, 14, 11, 10, 9, 8, 8};
-static const int kWavesAliased[9] = {0, 0, 25, 14, 11, 10, 18, 16, 16};
+static const int kWavesAliased[9] = {0, 0, 25, 14, 11, 21, 21, 18, 18};
 // explicit settings (flagcxLocalTune); -1 = choose from the tables above
 static std::atomic<int> gWaves[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
 
