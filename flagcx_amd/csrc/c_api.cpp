@@ -59,9 +59,10 @@ const DeviceInfo &deviceInfo() {
 // different channel groups, `aliased` when they collide; aliased launches also pace
 // their loads (reduce_device.h), which wants more wavefronts still (K = 8: 87-88 %
 // of peak at 8 when spread; aliased 78-82 % at 8, 81-83 % at 16, 85-86 % paced at
-// 18).  Up to four inputs one value serves both.
+// 18; pacing gains nothing up to four inputs).  Up to three inputs one value
+// serves both.
 static const int kWavesSpread[9] = {0, 0, 25, 14, 11, 10, 9, 8, 8};
-static const int kWavesAliased[9] = {0, 0, 25, 14, 11, 21, 21, 18, 18};
+static const int kWavesAliased[9] = {0, 0, 25, 14, 10, 21, 21, 18, 18};
 // explicit settings (flagcxLocalTune); -1 = choose from the tables above
 static std::atomic<int> gWaves[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
 
@@ -90,7 +91,7 @@ static inline unsigned channelGroupOf(const void *p) {
 }
 
 bool inputsSpread(const void *const *src, int k) {
-  if (k < 5) return true; // one table value serves both cases
+  if (k < 4) return true; // one table value serves both cases
   const int n = k < 8 ? k : 8;
   uint32_t seen = 0;
   int distinct = 0, middle = 0;

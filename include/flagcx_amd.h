@@ -142,7 +142,7 @@ flagcxResult_t flagcxLocalPlaceBuffers(void *pool, size_t poolbytes, size_t byte
  * how many one-wavefront workgroups may share a CU for a reduce of `nranks`
  * inputs (1..8; 0 selects the copy kernels).  wavesPerCU == 0 removes the cap,
  * -1 (the default, and what GetTune then reports) lets every launch choose from
- * the values measured on MI355X: for five or more inputs it looks at whether
+ * the values measured on MI355X: for four or more inputs it looks at whether
  * their addresses fall into different HBM channel groups (few wavefronts are
  * best) or collide (more are needed).  Process-wide. */
 flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU);
