@@ -4,7 +4,7 @@
 //
 //   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
 //             [-W wavesPerCU] [-L lingerPolls] [-s spinLimit] [-q ringCapacity]
-//             [-D windowBytes]
+//             [-D windowBytes] [-a separateAllocations]
 //
 // A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
 // staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
@@ -61,7 +61,7 @@ int main(int argc, char **argv) {
   long long spin = 1ll << 22;
   int tuneWaves = -1;
   long long linger = -1;
-  int capacity = 64;
+  int capacity = 64, separate = 0;
   size_t window = 0;
   for (int i = 1; i + 1 < argc; i += 2) {
     const char *f = argv[i], *v = argv[i + 1];
@@ -77,6 +77,7 @@ int main(int argc, char **argv) {
     else if (!strcmp(f, "-L")) linger = atoll(v);
     else if (!strcmp(f, "-q")) capacity = atoi(v);
     else if (!strcmp(f, "-D")) window = strtoull(v, 0, 0);
+    else if (!strcmp(f, "-a")) separate = atoi(v);
   }
   flagcxLocalReduceFifo_t fifo = nullptr;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
@@ -85,13 +86,19 @@ int main(int argc, char **argv) {
   flagcxLocalSetMaxSpinCount(spin); // an idle consumer leaves after this many polls
   const size_t shardBytes = chunkBytes * (size_t)nchunks;
   const size_t chunkCount = chunkBytes / ts;
-  std::vector<void *> src(k);
-  void *dst = nullptr;
-  for (int j = 0; j < k; j++) {
-    CK(hipMalloc(&src[j], shardBytes));
-    CK(hipMemset(src[j], 0, shardBytes)); // zeros are valid in every type; timing does not depend on values
+  // the k inputs and the output in one allocation, in different HBM channel groups
+  // (-a 1: k + 1 separate allocations instead, wherever the allocator puts them)
+  std::vector<void *> src(k + 1);
+  void *pool = nullptr;
+  if (separate) {
+    for (int j = 0; j <= k; j++) CK(hipMalloc(&src[j], shardBytes));
+  } else {
+    const size_t poolBytes = (size_t)(k + 1) * (shardBytes + 128 * 1024);
+    CK(hipMalloc(&pool, poolBytes));
+    FX(flagcxLocalPlaceBuffers(pool, poolBytes, shardBytes, k + 1, src.data()));
   }
-  CK(hipMalloc(&dst, shardBytes));
+  for (int j = 0; j <= k; j++) CK(hipMemset(src[j], 0, shardBytes)); // zeros are valid in every type
+  void *dst = src[k];
   flagcxStream st;
   CK(hipStreamCreateWithFlags(&st.base, hipStreamNonBlocking));
   CK(hipDeviceSynchronize());
@@ -194,7 +201,9 @@ int main(int argc, char **argv) {
          "launch -> stream sync %.2f us\n", fifoLat, parkedLat, median(t));
   FX(flagcxLocalReduceFifoDestroy(fifo));
   fifo = nullptr;
-  for (int j = 0; j < k; j++) CK(hipFree(src[j]));
-  CK(hipFree(dst));
+  if (separate)
+    for (int j = 0; j <= k; j++) CK(hipFree(src[j]));
+  else
+    CK(hipFree(pool));
   return 0;
 }
