@@ -173,7 +173,7 @@ def test_reduce_fifo_entry_points_validate_without_a_device():
 
 def test_place_buffers_spreads_over_channel_groups():
     """Host-only helper: addresses inside the pool, in order, KiB aligned, every buffer in a
-    channel group of its own, eight consecutive ones differing in the low three hash bits."""
+    channel group of its own, eight consecutive ones differing in the upper three hash bits."""
     group = lambda a: ((a >> 10) ^ (a >> 18) ^ (a >> 25)) & 31
     for base, nbytes, n in ((0x7f1234567001, 256 << 20, 9), (0x10000000, 4 << 20, 8), (0x4ff751600000, 1000, 32),
                             (0x20000400, 1 << 30, 2)):
@@ -185,7 +185,7 @@ def test_place_buffers_spreads_over_channel_groups():
         assert all(addrs[i + 1] - addrs[i] - nbytes <= 64 * 1024 + 1024 for i in range(n - 1))
         assert len({group(a) for a in addrs}) == n
         for i in range(0, n - 7, 8):
-            assert sorted(group(a) & 7 for a in addrs[i:i + 8]) == list(range(8))
+            assert sorted((group(a) >> 2) & 7 for a in addrs[i:i + 8]) == list(range(8))
     L = local.lib()
     out = (C.c_void_p * 4)()
     inv = int(local.Result.InvalidArgument)
