@@ -30,6 +30,7 @@ const DeviceInfo &deviceInfo();
 // `spread`: the inputs' addresses fall into different HBM channel groups.
 int wavesPerCUFor(int k, bool spread = true);
 void setWavesPerCU(int k, int waves);
+int tunedWavesPerCU(int k); // the explicit setting, or -1
 bool inputsSpread(const void *const *src, int k);
 
 // LDS bytes to reserve per workgroup so that at most `waves` one-wave workgroups

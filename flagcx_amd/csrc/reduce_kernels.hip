@@ -106,7 +106,13 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  const int lds = ldsReservation(wavesPerCUFor(c.k > 8 ? 8 : c.k, inputsSpread(c.src, c.k)));
+  // more than eight inputs are loaded eight at a time; measured on MI355X: 9..10
+  // inputs want 12 wavefronts per CU (88 % of peak against 79 % at 8), 11..13 want
+  // 10, more want 8 (85-86 %).  An explicit flagcxLocalTune(8, n) overrides.
+  int waves = c.k > 8 ? tunedWavesPerCU(8) : -1;
+  if (c.k <= 8) waves = wavesPerCUFor(c.k, inputsSpread(c.src, c.k));
+  else if (waves < 0) waves = c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
+  const int lds = ldsReservation(waves);
   if (s.vector)
     reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
   else
