@@ -167,6 +167,50 @@ def test_c5_sweep_reduce2_and_strided_pack_unpack(L, log2):
     assert bool((bv[:, ce:] == -3.0).all())
 
 
+@pytest.mark.parametrize("k,dt,op", [(8, O.BF16, O.SUM), (6, O.FP16, O.AVG), (5, O.INT32, O.MAX), (4, O.FP32, O.SUM)],
+                         ids=lambda v: str(v))
+def test_placed_and_aliased_layouts_give_the_same_bytes(L, k, dt, op):
+    """Launch shape depends on where the inputs sit: buffers placed in different HBM channel
+    groups take few wavefronts per CU, buffers that all start in one group take more and
+    space their loads out.  Large enough for both shapes to be the ones chosen (64 MiB per
+    input); both results equal the oracle's bit for bit."""
+    import torch
+    from tests.util import make_inputs
+    npdt = np.dtype(O.NP_OF[dt])
+    nbytes = 64 * MiB
+    n = nbytes // npdt.itemsize
+    hosts = make_inputs(dt, k, n, seed=900 + k, op=op)
+    rc, want = O.reduce(hosts, dt, op)
+    assert rc == 0
+    carrier = {2: torch.int16, 4: torch.int32}[npdt.itemsize]
+    group = lambda a: ((a >> 10) ^ (a >> 18) ^ (a >> 25)) & 31
+    # placed: one pool, addresses from the library
+    pool_bytes = (k + 1) * (nbytes + 128 * 1024)
+    pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    base = pool.data_ptr()
+    addrs = L.place_buffers(base, pool_bytes, nbytes, k + 1)
+    assert len({group(a) for a in addrs}) == k + 1
+    placed = [pool[a - base: a - base + nbytes].view(carrier) for a in addrs]
+    # aliased: one pool, inputs 258 MiB apart (equal channel group; where a caching allocator puts 256 MiB buffers)
+    stride = 258 * MiB
+    pool2 = torch.empty(k * stride + nbytes, dtype=torch.uint8, device="cuda")
+    base2 = (pool2.data_ptr() + 1023) & ~1023
+    addrs2 = [base2 + j * stride for j in range(k)]
+    assert len({group(a) for a in addrs2}) <= 2
+    aliased = [pool2[a - pool2.data_ptr(): a - pool2.data_ptr() + nbytes].view(carrier) for a in addrs2]
+    out2 = torch.empty(n, dtype=carrier, device="cuda")
+    for j in range(k):
+        src = torch.from_numpy(hosts[j].view(np.dtype("int%d" % (8 * npdt.itemsize)))).cuda()
+        placed[j].copy_(src)
+        aliased[j].copy_(src)
+    L.reduce(placed[:k], placed[k], op, dtype=dt)
+    L.reduce(aliased, out2, op, dtype=dt)
+    torch.cuda.synchronize()
+    nan_ok = dt in (O.BF16, O.FP16, O.FP32) and op in (O.SUM, O.AVG)
+    for got in (placed[k], out2):
+        assert same(got.cpu().numpy().view(npdt), want, nan_class=nan_ok, dtype=dt)
+
+
 def test_buffers_beyond_4GiB(L):
     """Counts and byte offsets past 2^32: reduce, copy, fill and strided pack."""
     import torch
