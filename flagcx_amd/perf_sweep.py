@@ -9,6 +9,7 @@ Per size S (bytes per buffer):
   pack      8 chunks of S/8 at stride S gathered contiguous  2*S
   unpack    the inverse scatter                              2*S
   memcpy    contiguous device-to-device copy                 2*S
+  memset    byte fill (the zero-fill of a refresh)           S
 Times are HIP-event medians per launch; GB/s uses the algorithmic bytes.
 Small sizes are cache resident; from a few hundred MiB on the data streams from HBM.
 """
@@ -68,8 +69,9 @@ def main():
     g = torch.Generator(device="cuda").manual_seed(0)
     rows = []
     size = args.min
-    print("%12s %10s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %8s" %
-          ("bytes", "", "reduce2us", "GB/s", "pack us", "GB/s", "unpack us", "GB/s", "memcpy us", "GB/s", "b2b us"))
+    print("%12s %10s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %8s" %
+          ("bytes", "", "reduce2us", "GB/s", "pack us", "GB/s", "unpack us", "GB/s", "memcpy us", "GB/s",
+           "memset us", "GB/s", "b2b us"))
     while size <= args.max:
         n = size // 4
         a = torch.rand(n, device="cuda", generator=g) * 2 - 1
@@ -84,20 +86,23 @@ def main():
         pk = lambda: lib.flagcxLocalPack(staged.data_ptr(), sparse.data_ptr(), 8, chunk, size, sref)
         up = lambda: lib.flagcxLocalUnpack(sparse.data_ptr(), staged.data_ptr(), 8, chunk, size, sref)
         cp = lambda: lib.flagcxLocalMemcpy(c.data_ptr(), a.data_ptr(), size, sref)
-        assert red() == 0 and pk() == 0 and up() == 0 and cp() == 0
+        ms = lambda: lib.flagcxLocalMemset(c.data_ptr(), 0, size, sref)
+        assert red() == 0 and pk() == 0 and up() == 0 and cp() == 0 and ms() == 0
         r_med, _ = timed(red)
         p_med, _ = timed(pk)
         u_med, _ = timed(up)
         c_med, _ = timed(cp)
+        m_med, _ = timed(ms)
         b2b = back_to_back(red, 1000 if size <= (1 << 20) else 50)
         row = {"bytes": size, "reduce2_us": r_med, "reduce2_gbps": 3 * size / r_med / 1e3,
                "pack_us": p_med, "pack_gbps": 2 * size / p_med / 1e3,
                "unpack_us": u_med, "unpack_gbps": 2 * size / u_med / 1e3,
-               "memcpy_us": c_med, "memcpy_gbps": 2 * size / c_med / 1e3, "reduce2_b2b_us": b2b}
+               "memcpy_us": c_med, "memcpy_gbps": 2 * size / c_med / 1e3,
+               "memset_us": m_med, "memset_gbps": size / m_med / 1e3, "reduce2_b2b_us": b2b}
         rows.append(row)
-        print("%12d %10s | %9.2f %9.1f | %9.2f %9.1f | %9.2f %9.1f | %9.2f %9.1f | %8.2f" %
+        print("%12d %10s | %9.2f %9.1f | %9.2f %9.1f | %9.2f %9.1f | %9.2f %9.1f | %9.2f %9.1f | %8.2f" %
               (size, "", r_med, row["reduce2_gbps"], p_med, row["pack_gbps"], u_med, row["unpack_gbps"],
-               c_med, row["memcpy_gbps"], b2b), flush=True)
+               c_med, row["memcpy_gbps"], m_med, row["memset_gbps"], b2b), flush=True)
         del a, b, c, sparse, staged
         size *= 2
     if args.json:
