@@ -53,24 +53,51 @@ const DeviceInfo &deviceInfo() {
 // 0 = no cap).  Measured on MI355X with HBM-resident buffers over a set of
 // inter-buffer strides.  About 48-128 KiB of loads in flight per CU saturates HBM;
 // more resident wavefronts only add DRAM page conflicts between the streams -
-// unless the K loads of a wavefront all land in the same channel group, in which
-// case their latencies add up and more wavefronts are needed to cover them.  So
-// there are two columns: `spread` when the inputs' addresses fall into (nearly) K
-// different channel groups, `aliased` when they collide; aliased launches also pace
-// their loads (reduce_device.h), which wants more wavefronts still (K = 8: 87-88 %
-// of peak at 8 when spread; aliased 78-82 % at 8, 81-83 % at 16, 85-86 % paced at
-// 18; pacing gains nothing up to four inputs).  Up to three inputs one value
-// serves both.
+// unless the K loads of a wavefront land in the same channel group, in which case
+// their latencies add up and more wavefronts are needed to cover them.  So launches
+// whose wavefronts ask for all K inputs at once have two columns: `spread` when the
+// inputs' addresses fall into K different channel groups, `aliased` when they
+// collide.  Large launches of four or more inputs keep two inputs in flight per
+// wavefront instead (reduce_device.h), which runs equally well over either kind of
+// layout and has its own column.  256 MiB per input, percent of peak, three sets
+// of buffers used in turn so that no launch finds its buffers in the memory-side
+// cache: K = 8 all at once 85 (spread, 8 per CU) / 78-81 (aliased, any number), two
+// in flight 84-87; K = 6: 86 / 82 / 85-87; K = 5: 86 / 82-83 / 83-85; K = 4: 86 /
+// 82-83 / 84-85.  (The same buffers launch after launch run two to four percent
+// higher throughout: part of the 256 MiB output stays in that cache.)
 static const int kWavesSpread[9] = {0, 0, 25, 14, 11, 10, 10, 9, 8};
-static const int kWavesAliased[9] = {0, 0, 25, 14, 10, 21, 21, 18, 18};
-// explicit settings (flagcxLocalTune); -1 = choose from the tables above
+static const int kWavesAliased[9] = {0, 0, 25, 14, 11, 21, 21, 18, 18};
+static const int kWavesTwoInFlight[9] = {0, 0, 0, 0, 14, 16, 14, 14, 14};
+// explicit settings (flagcxLocalTune, flagcxLocalTuneLoads); -1 = choose as above
 static std::atomic<int> gWaves[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
+static std::atomic<int> gLoads[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
 
-int wavesPerCUFor(int k, bool spread) {
+// KiB per input from which a launch keeps two inputs in flight per wavefront:
+// below, too few rounds of wavefronts run for the longer life of each to pay
+// (16 MiB per input; four inputs gain only from 128 MiB on, and only when aliased).
+static const uint64_t kMinTilesTwoInFlight[9] = {0, 0, 0, 0, 131072, 16384, 16384, 16384, 16384};
+
+int loadsInFlightFor(int k, uint64_t tiles) {
+  if (k < 4 || k > 8) return 0;
+  const int set = gLoads[k].load(std::memory_order_relaxed);
+  if (set >= 0) return set;
+  return tiles >= kMinTilesTwoInFlight[k] ? 2 : 0;
+}
+int tunedLoadsInFlight(int k) { return (k >= 0 && k <= 8) ? gLoads[k].load(std::memory_order_relaxed) : -1; }
+void setLoadsInFlight(int k, int loads) {
+  if (k >= 0 && k <= 8) gLoads[k].store(loads, std::memory_order_relaxed);
+}
+
+int wavesPerCUFor(int k, bool spread, int inflight) {
   if (k < 0) k = 0;
   if (k > 8) k = 8;
   const int set = gWaves[k].load(std::memory_order_relaxed);
   if (set >= 0) return set;
+  if (k >= 4 && inflight > 0) {
+    // the product of wavefronts and inputs in flight is what has to cover the latency
+    if (inflight == 2) return kWavesTwoInFlight[k];
+    return inflight == 1 ? 25 : 11;
+  }
   return spread ? kWavesSpread[k] : kWavesAliased[k];
 }
 int tunedWavesPerCU(int k) { return (k >= 0 && k <= 8) ? gWaves[k].load(std::memory_order_relaxed) : -1; }
@@ -101,9 +128,10 @@ bool inputsSpread(const void *const *src, int k) {
     seen |= 1u << g;
     middle += (g >> 2) & 1u;
   }
-  // at least three quarters of the inputs in groups of their own, and both values of
-  // the middle hash bit taken by at least a quarter of them
-  return 4 * (n - distinct) <= n && 4 * middle >= n && 4 * (n - middle) >= n;
+  // every input in a group of its own, and both values of the middle hash bit taken
+  // by at least a quarter of them (buffers that share groups in pairs already lose
+  // six percent with few wavefronts; a wrong `aliased` costs one to three)
+  return distinct == n && 4 * middle >= n && 4 * (n - middle) >= n;
 }
 
 int ldsReservation(int waves) {
@@ -339,6 +367,21 @@ flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU) {
   if (nranks < 0 || nranks > 8 || wavesPerCU < -1 || wavesPerCU > 64)
     return fail(flagcxInvalidArgument, "flagcxLocalTune: nranks %d / wavesPerCU %d out of range", nranks, wavesPerCU);
   setWavesPerCU(nranks, wavesPerCU);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight) {
+  if (nranks < 4 || nranks > 8 || inputsInFlight < -1 || inputsInFlight > 3)
+    return fail(flagcxInvalidArgument, "flagcxLocalTuneLoads: nranks %d (4..8) / inputsInFlight %d (-1..3) out of range", nranks,
+                inputsInFlight);
+  setLoadsInFlight(nranks, inputsInFlight);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalGetTuneLoads(int nranks, int *inputsInFlight) {
+  if (nranks < 4 || nranks > 8 || !inputsInFlight)
+    return fail(flagcxInvalidArgument, "flagcxLocalGetTuneLoads: nranks %d out of range (4..8) or NULL result", nranks);
+  *inputsInFlight = tunedLoadsInFlight(nranks);
   return flagcxSuccess;
 }
 

@@ -28,7 +28,9 @@ const DeviceInfo &deviceInfo();
 
 // Resident single-wave workgroups per CU for a k-input reduce (k = 0: copies);
 // `spread`: the inputs' addresses fall into different HBM channel groups.
-int wavesPerCUFor(int k, bool spread = true);
+int wavesPerCUFor(int k, bool spread = true, int inflight = 0);
+// inputs whose loads a wavefront keeps in flight (0 = all) in a launch of `tiles` KiB per input
+int loadsInFlightFor(int k, uint64_t tiles);
 void setWavesPerCU(int k, int waves);
 int tunedWavesPerCU(int k); // the explicit setting, or -1
 bool inputsSpread(const void *const *src, int k);

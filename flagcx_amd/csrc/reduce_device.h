@@ -42,7 +42,7 @@ struct ReduceParams {
   uint64_t head;   // elements before the body
   uint64_t tail;   // elements after the body
   int32_t k;       // number of inputs actually used (== K except generic)
-  int32_t pace;    // non-zero: space a wavefront's loads out in time (inputs that share one HBM channel group)
+  int32_t inflight; // 1..3: a wavefront keeps the loads of at most that many inputs in flight; 0: of all K
 };
 
 // ------------------------------------------------------------------ widen
@@ -209,10 +209,19 @@ __device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
 #pragma unroll
       for (int u = 0; u < U; u++)
         in[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + u * 1024u, 0, kLoadAux);
-      // K loads into one channel group (same bank, K different rows) issued back to
-      // back thrash the row buffers; about 0.3 us between them lets other
-      // wavefronts' accesses in (8 inputs 256 MiB apart: 82 -> 86 % of peak)
-      if (K >= 5 && j + 1 < K && p.pace) __builtin_amdgcn_s_sleep(12);
+      // K loads issued back to back by every resident wavefront reach DRAM as bursts
+      // that thrash the row buffers, worst when the K addresses share a channel
+      // group (same bank, K rows).  Waiting until at most inflight-1 earlier inputs
+      // are outstanding before asking for the next lets other wavefronts' accesses
+      // in between, and needs no timing constant (8 inputs 256 MiB apart, buffers
+      // not touched by the previous launch: 78 -> 86 % of peak with two in flight).
+      // s_waitcnt fields on gfx9: vmcnt [3:0], expcnt [6:4], lgkmcnt [11:8]; 0x0F70
+      // leaves the other two counters alone.
+      if (K >= 4 && j + 1 < K && p.inflight) {
+        if (p.inflight == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | U);
+        else if (p.inflight == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | 0);
+        else __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * U));
+      }
     }
     __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
         (void *)((char *)p.dst + headBytes + off), 0, span, kRsrcFlags);

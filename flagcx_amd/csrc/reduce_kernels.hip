@@ -45,7 +45,6 @@ typedef bf16 elem_t;
 constexpr int unrollFor(int) { return 1; }
 
 constexpr uint64_t kMaxGrid = 1u << 24;
-constexpr uint64_t kPaceMinTiles = 32768; // 32 MiB per input: eight rounds of 16 wavefronts on 256 CUs
 
 struct Split {
   uint64_t head, nvec, tail;
@@ -79,15 +78,16 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   p.head = s.head;
   p.tail = s.tail;
   p.k = K;
-  const bool spread = inputsSpread(c.src, K);
   const uint64_t tileBytes = 64ull * U * 16ull;
   uint64_t tiles = (s.nvec * 16 + tileBytes - 1) / tileBytes;
-  // pacing trades latency per wavefront for DRAM efficiency: only where the launch
-  // runs many rounds of resident wavefronts
-  p.pace = (!spread && tiles >= kPaceMinTiles) ? 1 : 0;
+  // a limit on the inputs in flight per wavefront trades latency per wavefront for
+  // DRAM efficiency: by default only where the launch runs many rounds of resident
+  // wavefronts
+  const int inflight = loadsInFlightFor(K, tiles);
+  p.inflight = inflight;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  const int lds = ldsReservation(wavesPerCUFor(K, spread));
+  const int lds = ldsReservation(wavesPerCUFor(K, inflight ? true : inputsSpread(c.src, K), inflight));
   reduceWaveKernel<elem_t, OP, K, U><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
   return (int)hipGetLastError();
 }
@@ -102,7 +102,7 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   p.head = s.head;
   p.tail = s.tail;
   p.k = c.k;
-  p.pace = 0;
+  p.inflight = 0;
   uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
@@ -154,15 +154,15 @@ static int launchBatchFixed(const ReduceCall *calls, const Split *splits, int n)
       p.head = s.head;
       p.tail = s.tail;
       p.k = K;
-      p.pace = 0;
+      p.inflight = 0;
       const uint64_t tiles = (s.nvec * 16 + tileBytes - 1) / tileBytes;
       if (tiles > maxTiles) maxTiles = tiles;
       totalTiles += tiles;
     }
     if (maxTiles > kMaxGrid) maxTiles = kMaxGrid;
-    if (totalTiles >= kPaceMinTiles)
-      for (int i = 0; i < m; i++) bp.seg[i].pace = inputsSpread(calls[base + i].src, K) ? 0 : 1;
-    const int lds = ldsReservation(wavesPerCUFor(K, inputsSpread(calls[base].src, K)));
+    const int inflight = loadsInFlightFor(K, totalTiles);
+    for (int i = 0; i < m; i++) bp.seg[i].inflight = inflight;
+    const int lds = ldsReservation(wavesPerCUFor(K, inputsSpread(calls[base].src, K), inflight));
     reduceBatchKernel<elem_t, OP, K, U>
         <<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, calls[0].stream>>>(bp);
     const int err = (int)hipGetLastError();

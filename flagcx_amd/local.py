@@ -114,7 +114,7 @@ class CopyArgs(C.Structure):         # flagcxLocalCopyArgs
 
 EXPORTS = [
     "flagcxLocalGetDataTypeSize", "flagcxLocalInit", "flagcxLocalGetErrorString", "flagcxLocalGetLastError",
-    "flagcxLocalTune", "flagcxLocalGetTune", "flagcxLocalPlaceBuffers", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
+    "flagcxLocalTune", "flagcxLocalGetTune", "flagcxLocalTuneLoads", "flagcxLocalGetTuneLoads", "flagcxLocalPlaceBuffers", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
     "flagcxLocalAllReduce", "flagcxLocalRingChunkTable", "flagcxLocalMemcpy", "flagcxLocalMemset",
     "flagcxLocalRefresh", "flagcxLocalPack", "flagcxLocalUnpack", "flagcxLocalPackList",
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
@@ -157,6 +157,8 @@ def lib():
         L.flagcxLocalTune.argtypes = [i, i]
         L.flagcxLocalPlaceBuffers.argtypes = [vp, sz, sz, i, pp]
         L.flagcxLocalGetTune.argtypes = [i, C.POINTER(i)]
+        L.flagcxLocalTuneLoads.argtypes = [i, i]
+        L.flagcxLocalGetTuneLoads.argtypes = [i, C.POINTER(i)]
         L.flagcxLocalReduce.argtypes = [pp, i, vp, sz, i, i, sp]
         L.flagcxLocalReduceScatter.argtypes = [pp, i, i, vp, sz, i, i, sp]
         L.flagcxLocalReduceScatterChunked.argtypes = [pp, i, i, vp, sz, i, i, sz, sp]

@@ -139,15 +139,23 @@ const char *flagcxLocalGetLastError(void);
  * buffers placed by this call at 87-89 %.  Host-only, no device access. */
 flagcxResult_t flagcxLocalPlaceBuffers(void *pool, size_t poolbytes, size_t bytes, int nbuffers, void **buffers);
 
-/* Launch-shape knob, in the spirit of the reference's FLAGCX_* tuning variables:
- * how many one-wavefront workgroups may share a CU for a reduce of `nranks`
+/* Launch-shape knobs, in the spirit of the reference's FLAGCX_* tuning variables.
+ * Tune: how many one-wavefront workgroups may share a CU for a reduce of `nranks`
  * inputs (1..8; 0 selects the copy kernels).  wavesPerCU == 0 removes the cap,
  * -1 (the default, and what GetTune then reports) lets every launch choose from
- * the values measured on MI355X: for four or more inputs it looks at whether
- * their addresses fall into different HBM channel groups (few wavefronts are
- * best) or collide (more are needed).  Process-wide. */
+ * the values measured on MI355X.
+ * TuneLoads: of how many of its `nranks` inputs (4..8) a wavefront keeps the loads
+ * in flight before it asks for the next: 1..3, 0 = all of them at once, -1 (the
+ * default) = two for launches of 16 MiB per input and more (128 MiB with four
+ * inputs), all at once below.
+ * Launches that ask for all inputs at once look at whether the inputs' addresses
+ * fall into different HBM channel groups (few wavefronts are best) or collide
+ * (more are needed); with a limit the layout of the inputs hardly matters.
+ * Process-wide. */
 flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU);
 flagcxResult_t flagcxLocalGetTune(int nranks, int *wavesPerCU);
+flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight);
+flagcxResult_t flagcxLocalGetTuneLoads(int nranks, int *inputsInFlight);
 
 /* ------------------------------------------------------------------------- */
 /* N-way elementwise reduction                                                */

@@ -170,10 +170,10 @@ def test_c5_sweep_reduce2_and_strided_pack_unpack(L, log2):
 @pytest.mark.parametrize("k,dt,op", [(8, O.BF16, O.SUM), (6, O.FP16, O.AVG), (5, O.INT32, O.MAX), (4, O.FP32, O.SUM)],
                          ids=lambda v: str(v))
 def test_placed_and_aliased_layouts_give_the_same_bytes(L, k, dt, op):
-    """Launch shape depends on where the inputs sit: buffers placed in different HBM channel
-    groups take few wavefronts per CU, buffers that all start in one group take more and
-    space their loads out.  Large enough for both shapes to be the ones chosen (64 MiB per
-    input); both results equal the oracle's bit for bit."""
+    """Where the inputs sit must not show in the result: buffers placed in different HBM
+    channel groups and buffers that all start in one group, at a size (64 MiB per input)
+    where five and more inputs are loaded two at a time and four all at once; both
+    results equal the oracle's bit for bit."""
     import torch
     from tests.util import make_inputs
     npdt = np.dtype(O.NP_OF[dt])
@@ -209,6 +209,48 @@ def test_placed_and_aliased_layouts_give_the_same_bytes(L, k, dt, op):
     nan_ok = dt in (O.BF16, O.FP16, O.FP32) and op in (O.SUM, O.AVG)
     for got in (placed[k], out2):
         assert same(got.cpu().numpy().view(npdt), want, nan_class=nan_ok, dtype=dt)
+
+
+@pytest.mark.parametrize("k,dt,op", [(8, O.BF16, O.SUM), (7, O.FP32, O.PROD), (6, O.FP16, O.AVG), (5, O.INT32, O.MAX), (4, O.FP64, O.SUM)],
+                         ids=lambda v: str(v))
+def test_every_number_of_inputs_in_flight_gives_the_same_bytes(L, k, dt, op):
+    """flagcxLocalTuneLoads only changes when a wavefront asks for its inputs, never the
+    fold order: all inputs at once, one, two or three in flight, and the library's choice
+    equal the oracle bit for bit; single launch and batch call, ragged count, and one input
+    that is also the output."""
+    import torch
+    from tests.util import make_inputs
+    npdt = np.dtype(O.NP_OF[dt])
+    n = (3 * MiB + 4096 + 24) // npdt.itemsize + 3
+    hosts = make_inputs(dt, k, n, seed=1700 + k, op=op)
+    rc, want = O.reduce(hosts, dt, op)
+    assert rc == 0
+    carrier = {2: torch.int16, 4: torch.int32, 8: torch.int64}[npdt.itemsize]
+    devs = [torch.from_numpy(h.view(np.dtype("int%d" % (8 * npdt.itemsize)))).cuda() for h in hosts]
+    nan_ok = dt in (O.BF16, O.FP16, O.FP32, O.FP64) and op in (O.SUM, O.AVG, O.PROD)
+    half = (n // 2) & ~7
+    try:
+        for loads in (0, 1, 2, 3, -1):
+            assert L.lib().flagcxLocalTuneLoads(k, loads) == 0
+            out = torch.zeros(n, dtype=carrier, device="cuda")
+            L.reduce(devs, out, op, dtype=dt)
+            torch.cuda.synchronize()
+            assert same(out.cpu().numpy().view(npdt), want, nan_class=nan_ok, dtype=dt), loads
+            # two segments in one batch call
+            out2 = torch.zeros(n, dtype=carrier, device="cuda")
+            esz = npdt.itemsize
+            descs = [([d.data_ptr() for d in devs], out2.data_ptr(), half),
+                     ([d.data_ptr() + half * esz for d in devs], out2.data_ptr() + half * esz, n - half)]
+            L.reduce_batch(descs, op, dt, k)
+            torch.cuda.synchronize()
+            assert same(out2.cpu().numpy().view(npdt), want, nan_class=nan_ok, dtype=dt), loads
+            # in place: the output is input 1
+            mine = [d.clone() for d in devs]
+            L.reduce(mine, mine[1], op, dtype=dt)
+            torch.cuda.synchronize()
+            assert same(mine[1].cpu().numpy().view(npdt), want, nan_class=nan_ok, dtype=dt), loads
+    finally:
+        assert L.lib().flagcxLocalTuneLoads(k, -1) == 0
 
 
 def test_buffers_beyond_4GiB(L):
