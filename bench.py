@@ -37,7 +37,7 @@ ALGO_BYTES = (K + 1) * N_ELEM * 2   # k reads + 1 write
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/reduce8_bf16_sum_256MiB_pmc.txt), scaled by a copy kernel of known size.
-MEASURED_TRAFFIC_BYTES = 2415853564
+MEASURED_TRAFFIC_BYTES = 2415851937
 
 
 def log(*a):
@@ -74,6 +74,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--allocator-layout", action="store_true",
                     help="inputs and output as separate torch allocations instead of placed in one")
+    ap.add_argument("--rotate-sets", type=int, default=3, metavar="S",
+                    help="also time the same launches over S sets of buffers used in turn (0: skip), "
+                         "reported as rotating_buffers")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also run N flagcxLocalMemcpy launches of 256 MiB (a copy of known size "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -133,6 +136,43 @@ def main():
     kern_ms = ev0.elapsed_time(ev1) / args.steps
     value = ALGO_BYTES / (wall_ms * 1e-3) / 1e9
     achieved = ALGO_BYTES / (kern_ms * 1e-3) / 1e9
+
+    # The timed loop above reduces the same nine buffers every step, as the metric is
+    # defined; part of the 256 MiB output of one step is then still in the memory-side
+    # cache when the next step writes it again.  For comparison: S sets of buffers
+    # used in turn, so that no launch finds anything of its own there.
+    rotating = None
+    if args.rotate_sets >= 2:
+        sets, keep = [bufs], []
+        for _ in range(args.rotate_sets - 1):
+            if args.allocator_layout:
+                more = [torch.empty(N_ELEM, dtype=torch.bfloat16, device="cuda") for _ in range(K + 1)]
+            else:
+                p2 = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+                keep.append(p2)
+                more = [p2[a - p2.data_ptr(): a - p2.data_ptr() + nbytes].view(torch.bfloat16)
+                        for a in L.place_buffers(p2.data_ptr(), pool_bytes, nbytes, K + 1)]
+            for j in range(K):
+                more[j].copy_(inputs[j])
+            sets.append(more)
+        nset = len(sets)
+        for i in range(2 * nset):
+            L.reduce(sets[i % nset][:K], sets[i % nset][K], L.RedOp.Sum)
+        torch.cuda.synchronize()
+        r0 = torch.cuda.Event(enable_timing=True)
+        r1 = torch.cuda.Event(enable_timing=True)
+        r0.record()
+        for i in range(args.steps):
+            L.reduce(sets[i % nset][:K], sets[i % nset][K], L.RedOp.Sum)
+        r1.record()
+        torch.cuda.synchronize()
+        rot_ms = r0.elapsed_time(r1) / args.steps
+        same_out = all(torch.equal(sets[i][K].view(torch.int16), out.view(torch.int16)) for i in range(1, nset))
+        rotating = {"sets": nset, "value": round(ALGO_BYTES / (rot_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                    "frac": round(ALGO_BYTES / (rot_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "avg_launch_ms": round(rot_ms, 5), "outputs_equal_first_set": bool(same_out)}
+        del sets, keep
+        torch.cuda.empty_cache()
 
     for _ in range(args.calibrate_copy):
         L.memcpy(out.data_ptr(), inputs[0].data_ptr(), N_ELEM * 2)
@@ -197,6 +237,7 @@ def main():
                    "nranks": K, "elements": N_ELEM, "bytes_per_step": ALGO_BYTES, "accumulate": "fp32",
                    "buffers": layout},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "rotating_buffers": rotating,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "reduceWaveKernel<bf16,sum,K=8,U=1>", "avg_launch_ms": round(kern_ms, 5),

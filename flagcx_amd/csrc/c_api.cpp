@@ -57,31 +57,34 @@ const DeviceInfo &deviceInfo() {
 // their latencies add up and more wavefronts are needed to cover them.  So launches
 // whose wavefronts ask for all K inputs at once have two columns: `spread` when the
 // inputs' addresses fall into K different channel groups, `aliased` when they
-// collide.  Large launches of four or more inputs keep two inputs in flight per
-// wavefront instead (reduce_device.h), which runs equally well over either kind of
-// layout and has its own column.  256 MiB per input, percent of peak, three sets
-// of buffers used in turn so that no launch finds its buffers in the memory-side
-// cache: K = 8 all at once 85 (spread, 8 per CU) / 78-81 (aliased, any number), two
-// in flight 84-87; K = 6: 86 / 82 / 85-87; K = 5: 86 / 82-83 / 83-85; K = 4: 86 /
-// 82-83 / 84-85.  (The same buffers launch after launch run two to four percent
-// higher throughout: part of the 256 MiB output stays in that cache.)
+// collide.  Large launches limit the inputs a wavefront has in flight instead
+// (reduce_device.h): that runs equally well over either kind of layout and has
+// its own column.  256 MiB per input, percent of peak, three sets of buffers used
+// in turn so that no launch finds its buffers in the memory-side cache: K = 8 all
+// at once 85 (spread, 8 per CU) / 78-81 (aliased, any number), two in flight 85-88;
+// K = 6: 86 / 82 / 85-87; K = 5: 86 / 82-83 / 83-85; K = 4: 86 / 82-83 / 84-85;
+// K = 3: 82 all at once, 85 one at a time; K = 2: 84 / 85.  (The same buffers launch
+// after launch run two to five percent higher throughout: part of the 256 MiB
+// output stays in that cache.)
 static const int kWavesSpread[9] = {0, 0, 25, 14, 11, 10, 10, 9, 8};
 static const int kWavesAliased[9] = {0, 0, 25, 14, 11, 21, 21, 18, 18};
-static const int kWavesTwoInFlight[9] = {0, 0, 0, 0, 14, 16, 14, 14, 14};
+// the large launches: inputs in flight per wavefront, wavefronts per CU with that,
+// and the KiB per input from which a launch counts as large.  Below, too few rounds
+// of wavefronts run for the longer life of each to pay: 16 MiB per input for five
+// and more inputs; two to four gain only from 128 MiB on.
+static const int kLoadsLarge[9] = {0, 0, 1, 1, 2, 2, 2, 2, 2};
+static const int kWavesLarge[9] = {0, 0, 25, 21, 14, 16, 14, 14, 14};
+static const uint64_t kNever = ~0ull;
+static const uint64_t kMinTilesLarge[9] = {kNever, kNever, 131072, 131072, 131072, 16384, 16384, 16384, 16384};
 // explicit settings (flagcxLocalTune, flagcxLocalTuneLoads); -1 = choose as above
 static std::atomic<int> gWaves[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
 static std::atomic<int> gLoads[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
 
-// KiB per input from which a launch keeps two inputs in flight per wavefront:
-// below, too few rounds of wavefronts run for the longer life of each to pay
-// (16 MiB per input; four inputs gain only from 128 MiB on, and only when aliased).
-static const uint64_t kMinTilesTwoInFlight[9] = {0, 0, 0, 0, 131072, 16384, 16384, 16384, 16384};
-
 int loadsInFlightFor(int k, uint64_t tiles) {
-  if (k < 4 || k > 8) return 0;
+  if (k < 2 || k > 8) return 0;
   const int set = gLoads[k].load(std::memory_order_relaxed);
-  if (set >= 0) return set;
-  return tiles >= kMinTilesTwoInFlight[k] ? 2 : 0;
+  if (set >= 0) return set < k ? set : 0;
+  return tiles >= kMinTilesLarge[k] ? kLoadsLarge[k] : 0;
 }
 int tunedLoadsInFlight(int k) { return (k >= 0 && k <= 8) ? gLoads[k].load(std::memory_order_relaxed) : -1; }
 void setLoadsInFlight(int k, int loads) {
@@ -93,10 +96,10 @@ int wavesPerCUFor(int k, bool spread, int inflight) {
   if (k > 8) k = 8;
   const int set = gWaves[k].load(std::memory_order_relaxed);
   if (set >= 0) return set;
-  if (k >= 4 && inflight > 0) {
+  if (k >= 2 && inflight > 0) {
     // the product of wavefronts and inputs in flight is what has to cover the latency
-    if (inflight == 2) return kWavesTwoInFlight[k];
-    return inflight == 1 ? 25 : 11;
+    if (inflight == kLoadsLarge[k]) return kWavesLarge[k];
+    return inflight == 1 ? 25 : inflight == 2 ? 14 : 11;
   }
   return spread ? kWavesSpread[k] : kWavesAliased[k];
 }
@@ -371,7 +374,7 @@ flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU) {
 }
 
 flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight) {
-  if (nranks < 4 || nranks > 8 || inputsInFlight < -1 || inputsInFlight > 3)
+  if (nranks < 2 || nranks > 8 || inputsInFlight < -1 || inputsInFlight > 3)
     return fail(flagcxInvalidArgument, "flagcxLocalTuneLoads: nranks %d (4..8) / inputsInFlight %d (-1..3) out of range", nranks,
                 inputsInFlight);
   setLoadsInFlight(nranks, inputsInFlight);
@@ -379,7 +382,7 @@ flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight) {
 }
 
 flagcxResult_t flagcxLocalGetTuneLoads(int nranks, int *inputsInFlight) {
-  if (nranks < 4 || nranks > 8 || !inputsInFlight)
+  if (nranks < 2 || nranks > 8 || !inputsInFlight)
     return fail(flagcxInvalidArgument, "flagcxLocalGetTuneLoads: nranks %d out of range (4..8) or NULL result", nranks);
   *inputsInFlight = tunedLoadsInFlight(nranks);
   return flagcxSuccess;

@@ -42,7 +42,7 @@ struct ReduceParams {
   uint64_t head;   // elements before the body
   uint64_t tail;   // elements after the body
   int32_t k;       // number of inputs actually used (== K except generic)
-  int32_t inflight; // 1..3: a wavefront keeps the loads of at most that many inputs in flight; 0: of all K
+  int32_t inflight; // 1..3 (< K): a wavefront keeps the loads of at most that many inputs in flight; 0: of all K
 };
 
 // ------------------------------------------------------------------ widen
@@ -217,7 +217,7 @@ __device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
       // not touched by the previous launch: 78 -> 86 % of peak with two in flight).
       // s_waitcnt fields on gfx9: vmcnt [3:0], expcnt [6:4], lgkmcnt [11:8]; 0x0F70
       // leaves the other two counters alone.
-      if (K >= 4 && j + 1 < K && p.inflight) {
+      if (K >= 2 && j + 1 < K && p.inflight) {
         if (p.inflight == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | U);
         else if (p.inflight == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | 0);
         else __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * U));

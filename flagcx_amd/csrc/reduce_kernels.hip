@@ -109,6 +109,8 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   // more than eight inputs are loaded eight at a time; measured on MI355X: 9..10
   // inputs want 12 wavefronts per CU (88 % of peak against 79 % at 8), 11..13 want
   // 10, more want 8 (85-86 %).  An explicit flagcxLocalTune(8, n) overrides.
+  // (A limit on the inputs in flight, as the kernels for up to eight inputs have
+  // it, gains nothing here: within one percent for 9..32 inputs.)
   int waves = c.k > 8 ? tunedWavesPerCU(8) : -1;
   if (c.k <= 8) waves = wavesPerCUFor(c.k, inputsSpread(c.src, c.k));
   else if (waves < 0) waves = c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;

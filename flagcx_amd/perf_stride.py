@@ -63,7 +63,7 @@ def main():
         iters = 20 * args.sets
         for cap in CAPS:
             L.check(L.lib().flagcxLocalTune(k, cap))
-            if k >= 4:
+            if k >= 2:
                 L.check(L.lib().flagcxLocalTuneLoads(k, args.loads if cap >= 0 else -1))
             for i in range(3 * args.sets):
                 L.reduce(srcs[i % args.sets], outs[i % args.sets], L.RedOp.Sum)
@@ -81,7 +81,7 @@ def main():
             row.append("%7.1f" % pct)
         print("%14d " % st + " ".join(row), flush=True)
     L.check(L.lib().flagcxLocalTune(k, default_cap))
-    if k >= 4:
+    if k >= 2:
         L.check(L.lib().flagcxLocalTuneLoads(k, -1))
     print("setting found for k=%d: %d (-1 = chosen per launch)" % (k, default_cap))
     print("%14s " % "worst..best" + " ".join("%3.0f..%-3.0f" % (worst[c], best[c]) for c in CAPS))

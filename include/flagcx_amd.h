@@ -144,10 +144,10 @@ flagcxResult_t flagcxLocalPlaceBuffers(void *pool, size_t poolbytes, size_t byte
  * inputs (1..8; 0 selects the copy kernels).  wavesPerCU == 0 removes the cap,
  * -1 (the default, and what GetTune then reports) lets every launch choose from
  * the values measured on MI355X.
- * TuneLoads: of how many of its `nranks` inputs (4..8) a wavefront keeps the loads
+ * TuneLoads: of how many of its `nranks` inputs (2..8) a wavefront keeps the loads
  * in flight before it asks for the next: 1..3, 0 = all of them at once, -1 (the
- * default) = two for launches of 16 MiB per input and more (128 MiB with four
- * inputs), all at once below.
+ * default) = two (one with two or three inputs) in large launches - 16 MiB per
+ * input and more, 128 MiB with up to four inputs - and all at once below.
  * Launches that ask for all inputs at once look at whether the inputs' addresses
  * fall into different HBM channel groups (few wavefronts are best) or collide
  * (more are needed); with a limit the layout of the inputs hardly matters.

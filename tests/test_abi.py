@@ -114,7 +114,7 @@ def test_other_entry_points_reject_bad_arguments():
     assert L.flagcxLocalTune(8, 8) == 0
     assert L.flagcxLocalTune(8, -1) == 0   # back to the per-launch choice
     got = C.c_int(7)
-    assert L.flagcxLocalTuneLoads(3, 2) == inv                                  # fewer than four inputs: nothing to limit
+    assert L.flagcxLocalTuneLoads(1, 1) == inv                                  # one input: nothing to limit
     assert L.flagcxLocalTuneLoads(8, 4) == inv
     assert L.flagcxLocalTuneLoads(8, 3) == 0
     assert L.flagcxLocalGetTuneLoads(8, C.byref(got)) == 0 and got.value == 3

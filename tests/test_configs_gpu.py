@@ -211,7 +211,7 @@ def test_placed_and_aliased_layouts_give_the_same_bytes(L, k, dt, op):
         assert same(got.cpu().numpy().view(npdt), want, nan_class=nan_ok, dtype=dt)
 
 
-@pytest.mark.parametrize("k,dt,op", [(8, O.BF16, O.SUM), (7, O.FP32, O.PROD), (6, O.FP16, O.AVG), (5, O.INT32, O.MAX), (4, O.FP64, O.SUM)],
+@pytest.mark.parametrize("k,dt,op", [(8, O.BF16, O.SUM), (7, O.FP32, O.PROD), (6, O.FP16, O.AVG), (5, O.INT32, O.MAX), (4, O.FP64, O.SUM), (3, O.UINT8, O.SUM), (2, O.INT64, O.MIN)],
                          ids=lambda v: str(v))
 def test_every_number_of_inputs_in_flight_gives_the_same_bytes(L, k, dt, op):
     """flagcxLocalTuneLoads only changes when a wavefront asks for its inputs, never the
@@ -225,7 +225,7 @@ def test_every_number_of_inputs_in_flight_gives_the_same_bytes(L, k, dt, op):
     hosts = make_inputs(dt, k, n, seed=1700 + k, op=op)
     rc, want = O.reduce(hosts, dt, op)
     assert rc == 0
-    carrier = {2: torch.int16, 4: torch.int32, 8: torch.int64}[npdt.itemsize]
+    carrier = {1: torch.int8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[npdt.itemsize]
     devs = [torch.from_numpy(h.view(np.dtype("int%d" % (8 * npdt.itemsize)))).cuda() for h in hosts]
     nan_ok = dt in (O.BF16, O.FP16, O.FP32, O.FP64) and op in (O.SUM, O.AVG, O.PROD)
     half = (n // 2) & ~7
