@@ -222,10 +222,14 @@ flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int ca
   q->dtype = dt;
   q->op = rop;
   q->typeSize = ts;
-  // Measured on MI355X (128 x 4 MiB chunks per input): few inputs want more
-  // wavefronts in flight, many inputs fewer; never more than half a CU's slots,
-  // so that residency does not depend on the last slot being free.
-  static const int kWaves[9] = {16, 16, 12, 12, 8, 8, 8, 8, 8};
+  // Measured on MI355X (64 x 4 MiB chunks per input, 6..16 wavefronts per CU): few
+  // inputs want more wavefronts in flight, many inputs fewer (two inputs 3.6 -> 5.1
+  // TB/s from 6 to 16, eight 6.0 / 6.1 / 5.8 at 6 / 10 / 16); never more than half a
+  // CU's slots, so that residency does not depend on the last slot being free.  (A
+  // limit on the inputs a worker has in flight, which the launched kernels use for
+  // large reduces, only costs here: 16 wavefronts per CU cannot cover the longer
+  // life of each.)
+  static const int kWaves[9] = {16, 16, 16, 16, 14, 14, 14, 10, 10};
   q->wavesPerCU = kWaves[maxRanks];
   const DeviceInfo &info = deviceInfo();
   q->maxGrid = (unsigned)info.numCU * 16u;
