@@ -134,9 +134,10 @@ const char *flagcxLocalGetLastError(void);
  * (beyond 32 buffers every run of 32 shares the groups out again).
  * The callers that allocate the ranks' staging / scratch buffers
  * (flagcx/core/c2c_algo.cc:2121-2137) can place them this way: an 8-input reduce
- * over buffers that all start in the same group (e.g. 258 MiB apart, where a
- * caching allocator puts 256 MiB buffers) runs at 85-86 % of the HBM peak, over
- * buffers placed by this call at 87-89 %.  Host-only, no device access. */
+ * of 256 MiB per input runs at 87 % of the HBM peak over buffers placed by this
+ * call and at 85-86 % over buffers that all start in the same group (e.g. 258 MiB
+ * apart, where a caching allocator puts 256 MiB buffers).  Host-only, no device
+ * access. */
 flagcxResult_t flagcxLocalPlaceBuffers(void *pool, size_t poolbytes, size_t bytes, int nbuffers, void **buffers);
 
 /* Launch-shape knobs, in the spirit of the reference's FLAGCX_* tuning variables.
