@@ -111,8 +111,13 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   // 10, more want 8 (85-86 %).  An explicit flagcxLocalTune(8, n) overrides.
   // (A limit on the inputs in flight, as the kernels for up to eight inputs have
   // it, gains nothing here: within one percent for 9..32 inputs.)
+  // Sources at another offset modulo 16 than the output (up to eight of them come
+  // here too) are bound by the unaligned loads themselves, 68-78 % of peak, and
+  // want more wavefronts to get there: measured 25, 21, 14 per CU for 2, 4, 8
+  // inputs, whatever their layout.
+  static const int kWavesUnaligned[9] = {0, 0, 25, 25, 21, 21, 16, 14, 14};
   int waves = c.k > 8 ? tunedWavesPerCU(8) : -1;
-  if (c.k <= 8) waves = wavesPerCUFor(c.k, inputsSpread(c.src, c.k));
+  if (c.k <= 8) waves = (!s.vector && tunedWavesPerCU(c.k) < 0) ? kWavesUnaligned[c.k] : wavesPerCUFor(c.k, inputsSpread(c.src, c.k));
   else if (waves < 0) waves = c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
   const int lds = ldsReservation(waves);
   if (s.vector)
