@@ -64,6 +64,30 @@ def cpu_baseline(inputs_bits, sample_elems):
     }, host, dst
 
 
+def cpu_other_configs():
+    """The CPU side of two more benchmark configurations: C1 (2 x fp32 sum, 64 MiB per
+    buffer, full size) and C4 (4 x int32 max, a 16 Mi-element sample of 128 Mi)."""
+    from oracle import cpu_oracle as O
+    rng = np.random.default_rng(0)
+    out = []
+    n1 = 16 * 1024 * 1024
+    fa = rng.uniform(-1, 1, n1).astype(np.float32)
+    fb = rng.uniform(-1, 1, n1).astype(np.float32)
+    fd = np.empty_like(fa)
+    for nth in (1, 2):
+        t = O.time_reduce([fa, fb], fd, O.FP32, O.SUM, nthreads=nth, warmup=1, iters=3)
+        out.append({"config": "C1 2x fp32 sum, 64 MiB per buffer, full size", "threads": nth,
+                    "value": round(3 * fa.nbytes / t / 1e9, 3), "unit": "GB/s"})
+    n4 = 16 * 1024 * 1024
+    ins = [rng.integers(-2**31, 2**31 - 1, n4, dtype=np.int64).astype(np.int32) for _ in range(4)]
+    dst = np.empty(n4, dtype=np.int32)
+    for nth in (1, 4):
+        t = O.time_reduce(ins, dst, O.INT32, O.MAX, nthreads=nth, warmup=1, iters=3)
+        out.append({"config": "C4 4x int32 max, 16 Mi-element sample of 128 Mi", "threads": nth,
+                    "value": round(5 * n4 * 4 / t / 1e9, 3), "unit": "GB/s"})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -72,6 +96,8 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=32 * 1024 * 1024,
                     help="elements per input the CPU baseline reduces")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--cpu-configs", action="store_true",
+                    help="cpu_baseline also times the oracle on the C1 and C4 configurations")
     ap.add_argument("--allocator-layout", action="store_true",
                     help="inputs and output as separate torch allocations instead of placed in one")
     ap.add_argument("--rotate-sets", type=int, default=3, metavar="S",
@@ -254,6 +280,8 @@ def main():
         sample = min(args.cpu_sample, N_ELEM)
         base, host, dst = cpu_baseline(bits, sample)
         result["cpu_baseline"] = base
+        if args.cpu_configs:
+            base["other_configs"] = cpu_other_configs()
         # spot check of the GPU result against the oracle on the sample
         got = out[:sample].view(torch.int16).cpu().numpy().view(np.uint16)
         result["spot_check_vs_oracle"] = "bit-exact" if got.tobytes() == dst.tobytes() else "MISMATCH"

@@ -1,6 +1,6 @@
 """Timings of the benchmark configurations other than the headline one, on one GPU:
 
-    python -m flagcx_amd.perf_configs [--json out.json] [--cpu] [--allocator-layout]
+    python -m flagcx_amd.perf_configs [--json out.json] [--allocator-layout]
 
   C1  2-input fp32 sum, 64 MiB per buffer
   C3  fp16 avg reduce-scatter shard (8 ranks x 1 GiB, shard = 128 MiB): one fused
@@ -8,8 +8,8 @@
   C4  4-input int32 max and min, 512 MiB per buffer
 5 warm-up + 20 timed iterations (test/perf/tools.cc:81-86), HIP events, back-to-back
 launches per iteration.  GB/s = (k+1) * n * size / time.  The ranks' buffers of C3 and
-the buffers of C4 sit in one allocation each, at the addresses flagcxLocalPlaceBuffers gives.  --cpu also times the CPU
-oracle (test infrastructure, imported only under this flag) on bounded samples.
+the buffers of C4 sit in one allocation each, at the addresses flagcxLocalPlaceBuffers gives.
+The CPU side of C1 and C4 is timed by bench.py --cpu-configs.
 """
 import argparse
 import json
@@ -56,7 +56,6 @@ def placed(count, nelem, dtype):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", default=None)
-    ap.add_argument("--cpu", action="store_true")
     ap.add_argument("--allocator-layout", action="store_true",
                     help="separate torch allocations instead of buffers placed in different HBM channel groups")
     args = ap.parse_args()
@@ -167,22 +166,6 @@ def main():
         ms = timed(lambda: L.reduce(ins, out, op))
         report("C4 4x int32 %s 512 MiB" % nm, 5 * n * 4, ms)
 
-    if args.cpu:
-        import numpy as np
-        from oracle import cpu_oracle as O
-        sample = 16 * MiB
-        hosts = [t[:sample].cpu().numpy() for t in ins]
-        dst = np.empty(sample, dtype=np.int32)
-        for nth in (1, 4):
-            t = O.time_reduce(hosts, dst, O.INT32, O.MAX, nthreads=nth, warmup=1, iters=3)
-            report("CPU oracle C4 int32 max, %d thread(s), 16 Mi-elem sample" % nth, 5 * sample * 4, t * 1e3)
-        rng = np.random.default_rng(0)
-        fa = rng.uniform(-1, 1, 16 * MiB).astype(np.float32)
-        fb = rng.uniform(-1, 1, 16 * MiB).astype(np.float32)
-        fd = np.empty_like(fa)
-        for nth in (1, 2):
-            t = O.time_reduce([fa, fb], fd, O.FP32, O.SUM, nthreads=nth, warmup=1, iters=3)
-            report("CPU oracle C1 fp32 sum, %d thread(s), full size" % nth, 3 * fa.nbytes, t * 1e3)
     if args.json:
         with open(args.json, "w") as f:
             json.dump(rows, f)
