@@ -47,6 +47,22 @@ inline char *slotOf(flagcxLocalRing *r, size_t step, int peer) {
   return r->buffer + ((step % (size_t)r->steps) * (size_t)r->npeers + (size_t)peer) * r->chunkBytes;
 }
 
+// Steps handed over together.  A hand-over between the producer and the consumer
+// costs about as much as moving a 4 MiB step (an event crossing streams, or a
+// polled one), so full steps travel in groups of four where the ring has room for
+// two such groups in flight and the slots of a group are one contiguous region
+// (every peer region in use).  The last, ragged step always travels alone.
+constexpr size_t kGroup = 4;
+inline size_t groupAt(const flagcxLocalRing *r, int nranks, size_t step, size_t nsteps, size_t size) {
+  if (nranks - 1 != r->npeers || r->steps % (int)kGroup || r->steps < (int)(2 * kGroup) || step % kGroup) return 1;
+  size_t m = nsteps - step < kGroup ? nsteps - step : kGroup;
+  // only whole chunks: a ragged last step leaves the group
+  if ((step + m) * r->chunkBytes > size) m--;
+  // one pack launch takes 64 source regions
+  while (m > 1 && m * (size_t)(nranks - 1) > 64) m--;
+  return m ? m : 1;
+}
+
 } // namespace
 
 #pragma GCC visibility push(default)
@@ -131,28 +147,41 @@ flagcxResult_t flagcxLocalRingReduceScatter(flagcxLocalRing *r, const void *cons
   HCHECK(hipStreamWaitEvent(ps, r->start, 0));
   const size_t size = recvcount * ts;
   const size_t nsteps = (size + r->chunkBytes - 1) / r->chunkBytes;
-  const void *peerSrc[FLAGCX_LOCAL_MAX_RANKS];
-  const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
-  for (size_t step = 0; step < nsteps; step++) {
+  const void *peerSrc[kGroup * FLAGCX_LOCAL_MAX_RANKS];
+  const void *ordered[kGroup][FLAGCX_LOCAL_MAX_RANKS];
+  flagcxLocalReduceDesc descs[kGroup];
+  for (size_t step = 0; step < nsteps;) {
+    const size_t m = groupAt(r, nranks, step, nsteps, size); // steps step .. step+m-1 share one hand-over
     const int slot = (int)(step % (size_t)r->steps);
     const size_t off = step * r->chunkBytes;
-    const size_t n = size - off < r->chunkBytes ? size - off : r->chunkBytes;
+    const size_t n = m > 1 || size - off >= r->chunkBytes ? r->chunkBytes : size - off;
     // ring order rank+1, ..., rank: the first nranks-1 are peers, the last is local
-    for (int j = 0; j < nranks - 1; j++) {
-      const int peer = (rank + 1 + j) % nranks;
-      peerSrc[j] = (const char *)sendbuffs[peer] + (size_t)rank * size + off;
-      ordered[j] = slotOf(r, step, j);
+    for (size_t i = 0; i < m; i++) {
+      for (int j = 0; j < nranks - 1; j++) {
+        const int peer = (rank + 1 + j) % nranks;
+        peerSrc[i * (size_t)(nranks - 1) + j] = (const char *)sendbuffs[peer] + (size_t)rank * size + off + i * n;
+        ordered[i][j] = slotOf(r, step + i, j);
+      }
+      ordered[i][nranks - 1] = (const char *)sendbuffs[rank] + (size_t)rank * size + off + i * n;
     }
-    ordered[nranks - 1] = (const char *)sendbuffs[rank] + (size_t)rank * size + off;
     if (step >= (size_t)r->steps) HCHECK(hipStreamWaitEvent(ps, r->freed[slot], 0));
-    // the slot's peer regions are contiguous: one launch stages all peers' chunks
-    RCHECK(flagcxLocalPackList(slotOf(r, step, 0), peerSrc, nranks - 1, n, copyStream));
+    // the peer regions of a slot, and the slots of a group, are contiguous: one launch stages them all
+    RCHECK(flagcxLocalPackList(slotOf(r, step, 0), peerSrc, (int)(m * (size_t)(nranks - 1)), n, copyStream));
     if (n != r->chunkBytes) // ragged last chunk: regions are n apart after a pack
-      for (int j = 0; j < nranks - 1; j++) ordered[j] = slotOf(r, step, 0) + (size_t)j * n;
+      for (int j = 0; j < nranks - 1; j++) ordered[0][j] = slotOf(r, step, 0) + (size_t)j * n;
     HCHECK(hipEventRecord(r->filled[slot], ps));
     HCHECK(hipStreamWaitEvent(cs, r->filled[slot], 0));
-    RCHECK(flagcxLocalReduce(ordered, nranks, (char *)recvbuff + off, n / ts, datatype, op, stream));
+    for (size_t i = 0; i < m; i++) {
+      descs[i].sendbuffs = ordered[i];
+      descs[i].recvbuff = (char *)recvbuff + off + i * n;
+      descs[i].count = n / ts;
+    }
+    if (m == 1)
+      RCHECK(flagcxLocalReduce(ordered[0], nranks, (char *)recvbuff + off, n / ts, datatype, op, stream));
+    else
+      RCHECK(flagcxLocalReduceBatch(descs, (int)m, nranks, datatype, op, stream));
     HCHECK(hipEventRecord(r->freed[slot], cs));
+    step += m;
   }
   return flagcxSuccess;
 }
@@ -182,25 +211,33 @@ flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing *r, flagcxLocalR
   const size_t nsteps = (size + r->chunkBytes - 1) / r->chunkBytes;
   const size_t depth = (size_t)r->steps;
   std::vector<uint64_t> ticket(depth, 0); // per slot: ticket of the entry that reads it
-  const void *peerSrc[FLAGCX_LOCAL_MAX_RANKS];
+  std::vector<int> lead(depth, 0);        // per slot: the slot whose `filled` event covers its copy
+  const void *peerSrc[kGroup * FLAGCX_LOCAL_MAX_RANKS];
   const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
   size_t copied = 0, handed = 0; // steps whose copy is issued / whose reduce is enqueued
   uint64_t lastTicket = 0, consumed = 0;
   while (handed < nsteps) {
     RCHECK(flagcxLocalReduceFifoQuery(fifo, nullptr, &consumed, nullptr));
-    // issue copies into free slots (sendHead side)
-    while (copied < nsteps && (copied < depth || (copied - depth < handed && consumed >= ticket[copied % depth]))) {
+    // issue copies into free slots (sendHead side), a group of steps per launch and event
+    while (copied < nsteps) {
+      const size_t m = groupAt(r, nranks, copied, nsteps, size);
+      const size_t last = copied + m - 1; // tickets grow with the step: the last slot of the group frees last
+      if (!(last < depth || (last - depth < handed && consumed >= ticket[last % depth]))) break;
       const size_t off = copied * r->chunkBytes;
-      const size_t n = size - off < r->chunkBytes ? size - off : r->chunkBytes;
-      for (int j = 0; j < nranks - 1; j++)
-        peerSrc[j] = (const char *)sendbuffs[(rank + 1 + j) % nranks] + (size_t)rank * size + off;
-      if (nranks > 1) RCHECK(flagcxLocalPackList(slotOf(r, copied, 0), peerSrc, nranks - 1, n, copyStream));
+      const size_t n = m > 1 || size - off >= r->chunkBytes ? r->chunkBytes : size - off;
+      for (size_t i = 0; i < m; i++)
+        for (int j = 0; j < nranks - 1; j++)
+          peerSrc[i * (size_t)(nranks - 1) + j] =
+              (const char *)sendbuffs[(rank + 1 + j) % nranks] + (size_t)rank * size + off + i * n;
+      if (nranks > 1)
+        RCHECK(flagcxLocalPackList(slotOf(r, copied, 0), peerSrc, (int)(m * (size_t)(nranks - 1)), n, copyStream));
       HCHECK(hipEventRecord(r->filled[copied % depth], ps));
-      copied++;
+      for (size_t i = 0; i < m; i++) lead[(copied + i) % depth] = (int)(copied % depth);
+      copied += m;
     }
     // hand on, in order, every step whose copy has completed (recvTail side)
     while (handed < copied) {
-      const hipError_t q = hipEventQuery(r->filled[handed % depth]);
+      const hipError_t q = hipEventQuery(r->filled[lead[handed % depth]]);
       if (q == hipErrorNotReady) break;
       if (q != hipSuccess) return flagcxUnhandledDeviceError;
       const size_t off = handed * r->chunkBytes;

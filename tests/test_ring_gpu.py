@@ -50,6 +50,9 @@ def test_ring_send_recv(L, size, chunk, steps):
     (O.BF16, O.SUM, 8, 1 << 20, 1 << 18, 16),
     (O.FP16, O.AVG, 8, (1 << 21) + 24, 0, 0),     # default 16 x 4 MiB ring
     (O.INT32, O.MAX, 2, 5000, 4096, 2),
+    (O.FP32, O.SUM, 8, 1024 * 37 + 25, 4096, 8),  # steps travel in groups of four: many wraps, 37 whole steps + a ragged one
+    (O.BF16, O.SUM, 8, 2048 * 70, 4096, 16),      # 70 whole steps, the last group of two
+    (O.INT32, O.MIN, 5, 1024 * 9 + 1, 4096, 8),   # groups in a ring with every peer region in use, 5 ranks
 ])
 def test_ring_reduce_scatter_equals_direct(L, dt, op, nranks, rcount, chunk, steps):
     import torch
@@ -80,6 +83,8 @@ def test_ring_reduce_scatter_equals_direct(L, dt, op, nranks, rcount, chunk, ste
     (O.FP16, O.AVG, 8, (1 << 21) + 24, 0, 0),     # default 16 x 4 MiB ring
     (O.INT32, O.MAX, 2, 5000, 4096, 2),
     (O.INT64, O.MIN, 3, 70001, 8192, 3),
+    (O.FP32, O.SUM, 8, 1024 * 37 + 25, 4096, 8),  # grouped steps, many wraps, ragged end
+    (O.BF16, O.SUM, 8, 2048 * 70, 4096, 16),
 ])
 def test_ring_reduce_scatter_through_the_reduce_queue(L, dt, op, nranks, rcount, chunk, steps):
     """Proxy-style progress: copies on one stream, polled events, reduces through the
