@@ -53,13 +53,13 @@ inline char *slotOf(flagcxLocalRing *r, size_t step, int peer) {
 // two such groups in flight and the slots of a group are one contiguous region
 // (every peer region in use).  The last, ragged step always travels alone.
 constexpr size_t kGroup = 4;
-inline size_t groupAt(const flagcxLocalRing *r, int nranks, size_t step, size_t nsteps, size_t size) {
-  if (nranks - 1 != r->npeers || r->steps % (int)kGroup || r->steps < (int)(2 * kGroup) || step % kGroup) return 1;
+inline size_t groupAt(const flagcxLocalRing *r, int regions, size_t step, size_t nsteps, size_t size) {
+  if (regions != r->npeers || r->steps % (int)kGroup || r->steps < (int)(2 * kGroup) || step % kGroup) return 1;
   size_t m = nsteps - step < kGroup ? nsteps - step : kGroup;
   // only whole chunks: a ragged last step leaves the group
   if ((step + m) * r->chunkBytes > size) m--;
   // one pack launch takes 64 source regions
-  while (m > 1 && m * (size_t)(nranks - 1) > 64) m--;
+  while (m > 1 && m * (size_t)regions > 64) m--;
   return m ? m : 1;
 }
 
@@ -114,16 +114,18 @@ flagcxResult_t flagcxLocalRingSendRecv(flagcxLocalRing *r, void *dst, const void
   HCHECK(hipEventRecord(r->start, cs)); // what the consumer stream produced so far is the sender's input
   HCHECK(hipStreamWaitEvent(ps, r->start, 0));
   const size_t nsteps = (size + r->chunkBytes - 1) / r->chunkBytes; // chunkSteps (flagcx/core/group.cc:179-181)
-  for (size_t step = 0; step < nsteps; step++) {
+  for (size_t step = 0; step < nsteps;) {
+    const size_t m = groupAt(r, 1, step, nsteps, size); // whole steps in consecutive slots share one hand-over
     const int slot = (int)(step % (size_t)r->steps);
     const size_t off = step * r->chunkBytes;
-    const size_t n = size - off < r->chunkBytes ? size - off : r->chunkBytes;
+    const size_t n = m > 1 ? m * r->chunkBytes : (size - off < r->chunkBytes ? size - off : r->chunkBytes);
     if (step >= (size_t)r->steps) HCHECK(hipStreamWaitEvent(ps, r->freed[slot], 0)); // recvTail > copied
     RCHECK(flagcxLocalMemcpy(slotOf(r, step, 0), (const char *)src + off, n, copyStream));
     HCHECK(hipEventRecord(r->filled[slot], ps));                                       // sendHead
     HCHECK(hipStreamWaitEvent(cs, r->filled[slot], 0));
     RCHECK(flagcxLocalMemcpy((char *)dst + off, slotOf(r, step, 0), n, stream));
     HCHECK(hipEventRecord(r->freed[slot], cs));                                        // recvTail
+    step += m;
   }
   return flagcxSuccess;
 }
@@ -151,7 +153,7 @@ flagcxResult_t flagcxLocalRingReduceScatter(flagcxLocalRing *r, const void *cons
   const void *ordered[kGroup][FLAGCX_LOCAL_MAX_RANKS];
   flagcxLocalReduceDesc descs[kGroup];
   for (size_t step = 0; step < nsteps;) {
-    const size_t m = groupAt(r, nranks, step, nsteps, size); // steps step .. step+m-1 share one hand-over
+    const size_t m = groupAt(r, nranks - 1, step, nsteps, size); // steps step .. step+m-1 share one hand-over
     const int slot = (int)(step % (size_t)r->steps);
     const size_t off = step * r->chunkBytes;
     const size_t n = m > 1 || size - off >= r->chunkBytes ? r->chunkBytes : size - off;
@@ -220,7 +222,7 @@ flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing *r, flagcxLocalR
     RCHECK(flagcxLocalReduceFifoQuery(fifo, nullptr, &consumed, nullptr));
     // issue copies into free slots (sendHead side), a group of steps per launch and event
     while (copied < nsteps) {
-      const size_t m = groupAt(r, nranks, copied, nsteps, size);
+      const size_t m = groupAt(r, nranks - 1, copied, nsteps, size);
       const size_t last = copied + m - 1; // tickets grow with the step: the last slot of the group frees last
       if (!(last < depth || (last - depth < handed && consumed >= ticket[last % depth]))) break;
       const size_t off = copied * r->chunkBytes;

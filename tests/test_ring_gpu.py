@@ -27,7 +27,8 @@ def streams(L):
 
 
 @pytest.mark.parametrize("size,chunk,steps", [(1, 4096, 4), (4096 * 3, 4096, 4), (4096 * 37 + 100, 4096, 4),
-                                              (1 << 20, 65536, 16), ((9 << 20) + 16, 0, 0)])
+                                              (1 << 20, 65536, 16), ((9 << 20) + 16, 0, 0),
+                                              (4096 * 70 + 7, 4096, 8), (4096 * 40, 4096, 16)])   # steps in groups of four, wraps
 def test_ring_send_recv(L, size, chunk, steps):
     import torch
     ring_mem = torch.empty((steps or 16) * (chunk or L.CHUNKSIZE), dtype=torch.uint8, device="cuda")
