@@ -49,13 +49,16 @@ inline char *slotOf(flagcxLocalRing *r, size_t step, int peer) {
 
 // Steps handed over together.  A hand-over between the producer and the consumer
 // costs about as much as moving a 4 MiB step (an event crossing streams, or a
-// polled one), so full steps travel in groups of four where the ring has room for
-// two such groups in flight and the slots of a group are one contiguous region
+// polled one), so full steps travel in groups of up to eight: half the ring, which
+// leaves two groups in flight, where the slots of a group are one contiguous region
 // (every peer region in use).  The last, ragged step always travels alone.
-constexpr size_t kGroup = 4;
+constexpr size_t kGroup = 8;
 inline size_t groupAt(const flagcxLocalRing *r, int regions, size_t step, size_t nsteps, size_t size) {
-  if (regions != r->npeers || r->steps % (int)kGroup || r->steps < (int)(2 * kGroup) || step % kGroup) return 1;
-  size_t m = nsteps - step < kGroup ? nsteps - step : kGroup;
+  if (regions != r->npeers) return 1;
+  size_t g = kGroup;
+  while (g > 1 && ((size_t)r->steps % g || (size_t)r->steps < 2 * g)) g >>= 1;
+  if (g == 1 || step % g) return 1;
+  size_t m = nsteps - step < g ? nsteps - step : g;
   // only whole chunks: a ragged last step leaves the group
   if ((step + m) * r->chunkBytes > size) m--;
   // one pack launch takes 64 source regions

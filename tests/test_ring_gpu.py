@@ -28,7 +28,7 @@ def streams(L):
 
 @pytest.mark.parametrize("size,chunk,steps", [(1, 4096, 4), (4096 * 3, 4096, 4), (4096 * 37 + 100, 4096, 4),
                                               (1 << 20, 65536, 16), ((9 << 20) + 16, 0, 0),
-                                              (4096 * 70 + 7, 4096, 8), (4096 * 40, 4096, 16)])   # steps in groups of four, wraps
+                                              (4096 * 70 + 7, 4096, 8), (4096 * 40, 4096, 16)])   # steps in groups of half the ring, wraps
 def test_ring_send_recv(L, size, chunk, steps):
     import torch
     ring_mem = torch.empty((steps or 16) * (chunk or L.CHUNKSIZE), dtype=torch.uint8, device="cuda")
@@ -51,7 +51,7 @@ def test_ring_send_recv(L, size, chunk, steps):
     (O.BF16, O.SUM, 8, 1 << 20, 1 << 18, 16),
     (O.FP16, O.AVG, 8, (1 << 21) + 24, 0, 0),     # default 16 x 4 MiB ring
     (O.INT32, O.MAX, 2, 5000, 4096, 2),
-    (O.FP32, O.SUM, 8, 1024 * 37 + 25, 4096, 8),  # steps travel in groups of four: many wraps, 37 whole steps + a ragged one
+    (O.FP32, O.SUM, 8, 1024 * 37 + 25, 4096, 8),  # steps travel in groups of four here: many wraps, 37 whole steps + a ragged one
     (O.BF16, O.SUM, 8, 2048 * 70, 4096, 16),      # 70 whole steps, the last group of two
     (O.INT32, O.MIN, 5, 1024 * 9 + 1, 4096, 8),   # groups in a ring with every peer region in use, 5 ranks
 ])
