@@ -153,7 +153,26 @@ def main():
             L.reduce_scatter(send, rk, recv, L.RedOp.Avg)
     ms = timed(all_shards, warmup=2, iters=5)
     report("C3 all 8 shards (8 fused launches, 1 GiB out)", 8 * nb, ms)
-    del send, recv, send_pool
+
+    # The stage after it in an all-reduce: every rank holds one reduced slice in a buffer of the
+    # full size.  The reference zero-fills the rest of each buffer and sum-all-reduces the buffers
+    # (flagcx/core/c2c_algo.cc:586-608 + :310-336); rank-local primitives copy the eight slices into place.
+    full = torch.empty(per_rank, dtype=torch.float16, device="cuda")
+
+    def refresh_and_sum():
+        for rk in range(nranks):
+            L.refresh(send[rk], 0, rk * shard, shard, per_rank, L.RedOp.Sum)
+        L.reduce(send, full, L.RedOp.Sum)
+    ms = timed(refresh_and_sum, warmup=2, iters=5)
+    traffic = nranks * (per_rank - shard) * 2 + (nranks + 1) * per_rank * 2
+    report("C3 gather of the 8 slices: zero-fill + 8-input sum", traffic, ms, "1 GiB result")
+
+    def copy_slices():
+        for rk in range(nranks):
+            L.memcpy(full.data_ptr() + rk * shard * 2, send[rk].data_ptr() + rk * shard * 2, shard * 2)
+    ms = timed(copy_slices, warmup=2, iters=5)
+    report("C3 gather of the 8 slices: 8 slice copies", 2 * per_rank * 2, ms, "1 GiB result")
+    del send, recv, send_pool, full
 
     # C4
     n = 128 * MiB
