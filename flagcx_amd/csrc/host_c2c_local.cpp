@@ -228,6 +228,25 @@ static char *pick(const Bufs &b, int rank, int type) {
     if (r_ != flagcxSuccess) return r_;                                        \
   } while (0)
 
+// n blocks of `bytes` from the pointers in `src` into dst, back to back: one launch
+// unless a block already lies inside the destination (in-place all-gather,
+// flagcx/include/flagcx.h:373), which the list copy refuses; then block by block,
+// where a copy onto itself is nothing.
+static flagcxResult_t gatherBlocks(char *dst, const std::vector<const void *> &src, size_t bytes, flagcxStream_t stream) {
+  const int n = (int)src.size();
+  bool inside = n > 64;
+  for (int j = 0; j < n && !inside; j++) {
+    const char *s = (const char *)src[j];
+    inside = s < dst + (size_t)n * bytes && dst < s + bytes;
+  }
+  if (!inside) return flagcxLocalPackList(dst, src.data(), n, bytes, stream);
+  for (int j = 0; j < n; j++) {
+    const flagcxResult_t r = flagcxLocalMemcpy(dst + (size_t)j * bytes, src[j], bytes, stream);
+    if (r != flagcxSuccess) return r;
+  }
+  return flagcxSuccess;
+}
+
 // One homo function slot (step s, index i of one table) across all ranks.
 static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const HomoFunc *> &fn, const Bufs &b,
                                   flagcxDataType_t dt, int root, flagcxStream_t stream) {
@@ -306,15 +325,15 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
         LCHECK(flagcxLocalReduceBatch(descs.data(), n, n, dt, rop, stream));
         break;
       }
-      case flagcxCommOpAllGather:
-        for (int h = 0; h < n; h++)
-          for (int j = 0; j < n; j++)
-            LCHECK(flagcxLocalMemcpy(D[h] + (size_t)j * count * ts, S[j], count * ts, stream));
+      case flagcxCommOpAllGather: {
+        const std::vector<const void *> blocks(S.begin(), S.end());
+        for (int h = 0; h < n; h++) LCHECK(gatherBlocks(D[h], blocks, count * ts, stream));
         break;
+      }
       case flagcxCommOpGather: {
         const int rt = homoRoot(first);
         if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
-        for (int j = 0; j < n; j++) LCHECK(flagcxLocalMemcpy(D[rt] + (size_t)j * count * ts, S[j], count * ts, stream));
+        LCHECK(gatherBlocks(D[rt], std::vector<const void *>(S.begin(), S.end()), count * ts, stream));
         break;
       }
       case flagcxCommOpScatter: {
@@ -329,11 +348,14 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
         for (int h = 0; h < n; h++) LCHECK(flagcxLocalMemcpy(D[h], S[rt], count * ts, stream));
         break;
       }
-      case flagcxCommOpAlltoAll:
-        for (int h = 0; h < n; h++)
-          for (int j = 0; j < n; j++)
-            LCHECK(flagcxLocalMemcpy(D[h] + (size_t)j * count * ts, S[j] + (size_t)h * count * ts, count * ts, stream));
+      case flagcxCommOpAlltoAll: {
+        std::vector<const void *> blocks(n);
+        for (int h = 0; h < n; h++) {
+          for (int j = 0; j < n; j++) blocks[j] = S[j] + (size_t)h * count * ts;
+          LCHECK(gatherBlocks(D[h], blocks, count * ts, stream));
+        }
         break;
+      }
       case flagcxCommNoOp:
         break;
       default:
