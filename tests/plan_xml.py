@@ -111,3 +111,12 @@ def allreduce_2x2_reference_ops_only(prefix):
             het = [[[p2p(r, (r + 1) % 4, 0, 4, 1)]]]
         inter = [[homo(ALLREDUCE, 1, 1, 0, 0, 4, 1)]]
         write_rank(prefix, r, 4, (1, 0, 1, 0, 0), refresh, pre, het, inter, [])
+
+
+def one_cluster_collective(prefix, commop, nranks=4, root=2):
+    """One cluster of `nranks`, one homo step from the user send buffer (type 0) into recv
+    (type 1): all-gather / gather of one chunk per rank, or all-to-all of one chunk per pair.
+    nChunks = nranks, so a chunk is totalCount / nranks elements."""
+    for r in range(nranks):
+        pre = [[homo(commop, 0, 1, 0, 0, 1, 0, rootRank=root if commop == GATHER else -1)]]
+        write_rank(prefix, r, nranks, (1, 0, 0, 0, 0), NO_REFRESH, pre, [], [], [])

@@ -94,3 +94,33 @@ def test_plan_execute_allreduce_2x2(tmp_path, maker, scratch, dt):
     for r in range(4):
         assert same(from_dev(recv[r], npdt), want), (maker.__name__, r)
         assert torch.equal(send[r], keep[r])                        # user send buffers untouched
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("commop", [PX.ALLGATHER, PX.GATHER, PX.ALLTOALL], ids=["allgather", "gather", "alltoall"])
+def test_plan_execute_one_cluster_block_moves(tmp_path, commop):
+    """Out-of-place block movers of one cluster (four ranks): every destination is filled by
+    one list copy; bytes compared with numpy slicing."""
+    import torch
+    nranks, chunk, root = 4, 30001, 2
+    prefix = str(tmp_path / "plan")
+    PX.one_cluster_collective(prefix, commop, nranks, root)
+    n = nranks * chunk
+    plan = local.Plan([0] * nranks, n, commop, local.RedOp.Sum)
+    plan.import_xml(prefix)
+    rng = np.random.default_rng(commop)
+    hosts = [rng.integers(-2**30, 2**30, n, dtype=np.int32) for _ in range(nranks)]
+    send = [to_dev(h) for h in hosts]
+    recv = [dev_empty(n, 4, fill=0x55) for _ in range(nranks)]
+    plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, O.INT32, root=root)
+    torch.cuda.synchronize()
+    untouched = np.full(n, 0x55, dtype=np.int32)
+    for r in range(nranks):
+        got = from_dev(recv[r], np.int32)
+        if commop == PX.ALLGATHER:
+            want = np.concatenate([hosts[j][:chunk] for j in range(nranks)])
+        elif commop == PX.GATHER:
+            want = np.concatenate([hosts[j][:chunk] for j in range(nranks)]) if r == root else untouched
+        else:
+            want = np.concatenate([hosts[j][r * chunk:(r + 1) * chunk] for j in range(nranks)])
+        assert same(got, want), (commop, r)
