@@ -97,10 +97,11 @@ def test_plan_execute_allreduce_2x2(tmp_path, maker, scratch, dt):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("commop", [PX.ALLGATHER, PX.GATHER, PX.ALLTOALL], ids=["allgather", "gather", "alltoall"])
+@pytest.mark.parametrize("commop", [PX.ALLGATHER, PX.GATHER, PX.ALLTOALL, PX.SCATTER, PX.BROADCAST],
+                         ids=["allgather", "gather", "alltoall", "scatter", "broadcast"])
 def test_plan_execute_one_cluster_block_moves(tmp_path, commop):
-    """Out-of-place block movers of one cluster (four ranks): every destination is filled by
-    one list copy; bytes compared with numpy slicing."""
+    """Out-of-place block movers of one cluster (four ranks): gathers fill every destination
+    with one list copy; bytes compared with numpy slicing, the rest of recv untouched."""
     import torch
     nranks, chunk, root = 4, 30001, 2
     prefix = str(tmp_path / "plan")
@@ -121,6 +122,10 @@ def test_plan_execute_one_cluster_block_moves(tmp_path, commop):
             want = np.concatenate([hosts[j][:chunk] for j in range(nranks)])
         elif commop == PX.GATHER:
             want = np.concatenate([hosts[j][:chunk] for j in range(nranks)]) if r == root else untouched
-        else:
+        elif commop == PX.ALLTOALL:
             want = np.concatenate([hosts[j][r * chunk:(r + 1) * chunk] for j in range(nranks)])
+        elif commop == PX.SCATTER:
+            want = np.concatenate([hosts[root][r * chunk:(r + 1) * chunk], untouched[chunk:]])
+        else:
+            want = np.concatenate([hosts[root][:chunk], untouched[chunk:]])
         assert same(got, want), (commop, r)
