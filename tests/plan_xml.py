@@ -118,5 +118,5 @@ def one_cluster_collective(prefix, commop, nranks=4, root=2):
     (type 1): all-gather / gather of one chunk per rank, or all-to-all of one chunk per pair.
     nChunks = nranks, so a chunk is totalCount / nranks elements."""
     for r in range(nranks):
-        pre = [[homo(commop, 0, 1, 0, 0, 1, 0, rootRank=root if commop == GATHER else -1)]]
+        pre = [[homo(commop, 0, 1, 0, 0, 1, 0, rootRank=root if commop in (GATHER, REDUCE) else -1)]]
         write_rank(prefix, r, nranks, (1, 0, 0, 0, 0), NO_REFRESH, pre, [], [], [])

@@ -97,8 +97,9 @@ def test_plan_execute_allreduce_2x2(tmp_path, maker, scratch, dt):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("commop", [PX.ALLGATHER, PX.GATHER, PX.ALLTOALL, PX.SCATTER, PX.BROADCAST],
-                         ids=["allgather", "gather", "alltoall", "scatter", "broadcast"])
+@pytest.mark.parametrize("commop", [PX.ALLGATHER, PX.GATHER, PX.ALLTOALL, PX.SCATTER, PX.BROADCAST, PX.REDUCE,
+                                    PX.REDUCESCATTER],
+                         ids=["allgather", "gather", "alltoall", "scatter", "broadcast", "reduce", "reducescatter"])
 def test_plan_execute_one_cluster_block_moves(tmp_path, commop):
     """Out-of-place block movers of one cluster (four ranks): gathers fill every destination
     with one list copy; bytes compared with numpy slicing, the rest of recv untouched."""
@@ -110,7 +111,7 @@ def test_plan_execute_one_cluster_block_moves(tmp_path, commop):
     plan = local.Plan([0] * nranks, n, commop, local.RedOp.Sum)
     plan.import_xml(prefix)
     rng = np.random.default_rng(commop)
-    hosts = [rng.integers(-2**30, 2**30, n, dtype=np.int32) for _ in range(nranks)]
+    hosts = [rng.integers(-2**28, 2**28, n, dtype=np.int32) for _ in range(nranks)]
     send = [to_dev(h) for h in hosts]
     recv = [dev_empty(n, 4, fill=0x55) for _ in range(nranks)]
     plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, O.INT32, root=root)
@@ -126,6 +127,10 @@ def test_plan_execute_one_cluster_block_moves(tmp_path, commop):
             want = np.concatenate([hosts[j][r * chunk:(r + 1) * chunk] for j in range(nranks)])
         elif commop == PX.SCATTER:
             want = np.concatenate([hosts[root][r * chunk:(r + 1) * chunk], untouched[chunk:]])
-        else:
+        elif commop == PX.BROADCAST:
             want = np.concatenate([hosts[root][:chunk], untouched[chunk:]])
+        elif commop == PX.REDUCE:   # int32 sums of values below 2^28 in magnitude: no overflow for four ranks
+            want = np.concatenate([sum(h[:chunk] for h in hosts), untouched[chunk:]]) if r == root else untouched
+        else:
+            want = np.concatenate([sum(h[r * chunk:(r + 1) * chunk] for h in hosts), untouched[chunk:]])
         assert same(got, want), (commop, r)
