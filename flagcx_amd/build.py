@@ -41,6 +41,7 @@ def build(verbose=False, jobs=None):
     units.append((os.path.join(CSRC, "copy_kernels.hip"), os.path.join(OBJ, "copy_kernels.o"), []))
     units.append((os.path.join(CSRC, "async_kernels.hip"), os.path.join(OBJ, "async_kernels.o"), []))
     units.append((os.path.join(CSRC, "fifo_kernels.hip"), os.path.join(OBJ, "fifo_kernels.o"), []))
+    units.append((os.path.join(CSRC, "static_staging.hip"), os.path.join(OBJ, "static_staging.o"), []))
     units.append((os.path.join(CSRC, "c_api.cpp"), os.path.join(OBJ, "c_api.o"), ["-x", "hip"]))
     extra = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.startswith("host_") and f.endswith(".cpp")]
     for f in extra:

@@ -26,6 +26,8 @@ static flagcxResult_t fail(flagcxResult_t code, const char *fmt, ...) {
   return code;
 }
 
+void setLastError(const char *text) { snprintf(tlsLastError, sizeof(tlsLastError), "%s", text ? text : ""); }
+
 static flagcxResult_t fromHip(int err, const char *what) {
   if (err == (int)hipSuccess) return flagcxSuccess;
   // any runtime error maps to one code, like DEVCHECK
@@ -310,7 +312,8 @@ size_t flagcxLocalGetDataTypeSize(flagcxDataType_t dtype) { return typeSize(bits
 flagcxResult_t flagcxLocalInit(void) {
   (void)deviceInfo();
   if (gInfoErr) return fromHip(gInfoErr, "flagcxLocalInit");
-  return flagcxSuccess;
+  // the staging area of flagcxLocalStagedReduceScatterNoAlloc on this device
+  return (flagcxResult_t)resolveStaticStaging();
 }
 
 const char *flagcxLocalGetErrorString(flagcxResult_t result) {

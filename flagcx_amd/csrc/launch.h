@@ -108,4 +108,10 @@ struct Copy2D {
 int launchCopy2D(const Copy2D &c);
 int launchFill(void *p0, uint64_t n0, void *p1, uint64_t n1, int value, hipStream_t stream);
 
+// Text that flagcxLocalGetLastError returns to the calling thread (c_api.cpp).
+void setLastError(const char *text);
+// Looks up, for the current device, the library's static staging area
+// (static_staging.hip); returns a flagcxResult_t value.
+int resolveStaticStaging();
+
 } // namespace flagcx_amd

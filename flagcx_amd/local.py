@@ -130,7 +130,7 @@ EXPORTS = [
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
     "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoSetLinger", "flagcxLocalReduceFifoSetWindow", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
-    "flagcxLocalReduceFifoGetLastError",
+    "flagcxLocalReduceFifoGetLastError", "flagcxLocalStagedReduceScatterNoAlloc",
 ]
 
 
@@ -185,6 +185,7 @@ def lib():
         L.flagcxLocalRingDestroy.argtypes = [vp]
         L.flagcxLocalRingSendRecv.argtypes = [vp, vp, vp, sz, sp, sp]
         L.flagcxLocalRingReduceScatter.argtypes = [vp, pp, i, i, vp, sz, i, i, sp, sp]
+        L.flagcxLocalStagedReduceScatterNoAlloc.argtypes = [pp, i, i, vp, sz, i, i, sp]
         L.flagcxLocalGetDeviceAdaptor.restype = vp
         L.flagcxLocalGetDeviceAdaptor.argtypes = []
         L.flagcxLocalDeviceAdaptorLayout.argtypes = [C.POINTER(sz), i]
@@ -292,6 +293,19 @@ def reduce_scatter(sendbuffs, rank, recv, op, dtype=None, chunkbytes=None, strea
     else:
         check(lib().flagcxLocalReduceScatterChunked(ptrs, len(sendbuffs), rank, recv.data_ptr(), recv.numel(),
                                                     int(dt), int(op), chunkbytes, _sref(st)))
+    return recv
+
+
+STATIC_STAGING_BYTES = 8 * 1024 * 1024
+
+
+def staged_reduce_scatter_noalloc(sendbuffs, rank, recv, op, dtype=None, stream="current"):
+    """flagcxLocalStagedReduceScatterNoAlloc: peers' slices staged in the library's static area."""
+    st = current_stream() if stream == "current" else stream
+    dt = dtype_of(recv, dtype)
+    check(lib().flagcxLocalStagedReduceScatterNoAlloc(_ptr_array([s.data_ptr() for s in sendbuffs]), len(sendbuffs),
+                                                      rank, recv.data_ptr(), recv.numel(), int(dt), int(op),
+                                                      _sref(st)))
     return recv
 
 

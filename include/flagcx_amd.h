@@ -117,8 +117,10 @@ size_t flagcxLocalGetDataTypeSize(flagcxDataType_t dtype);
 /* Library                                                                    */
 /* ------------------------------------------------------------------------- */
 
-/* Caches the properties of the current device (CU count).  Optional: every
- * entry point does this on first use.  Thread-safe. */
+/* Caches the properties of the current device (CU count) and looks up where the
+ * library's static staging area lives on it (flagcxLocalStagedReduceScatterNoAlloc).
+ * Optional: every entry point does its part on first use.  Call it once per device,
+ * with that device current, before capturing graphs there.  Thread-safe. */
 flagcxResult_t flagcxLocalInit(void);
 
 /* Static string for a result code (never NULL). */
@@ -490,6 +492,27 @@ flagcxResult_t flagcxLocalRingReduceScatter(flagcxLocalRing_t ring, const void *
 flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing_t ring, flagcxLocalReduceFifo_t fifo,
                                                 const void *const *sendbuffs, int nranks, int rank,
                                                 void *recvbuff, size_t recvcount, flagcxStream_t copyStream);
+
+/* No counterpart in the reference: this entry point exists for callers that cannot
+ * allocate - code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc - and so can neither create a ring (events) nor bring a ring
+ * buffer.  It is flagcxLocalRingReduceScatter on ONE stream with the staging slots
+ * in a fixed area inside the library's own device image
+ * (FLAGCX_LOCAL_STATIC_STAGING_BYTES per GPU, held from the moment the library's
+ * code is loaded on that GPU until the process ends): one launch stages the
+ * nranks-1 peers' slices of shard `rank` there, one reduce folds them with the
+ * local slice into recvbuff, in the ring's order rank+1, ..., rank - the same
+ * bytes as flagcxLocalRingReduceScatter and flagcxLocalReduceScatter.  Calls no
+ * hipMalloc / hipFree and creates no stream or event.
+ * Limit: (nranks - 1) * roundUp(recvcount * elementSize + (recvbuff mod 16), 256)
+ * <= FLAGCX_LOCAL_STATIC_STAGING_BYTES, else flagcxInvalidArgument.  Every call on
+ * a GPU uses that GPU's one staging area: calls on one stream follow one another;
+ * calls that overlap in time on different streams of one GPU race on it. */
+#define FLAGCX_LOCAL_STATIC_STAGING_BYTES (8ULL * 1024 * 1024)
+flagcxResult_t flagcxLocalStagedReduceScatterNoAlloc(const void *const *sendbuffs, int nranks, int rank,
+                                                     void *recvbuff, size_t recvcount,
+                                                     flagcxDataType_t datatype, flagcxRedOp_t op,
+                                                     flagcxStream_t stream);
 
 /* ------------------------------------------------------------------------- */
 /* C2C plan replay on one GPU                                                  */
