@@ -222,14 +222,14 @@ flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int ca
   q->dtype = dt;
   q->op = rop;
   q->typeSize = ts;
-  // Measured on MI355X (64 x 4 MiB chunks per input, 6..16 wavefronts per CU): few
-  // inputs want more wavefronts in flight, many inputs fewer (two inputs 3.6 -> 5.1
-  // TB/s from 6 to 16, eight 6.0 / 6.1 / 5.8 at 6 / 10 / 16); never more than half a
-  // CU's slots, so that residency does not depend on the last slot being free.  (A
-  // limit on the inputs a worker has in flight, which the launched kernels use for
-  // large reduces, only costs here: 16 wavefronts per CU cannot cover the longer
-  // life of each.)
-  static const int kWaves[9] = {16, 16, 16, 16, 14, 14, 14, 10, 10};
+  // Measured on MI355X (32 x 4 MiB chunks per input): with the workers' units of
+  // 8 / 4 / 1 KiB per input for up to 2 / up to 4 / more inputs, about 64-80 KiB of
+  // loads in flight per CU are enough (two inputs 5.5 / 5.6 / 6.0 TB/s at 16 / 12 / 8
+  // wavefronts per CU, four 5.7 / 6.0 at 14 / 10, eight 6.0 / 6.0 / 5.8 at 8 / 10 / 14);
+  // never more than half a CU's slots, so that residency does not depend on the last
+  // slot being free.  (A limit on the inputs a worker has in flight, which the
+  // launched kernels use for large reduces, only costs here.)
+  static const int kWaves[9] = {8, 8, 8, 10, 10, 10, 10, 10, 10};
   q->wavesPerCU = kWaves[maxRanks];
   const DeviceInfo &info = deviceInfo();
   q->maxGrid = (unsigned)info.numCU * 16u;

@@ -273,37 +273,53 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
   }
 }
 
-// This worker's KiB tiles of one entry, K inputs known at compile time.  ALIGNED:
+// Tiles per unit.  A worker folds one unit at a time: G consecutive KiB tiles of
+// every input, all G*K loads issued before the first use.  Few inputs take several
+// tiles at a time, so that a wavefront keeps as many bytes in flight as one with
+// many inputs does and reads an entry's descriptor once per 8 KiB instead of once
+// per KiB (two fp32 inputs, 32 entries of 4 MiB: 4.6 -> 5.9 TB/s).
+constexpr int queueUnitTiles(int k) { return k <= 2 ? 8 : k <= 4 ? 4 : 1; }
+
+// This worker's units of one entry, K inputs known at compile time.  ALIGNED:
 // every pointer agrees modulo 16 and tiles go through clipped buffer descriptors;
 // otherwise the destination's tiling with unaligned 16-byte loads.
-template <typename T, int OP, int K, bool ALIGNED>
+template <typename T, int OP, int K, int G, bool ALIGNED>
 __device__ __forceinline__ void queueTiles(const uint64_t (&src)[8], uint64_t dst, uint64_t headBytes,
                                            uint64_t bodyBytes, uint64_t first, uint64_t stride) {
+  constexpr uint32_t kUnitBytes = 1024u * G;
   const uint32_t voff = threadIdx.x * 16u;
-  const uint64_t ntiles = (bodyBytes + 1023) / 1024;
-  for (uint64_t t = first; t < ntiles; t += stride) {
-    const uint64_t off = headBytes + t * 1024;
-    const uint64_t left = bodyBytes - t * 1024;
-    const uint32_t span = left < 1024 ? (uint32_t)left : 1024u;
-    u32x4 in[K];
+  const uint64_t nunits = (bodyBytes + kUnitBytes - 1) / kUnitBytes;
+  for (uint64_t u = first; u < nunits; u += stride) {
+    const uint64_t off = headBytes + u * kUnitBytes;
+    const uint64_t left = bodyBytes - u * kUnitBytes;
+    const uint32_t span = left < kUnitBytes ? (uint32_t)left : kUnitBytes;
+    u32x4 in[G][K];
     if (ALIGNED) {
 #pragma unroll
       for (int j = 0; j < K; j++) {
         __amdgpu_buffer_rsrc_t rs =
             __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)(src[j] + off), 0, span, kRsrcFlags);
-        in[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kCoherentLoadAux);
+#pragma unroll
+        for (int g = 0; g < G; g++)
+          in[g][j] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + g * 1024u, 0, kCoherentLoadAux);
       }
-      __amdgpu_buffer_rsrc_t rd =
-          __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)(dst + off), 0, span, kRsrcFlags);
-      __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, voff, 0, kCoherentStoreAux);
-    } else if (voff < span) {
+    } else {
 #pragma unroll
       for (int j = 0; j < K; j++)
-        in[j] = __builtin_nontemporal_load((const u32x4_unaligned *)(uintptr_t)(src[j] + off + voff));
-      __amdgpu_buffer_rsrc_t rd =
-          __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)(dst + off), 0, span, kRsrcFlags);
-      __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, voff, 0, kCoherentStoreAux);
+#pragma unroll
+        for (int g = 0; g < G; g++)
+          in[g][j] = voff + g * 1024u < span
+                         ? __builtin_nontemporal_load(
+                               (const u32x4_unaligned *)(uintptr_t)(src[j] + off + voff + g * 1024u))
+                         : u32x4{0, 0, 0, 0};
     }
+    __amdgpu_buffer_rsrc_t rd =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)(dst + off), 0, span, kRsrcFlags);
+#pragma unroll
+    for (int g = 0; g < G; g++)
+      if (ALIGNED || voff + g * 1024u < span)
+        __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in[g], K), rd, voff + g * 1024u, 0,
+                                               kCoherentStoreAux);
   }
 }
 
@@ -311,15 +327,16 @@ template <typename T, int OP, int K>
 __device__ __forceinline__ void queueEntry(const uint64_t (&src)[8], uint64_t dst, uint32_t head, uint32_t tail,
                                            uint64_t nvec, bool aligned, uint64_t first, uint64_t stride) {
   constexpr int N = 16 / sizeof(T);
+  constexpr int G = queueUnitTiles(K);
   const uint64_t headBytes = (uint64_t)head * sizeof(T);
   if (aligned) {
-    queueTiles<T, OP, K, true>(src, dst, headBytes, nvec * 16, first, stride);
+    queueTiles<T, OP, K, G, true>(src, dst, headBytes, nvec * 16, first, stride);
   } else {
     // plain global loads carry no scope bits: drop whatever this CU and L2 hold
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-    queueTiles<T, OP, K, false>(src, dst, headBytes, nvec * 16, first, stride);
+    queueTiles<T, OP, K, G, false>(src, dst, headBytes, nvec * 16, first, stride);
   }
-  // head and tail elements: the worker that owns tile 0, one lane each
+  // head and tail elements: the worker that owns unit 0, one lane each
   if (first == 0 && threadIdx.x < head + tail) {
     const uint64_t i = threadIdx.x < head ? threadIdx.x : head + nvec * N + (threadIdx.x - head);
     typedef Fold<T, OP> F;
@@ -336,7 +353,7 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
   const uint32_t worker = blockIdx.x - 1;
   uint64_t done = 0; // entries this worker has finished since this launch (entry index = q.base + done)
   uint64_t lastBeat = 0;
-  uint32_t rot = 0;  // tiles handed out so far, modulo nworkers
+  uint32_t rot = 0;  // units handed out so far, modulo nworkers
   for (;;) {
     uint64_t produced;
     int64_t spins = 0;
@@ -379,7 +396,8 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
       const uint64_t nvec = laneWord(cur, 9);
       const uint64_t ht = laneWord(cur, 10);
       const uint32_t head = (uint32_t)ht, tail = (uint32_t)(ht >> 32);
-      const uint64_t ntiles = (nvec * 16 + 1023) / 1024;
+      const uint64_t unitBytes = 1024ull * (uint32_t)queueUnitTiles(k);
+      const uint64_t nunits = (nvec * 16 + unitBytes - 1) / unitBytes;
       const uint32_t first = worker >= rot ? worker - rot : worker + nworkers - rot;
       switch (k) {
         case 1: queueEntry<T, OP, 1>(src, dst, head, tail, nvec, vector, first, nworkers); break;
@@ -391,7 +409,7 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
         case 7: queueEntry<T, OP, 7>(src, dst, head, tail, nvec, vector, first, nworkers); break;
         default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nworkers); break;
       }
-      rot = (uint32_t)((rot + ntiles) % nworkers);
+      rot = (uint32_t)((rot + nunits) % nworkers);
       // in a long run of entries let the count move every fourth entry, so that the
       // leader's window and the producer's ring move while the run is still going
       if ((done & 3) == 0 && done < produced) {
