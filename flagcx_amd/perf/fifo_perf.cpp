@@ -4,12 +4,15 @@
 //
 //   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
 //             [-W wavesPerCU] [-L lingerPolls] [-s spinLimit] [-q ringCapacity]
-//             [-D windowBytes] [-a separateAllocations]
+//             [-D windowBytes] [-a separateAllocations] [-g arrivalGapUs]
 //
 // A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
 // staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
 // chunk.  Times are host wall clock from the first enqueue (or launch) to the
 // moment the last chunk is known to be done; GB/s = (k+1)*bytes/time.
+// With -g the chunks are handed over one every arrivalGapUs microseconds of host
+// time (chunks that arrive one by one, the case the queue is for) instead of all at
+// once; the batch call, which needs every chunk, then starts after the last arrival.
 // Also: latency of ONE small entry, enqueue -> Wait, against launch -> stream sync.
 #include "../../include/flagcx_amd.h"
 
@@ -62,6 +65,7 @@ int main(int argc, char **argv) {
   int tuneWaves = -1;
   long long linger = -1;
   int capacity = 64, separate = 0;
+  double gapUs = 0.0;
   size_t window = 0;
   for (int i = 1; i + 1 < argc; i += 2) {
     const char *f = argv[i], *v = argv[i + 1];
@@ -78,6 +82,7 @@ int main(int argc, char **argv) {
     else if (!strcmp(f, "-q")) capacity = atoi(v);
     else if (!strcmp(f, "-D")) window = strtoull(v, 0, 0);
     else if (!strcmp(f, "-a")) separate = atoi(v);
+    else if (!strcmp(f, "-g")) gapUs = atof(v);
   }
   flagcxLocalReduceFifo_t fifo = nullptr;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
@@ -105,6 +110,15 @@ int main(int argc, char **argv) {
   const double algo = (k + 1.0) * (double)shardBytes;
   printf("# k=%d dtype=%d op=%d chunk=%zu B x %d chunks (%.0f MiB per input), warmup=%d iters=%d\n", k, dtype, op,
          chunkBytes, nchunks, shardBytes / 1048576.0, warmup, iters);
+  if (gapUs > 0)
+    printf("# chunks arrive %.2f us apart: the last one %.1f us after the first, i.e. at most %.1f GB/s\n", gapUs,
+           gapUs * (nchunks - 1), algo / (gapUs * (nchunks - 1)) / 1e3);
+  // chunk c is available from t0 + c * gapUs on
+  auto arrive = [&](double t0, int c) {
+    if (gapUs > 0)
+      while (nowUs() < t0 + gapUs * c) {
+      }
+  };
 
   std::vector<std::vector<const void *>> chunkSrc(nchunks, std::vector<const void *>(k));
   std::vector<flagcxLocalReduceDesc> descs(nchunks);
@@ -119,9 +133,11 @@ int main(int argc, char **argv) {
   std::vector<double> t;
   for (int it = 0; it < warmup + iters; it++) {
     const double t0 = nowUs();
-    for (int c = 0; c < nchunks; c++)
+    for (int c = 0; c < nchunks; c++) {
+      arrive(t0, c);
       FX(flagcxLocalReduce(chunkSrc[c].data(), k, descs[c].recvbuff, chunkCount, (flagcxDataType_t)dtype,
                            (flagcxRedOp_t)op, &st));
+    }
     CK(hipStreamSynchronize(st.base));
     if (it >= warmup) t.push_back(nowUs() - t0);
   }
@@ -131,6 +147,7 @@ int main(int argc, char **argv) {
   t.clear();
   for (int it = 0; it < warmup + iters; it++) {
     const double t0 = nowUs();
+    arrive(t0, nchunks - 1);
     FX(flagcxLocalReduceBatch(descs.data(), nchunks, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op, &st));
     CK(hipStreamSynchronize(st.base));
     if (it >= warmup) t.push_back(nowUs() - t0);
@@ -150,6 +167,7 @@ int main(int argc, char **argv) {
     const double t0 = nowUs();
     uint64_t ticket = 0;
     for (int c = 0; c < nchunks; c++) {
+      arrive(t0, c);
       flagcxResult_t r;
       while ((r = flagcxLocalReduceFifoEnqueueReduce(fifo, chunkSrc[c].data(), k, descs[c].recvbuff, chunkCount,
                                                      &ticket)) == flagcxInProgress) {
