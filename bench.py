@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
-"""Benchmark of the local N-way reduce on one MI355X.
+"""Benchmark of the local N-way reduce and chunk movers on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]          the driver's line
+    python bench.py --table sweep|sweep-rotate|configs|dtypes|stride [...]   tables only
 
 One "step" is one pass of the hot path over one batch: a single 8-input bf16 sum
 (fp32 accumulation) over 256 MiB per input buffer, i.e. one simulated rank's
@@ -12,17 +13,35 @@ the timed region.  Prints ONE JSON line on stdout:
              ((k+1) * n * sizeof(bf16) per step)
   roofline   the same bytes over the kernel's average launch duration measured
              with HIP events on the launch stream, against 8 TB/s of HBM3E
+  configs    the other benchmark configurations, each with its algorithmic bytes,
+             ms per pass, GB/s and fraction of the HBM peak: C1 (2 x fp32 sum, 64 MiB),
+             C3 (fp16 avg reduce-scatter shard: fused, one batch of 32 chunks, chunk
+             by chunk through the reduce queue, 32 chunk launches), C4 (4 x int32
+             max / min), C5 (2-input sum, pack, unpack at 4 KiB, 64 MiB, 1 GiB)
   cpu_baseline  the CPU oracle (a port of the reference's host reduce) timed on
-             this machine's cores on a bounded sample of the same workload
+             this machine's cores on a bounded sample of the headline workload, and
+             the reference's own host path for C1 (its ring all-reduce of two ranks:
+             one sum<float> per rank over half the vector), through the library built
+             from the reference's templates where that exists
   latency_us_4KiB  per-launch time of a 2-input fp32 sum over 4 KiB buffers
 
 Everything on the GPU goes through the C ABI of libflagcx_amd.so; the oracle is
-used only for the cpu_baseline leg and a spot check of the result.
+used only for the cpu_baseline leg and spot checks of results.
+
+Tables (human-readable, no JSON line; the summaries under profiles/ come from them):
+  --table sweep         C5: 1 KiB .. 1 GiB, 2-input fp32 sum, pack, unpack, copy, fill
+  --table sweep-rotate  the same over several sets of buffers in turn, from --min on
+  --table configs       every C1 / C3 / C4 row incl. HIP graph, staging ring, gather
+  --table dtypes        every element type x operation, --k inputs of --mib MiB
+  --table stride        k-input reduce against the inputs' relative placement,
+                        wavefronts per CU and inputs in flight
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
+import threading
 import time
 
 import numpy as np
@@ -34,18 +53,98 @@ HBM_PEAK_GBPS = 8000.0
 K = 8
 N_ELEM = 128 * 1024 * 1024          # 256 MiB of bf16 per input
 ALGO_BYTES = (K + 1) * N_ELEM * 2   # k reads + 1 write
+MiB = 1 << 20
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/reduce8_bf16_sum_256MiB_pmc.txt), scaled by a copy kernel of known size.
-MEASURED_TRAFFIC_BYTES = 2415851937
+# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a copy of
+# known size; not measured by this program.
+TRAFFIC_SOURCE = "profiles/reduce8_bf16_sum_256MiB_pmc.txt"
+TRAFFIC_BYTES = 2415851937
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(inputs_bits, sample_elems):
-    """Times the oracle on a leading sample of the same inputs (host copies)."""
+# --------------------------------------------------------------------- timing
+
+def timed_ms(fn, warmup=5, iters=20):
+    """ms per call of `iters` back-to-back calls (HIP events on the current stream)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def timed_sets_ms(fn, nsets, warmup=None, iters=20):
+    """The same with fn(i) cycling through nsets sets of buffers."""
+    import torch
+    for i in range(warmup if warmup is not None else max(5, nsets)):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(iters):
+        fn(i % nsets)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def single_launch_us(fn, nsets=1, warmup=5, iters=20):
+    """(median, min) microseconds of single launches, each between its own event pair."""
+    import torch
+    for i in range(max(warmup, nsets)):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    ts = []
+    for i in range(iters):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn(i % nsets)
+        e1.record()
+        e1.synchronize()
+        ts.append(e0.elapsed_time(e1) * 1e3)
+    ts.sort()
+    return ts[len(ts) // 2], ts[0]
+
+
+def row(nbytes, ms, **extra):
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    r = {"bytes": int(nbytes), "ms": round(ms, 5), "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    r.update(extra)
+    return r
+
+
+def placed(L, count, nelem, dtype, separate=False):
+    """`count` tensors of nelem elements inside one allocation, at the addresses
+    flagcxLocalPlaceBuffers gives (different HBM channel groups); the pool is returned
+    too so that it stays alive.  separate: plain torch allocations instead."""
+    import torch
+    if separate:
+        return [torch.empty(nelem, dtype=dtype, device="cuda") for _ in range(count)], None
+    esz = torch.empty(0, dtype=dtype).element_size()
+    nbytes = nelem * esz
+    pool_bytes = count * (nbytes + 128 * 1024)
+    pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    base = pool.data_ptr()
+    return [pool[a - base: a - base + nbytes].view(dtype) for a in L.place_buffers(base, pool_bytes, nbytes, count)], pool
+
+
+# --------------------------------------------------------------- CPU baselines
+
+def cpu_headline(inputs_bits, sample_elems):
+    """The oracle on a leading sample of the headline inputs (host copies)."""
     from oracle import cpu_oracle as O
     host = [np.ascontiguousarray(t[:sample_elems].cpu().numpy().view(np.uint16)) for t in inputs_bits]
     dst = np.empty(sample_elems, dtype=np.uint16)
@@ -64,29 +163,423 @@ def cpu_baseline(inputs_bits, sample_elems):
     }, host, dst
 
 
-def cpu_other_configs():
-    """The CPU side of two more benchmark configurations: C1 (2 x fp32 sum, 64 MiB per
-    buffer, full size) and C4 (4 x int32 max, a 16 Mi-element sample of 128 Mi)."""
+def cpu_c1_reference_path():
+    """C1 the way the reference runs it on the host: a ring all-reduce of two ranks
+    (flagcx/service/bootstrap.cc:702-749) cuts the 64 MiB vector into two 32 MiB
+    chunks and each rank folds one of them with ONE sum<float>(res = partial,
+    op1 = local, op2 = partial) (bootstrap.cc:651-653).  Timed through the library
+    built from the reference's own templates when it is there, through the oracle's
+    restatement otherwise; sockets and PCIe copies of that path are left out."""
     from oracle import cpu_oracle as O
+    n = 16 * 1024 * 1024
     rng = np.random.default_rng(0)
-    out = []
-    n1 = 16 * 1024 * 1024
-    fa = rng.uniform(-1, 1, n1).astype(np.float32)
-    fb = rng.uniform(-1, 1, n1).astype(np.float32)
-    fd = np.empty_like(fa)
-    for nth in (1, 2):
-        t = O.time_reduce([fa, fb], fd, O.FP32, O.SUM, nthreads=nth, warmup=1, iters=3)
-        out.append({"config": "C1 2x fp32 sum, 64 MiB per buffer, full size", "threads": nth,
-                    "value": round(3 * fa.nbytes / t / 1e9, 3), "unit": "GB/s"})
-    n4 = 16 * 1024 * 1024
-    ins = [rng.integers(-2**31, 2**31 - 1, n4, dtype=np.int64).astype(np.int32) for _ in range(4)]
-    dst = np.empty(n4, dtype=np.int32)
-    for nth in (1, 4):
-        t = O.time_reduce(ins, dst, O.INT32, O.MAX, nthreads=nth, warmup=1, iters=3)
-        out.append({"config": "C4 4x int32 max, 16 Mi-element sample of 128 Mi", "threads": nth,
-                    "value": round(5 * n4 * 4 / t / 1e9, 3), "unit": "GB/s"})
-    return out
+    a = rng.uniform(-1, 1, n).astype(np.float32)     # in0, then in1, one generator
+    b = rng.uniform(-1, 1, n).astype(np.float32)
+    half = n // 2
+    ref = O.ref_lib()
+    kind = "reference" if ref is not None else "port"
 
+    def fold(local, partial):
+        # data_for_recv = sum(sendbuff + offset, data_for_recv)
+        if ref is not None:
+            rc = ref.ref_binary(O.SUM, O.FP32, partial.ctypes.data, local.ctypes.data, partial.ctypes.data, partial.size)
+        else:
+            rc = O.lib().oracle_binary(O.SUM, O.FP32, partial.ctypes.data, local.ctypes.data, partial.ctypes.data,
+                                       partial.size, 1)
+        assert rc == 0
+
+    def one_pass(threads):
+        # rank 0 ends with chunk 0 = in1[0:half] (received) + in0[0:half] (local); rank 1 with chunk 1
+        p0, p1 = b[:half].copy(), a[half:].copy()
+        jobs = [(a[:half], p0), (b[half:], p1)]
+        t0 = time.perf_counter()
+        if threads == 1:
+            for loc, par in jobs:
+                fold(loc, par)
+        else:
+            th = [threading.Thread(target=fold, args=j) for j in jobs]
+            for t in th:
+                t.start()
+            for t in th:
+                t.join()
+        return time.perf_counter() - t0, p0, p1
+
+    res = {}
+    for threads in (1, 2):
+        one_pass(threads)
+        ts = sorted(one_pass(threads)[0] for _ in range(5))
+        res[threads] = ts[len(ts) // 2]
+    _, p0, p1 = one_pass(1)
+    want = a + b
+    ok = bool(np.array_equal(np.concatenate([p0, p1]), want))
+    nbytes = 3 * n * 4
+    return {
+        "config": "C1: 2-input fp32 sum, 64 MiB per buffer, uniform[-1,1) seed 0, as the reference's 2-rank host "
+                  "ring all-reduce folds it (two sum<float> calls over 8 Mi elements each)",
+        "value": round(nbytes / res[1] / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind,
+        "sample": "the whole configuration (192 MiB of traffic), median of 5 passes after 1 warm-up",
+        "threads_2": {"value": round(nbytes / res[2] / 1e9, 3), "threads": 2,
+                      "note": "one thread per simulated rank, each folding its own chunk"},
+        "result_equals_in0_plus_in1": ok,
+    }, a, b
+
+
+# ------------------------------------------------------------- configurations
+
+def config_c1(L, separate=False):
+    """2-input fp32 sum, 64 MiB per buffer: over the same three buffers launch after
+    launch (they fit the 256 MB memory-side cache), over rotating sets, and as the
+    reference's ring all-reduce (two chunk folds in one launch)."""
+    import torch
+    n = 16 * MiB
+    nb = 3 * n * 4
+    nsets = 9    # 9 x 192 MiB = 1.7 GiB in turn: nothing of a launch's buffers is left in the cache
+    sets, keep = [], []
+    g = torch.Generator(device="cuda").manual_seed(0)
+    for s in range(nsets):
+        bufs, pool = placed(L, 3, n, torch.float32, separate)
+        keep.append(pool)
+        if s == 0:
+            bufs[0].copy_(torch.rand(n, generator=g, device="cuda") * 2 - 1)
+            bufs[1].copy_(torch.rand(n, generator=g, device="cuda") * 2 - 1)
+        else:
+            bufs[0].copy_(sets[0][0])
+            bufs[1].copy_(sets[0][1])
+        sets.append(bufs)
+    a, b, out = sets[0]
+    out_rows = {}
+    ms = timed_ms(lambda: L.reduce([a, b], out, L.RedOp.Sum))
+    out_rows["C1_same_buffers"] = row(nb, ms, note="192 MiB working set: inside the 256 MB memory-side cache")
+    ms = timed_sets_ms(lambda i: L.reduce(sets[i][:2], sets[i][2], L.RedOp.Sum), nsets)
+    out_rows["C1_rotating_buffers"] = row(nb, ms, sets=nsets)
+    ms = timed_ms(lambda: L.all_reduce([a, b], out, L.RedOp.Sum))
+    out_rows["C1_ring_allreduce"] = row(nb, ms, note="chunk table of the reference's ring: two 32 MiB chunks, one launch")
+    ms = timed_sets_ms(lambda i: L.all_reduce(sets[i][:2], sets[i][2], L.RedOp.Sum), nsets)
+    out_rows["C1_ring_allreduce_rotating"] = row(nb, ms, sets=nsets)
+    return out_rows, (a, b, out)
+
+
+def make_c3(L, separate=False):
+    """8 ranks x 1 GiB fp16, N(0, sigma = 0.01) seeded per rank; shard = 128 MiB."""
+    import torch
+    nranks, per_rank = 8, 512 * MiB
+    shard = per_rank // nranks
+    send, pool = placed(L, nranks, per_rank, torch.float16, separate)
+    for r in range(nranks):
+        g = torch.Generator(device="cuda").manual_seed(100 + r)
+        for s in range(nranks):
+            send[r][s * shard:(s + 1) * shard] = (torch.randn(shard, generator=g, device="cuda") * 0.01).to(torch.float16)
+    recv = torch.empty(shard, dtype=torch.float16, device="cuda")
+    return nranks, per_rank, shard, send, recv, pool
+
+
+def c3_chunk_descs(L, nranks, shard, send, recv, rank):
+    chunk_elems = L.CHUNKSIZE // 2
+    descs = []
+    for c in range(shard // chunk_elems):
+        srcs = [send[(rank + 1 + j) % nranks].data_ptr() + (rank * shard + c * chunk_elems) * 2 for j in range(nranks)]
+        descs.append((srcs, recv.data_ptr() + c * chunk_elems * 2, chunk_elems))
+    return descs
+
+
+def c3_queue_ms(L, nranks, descs, warmup=5, iters=20):
+    """The shard chunk by chunk through the resident reduce queue: host wall clock from
+    the first enqueue to the return of Wait on the last ticket."""
+    import torch
+    lib = L.lib()
+    fifo = L.ReduceFifo(64, nranks, L.DataType.Float16, L.RedOp.Avg)
+    arrs = [((C.c_void_p * nranks)(*d[0]), d[1], d[2]) for d in descs]
+    ticket = C.c_uint64()
+    enq = lib.flagcxLocalReduceFifoEnqueueReduce
+    times = []
+    torch.cuda.synchronize()
+    lib.flagcxLocalSetMaxSpinCount(1 << 22)
+    try:
+        with fifo:
+            for it in range(warmup + iters):
+                t0 = time.perf_counter()
+                for srcs, dst, cnt in arrs:
+                    while True:
+                        rc = enq(fifo._h, srcs, nranks, dst, cnt, C.byref(ticket))
+                        if rc != L.Result.InProgress:
+                            break
+                    fifo._check(rc)
+                fifo.wait(ticket.value)
+                if it >= warmup:
+                    times.append((time.perf_counter() - t0) * 1e3)
+            grid = fifo.grid()
+    finally:
+        fifo.close()
+        lib.flagcxLocalSetMaxSpinCount(-1)
+    times.sort()
+    return times[len(times) // 2], grid
+
+
+def config_c3(L, full=False, separate=False):
+    import torch
+    nranks, per_rank, shard, send, recv, pool = make_c3(L, separate)
+    rank = 3
+    nb = 9 * shard * 2
+    rows = {}
+    ms = timed_ms(lambda: L.reduce_scatter(send, rank, recv, L.RedOp.Avg))
+    rows["C3_fused"] = row(nb, ms, note="one launch for the 128 MiB shard")
+    descs = c3_chunk_descs(L, nranks, shard, send, recv, rank)
+    ms = timed_ms(lambda: L.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks))
+    rows["C3_batch_32x4MiB"] = row(nb, ms, note="32 chunk descriptors, one batch call (needs every chunk present)")
+    ms, grid = c3_queue_ms(L, nranks, descs)
+    rows["C3_queue_32x4MiB"] = row(nb, ms, note="chunk by chunk through the resident reduce queue, host wall clock "
+                                                "first enqueue -> Wait; %d resident wavefronts" % grid)
+    ms = timed_ms(lambda: L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE))
+    rows["C3_per_chunk_launches"] = row(nb, ms, note="32 launches of 4 MiB chunks on one stream, %.2f us per launch"
+                                                     % (ms * 1e3 / 32))
+    if full:
+        # the 32 chunk launches captured once into a HIP graph and replayed
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE)
+        rows["C3_per_chunk_launches_hip_graph"] = row(nb, timed_ms(graph.replay))
+        del graph
+        # the 7 peers' slices staged through a 16 x 4 MiB ring on a second stream
+        ring_mem = torch.empty(L.CHUNKSIZE * 16 * (nranks - 1), dtype=torch.uint8, device="cuda")
+        ring = L.Ring(ring_mem, nranks - 1)
+        copy_t = torch.cuda.Stream()
+        cs, ms_ = L.Stream(copy_t.cuda_stream), L.current_stream()
+        staged = nb + 2 * (nranks - 1) * shard * 2
+        ms = timed_ms(lambda: ring.reduce_scatter(send, rank, recv, L.RedOp.Avg, cs, ms_))
+        rows["C3_staging_ring_2_streams"] = row(nb, ms, hbm_bytes_incl_staging=staged,
+                                                hbm_gbps=round(staged / ms / 1e6, 1))
+        L.lib().flagcxLocalSetMaxSpinCount(1 << 22)
+        fifo = L.ReduceFifo(64, nranks, L.DataType.Float16, L.RedOp.Avg)
+        torch.cuda.synchronize()
+        with fifo:
+            for _ in range(5):
+                ring.reduce_scatter_fifo(fifo, send, rank, recv, cs)
+            t0 = time.perf_counter()
+            for _ in range(20):
+                ring.reduce_scatter_fifo(fifo, send, rank, recv, cs)
+            ms = (time.perf_counter() - t0) * 1e3 / 20
+        fifo.close()
+        L.lib().flagcxLocalSetMaxSpinCount(-1)
+        rows["C3_staging_ring_polled_into_queue"] = row(nb, ms, hbm_bytes_incl_staging=staged,
+                                                        hbm_gbps=round(staged / ms / 1e6, 1))
+        ring.close()
+        del ring_mem
+
+        def all_shards():
+            for rk in range(nranks):
+                L.reduce_scatter(send, rk, recv, L.RedOp.Avg)
+        rows["C3_all_8_shards"] = row(8 * nb, timed_ms(all_shards, warmup=2, iters=5))
+        # The stage after it in an all-reduce: every rank holds one reduced slice in a buffer of
+        # the full size.  The reference zero-fills the rest of each buffer and sum-all-reduces the
+        # buffers (flagcx/core/c2c_algo.cc:586-608 + :310-336); slice copies do the same job.
+        fullbuf = torch.empty(per_rank, dtype=torch.float16, device="cuda")
+
+        def refresh_and_sum():
+            for rk in range(nranks):
+                L.refresh(send[rk], 0, rk * shard, shard, per_rank, L.RedOp.Sum)
+            L.reduce(send, fullbuf, L.RedOp.Sum)
+        traffic = nranks * (per_rank - shard) * 2 + (nranks + 1) * per_rank * 2
+        rows["C3_gather_zero_fill_plus_sum"] = row(traffic, timed_ms(refresh_and_sum, warmup=2, iters=5))
+
+        def copy_slices():
+            for rk in range(nranks):
+                L.memcpy(fullbuf.data_ptr() + rk * shard * 2, send[rk].data_ptr() + rk * shard * 2, shard * 2)
+        rows["C3_gather_8_slice_copies"] = row(2 * per_rank * 2, timed_ms(copy_slices, warmup=2, iters=5))
+        del fullbuf
+    del send, recv, pool
+    torch.cuda.empty_cache()
+    return rows
+
+
+def config_c4(L, separate=False):
+    import torch
+    n = 128 * MiB
+    g = torch.Generator(device="cuda").manual_seed(3)
+    bufs, pool = placed(L, 5, n, torch.int32, separate)
+    ins, out = bufs[:4], bufs[4]
+    for t in ins:
+        t.copy_(torch.randint(-2**31, 2**31 - 1, (n,), generator=g, device="cuda", dtype=torch.int32))
+    rows = {}
+    for op, nm in ((L.RedOp.Max, "max"), (L.RedOp.Min, "min")):
+        rows["C4_" + nm] = row(5 * n * 4, timed_ms(lambda: L.reduce(ins, out, op)))
+    del bufs, pool
+    torch.cuda.empty_cache()
+    return rows
+
+
+def sweep_point(L, size, rotate, g):
+    """One size of C5: (nsets, {kernel: (median us, GB/s)}, back-to-back us of the 2-input sum)."""
+    import torch
+    lib = L.lib()
+    st = L.current_stream()
+    sref = C.byref(st)
+    f32, opsum = int(L.DataType.Float32), int(L.RedOp.Sum)
+    n = size // 4
+    chunk = size // 8
+    nsets = 1
+    if rotate:
+        nsets = max(2, min(16, ((3 << 29) + 2 * size - 1) // (2 * size)))
+    bufs = []
+    for _ in range(nsets):
+        a = torch.rand(n, device="cuda", generator=g) * 2 - 1
+        b = torch.rand(n, device="cuda", generator=g) * 2 - 1
+        c = torch.empty(n, device="cuda")
+        # sparse source of 8*size bytes holding 8 chunks of size/8 at stride `size`
+        sparse = torch.rand(8 * n, device="cuda", generator=g)
+        staged = torch.empty(n, device="cuda")
+        bufs.append((a, b, c, sparse, staged, (C.c_void_p * 2)(a.data_ptr(), b.data_ptr())))
+    fns = {
+        "reduce2": (3 * size, lambda i: lib.flagcxLocalReduce(bufs[i][5], 2, bufs[i][2].data_ptr(), n, f32, opsum, sref)),
+        "pack": (2 * size, lambda i: lib.flagcxLocalPack(bufs[i][4].data_ptr(), bufs[i][3].data_ptr(), 8, chunk, size, sref)),
+        "unpack": (2 * size, lambda i: lib.flagcxLocalUnpack(bufs[i][3].data_ptr(), bufs[i][4].data_ptr(), 8, chunk, size, sref)),
+        "memcpy": (2 * size, lambda i: lib.flagcxLocalMemcpy(bufs[i][2].data_ptr(), bufs[i][0].data_ptr(), size, sref)),
+        "memset": (size, lambda i: lib.flagcxLocalMemset(bufs[i][2].data_ptr(), 0, size, sref)),
+    }
+    out = {}
+    for name, (nb, fn) in fns.items():
+        assert fn(0) == 0, name
+        med, _ = single_launch_us(fn, nsets)
+        out[name] = (med, nb / med / 1e3, nb)
+    nb2b = 1000 if size <= (1 << 20) else 50
+    b2b = timed_sets_ms(fns["reduce2"][1], nsets, warmup=20, iters=nb2b) * 1e3
+    del bufs
+    torch.cuda.empty_cache()
+    return nsets, out, b2b
+
+
+def config_c5(L):
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(0)
+    rows = {}
+    for size, name, rotate in ((4096, "C5_4KiB", False), (64 * MiB, "C5_64MiB", True), (1 << 30, "C5_1GiB", True)):
+        nsets, out, b2b = sweep_point(L, size, rotate, g)
+        r = {"bytes_per_buffer": size, "sets": nsets}
+        for k in ("reduce2", "pack", "unpack"):
+            med, gbps, nb = out[k]
+            r[k] = {"bytes": nb, "us": round(med, 2), "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+        r["reduce2"]["back_to_back_us"] = round(b2b, 2)
+        if size == 4096:
+            r["note"] = "launch-latency bound: us per single launch between its own event pair"
+        rows[name] = r
+    return rows
+
+
+# --------------------------------------------------------------------- tables
+
+def table_sweep(L, args):
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(0)
+    print("%12s %10s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %8s" %
+          ("bytes", "sets", "reduce2us", "GB/s", "pack us", "GB/s", "unpack us", "GB/s", "memcpy us", "GB/s",
+           "memset us", "GB/s", "b2b us"))
+    size = args.min
+    while size <= args.max:
+        nsets, out, b2b = sweep_point(L, size, args.table == "sweep-rotate", g)
+        print("%12d %10d | " % (size, nsets) +
+              " | ".join("%9.2f %9.1f" % out[k][:2] for k in ("reduce2", "pack", "unpack", "memcpy", "memset")) +
+              " | %8.2f" % b2b, flush=True)
+        size *= 2
+
+
+def table_configs(L, args):
+    rows = {}
+    rows.update(config_c1(L, args.allocator_layout)[0])
+    rows.update(config_c3(L, full=True, separate=args.allocator_layout))
+    rows.update(config_c4(L, args.allocator_layout))
+    for name, r in rows.items():
+        extra = "  ".join("%s=%s" % (k, v) for k, v in r.items() if k not in ("bytes", "ms", "gbps", "frac"))
+        print("%-36s %14d B  %9.4f ms  %8.1f GB/s  %5.1f %%  %s" % (name, r["bytes"], r["ms"], r["gbps"],
+                                                                      100 * r["frac"], extra), flush=True)
+
+
+def table_dtypes(L, args):
+    import torch
+    lib = L.lib()
+    names = ["int8", "uint8", "int32", "uint32", "int64", "uint64", "fp16", "fp32", "fp64", "bf16"]
+    sizes = [1, 1, 4, 4, 8, 8, 2, 4, 8, 2]
+    ops = [("sum", L.RedOp.Sum), ("prod", L.RedOp.Prod), ("max", L.RedOp.Max), ("min", L.RedOp.Min), ("avg", L.RedOp.Avg)]
+    nbytes = args.mib * MiB
+    st = L.current_stream()
+    sref = C.byref(st)
+    for k in args.k:
+        sets = []
+        for _ in range(args.sets):
+            pool_bytes = (k + 1) * (nbytes + 128 * 1024)
+            pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+            pool.view(torch.int16).random_(0, 16000)     # finite, normal values in every floating-point type
+            addrs = L.place_buffers(pool.data_ptr(), pool_bytes, nbytes, k + 1)
+            sets.append(((C.c_void_p * k)(*addrs[:k]), addrs[k], pool))
+        print("k=%d, %d MiB per input, %d buffer set(s) in turn; percent of 8 TB/s" % (k, args.mib, args.sets), flush=True)
+        for dt in range(10):
+            count = nbytes // sizes[dt]
+            line = "  %-7s" % names[dt]
+            for oname, op in ops:
+                def go(i):
+                    srcs, dst, _ = sets[i]
+                    L.check(lib.flagcxLocalReduce(srcs, k, dst, count, dt, int(op), sref))
+                ms = timed_sets_ms(go, args.sets, warmup=2 * args.sets, iters=16)
+                line += "  %s %5.1f" % (oname, (k + 1) * nbytes / (ms * 1e-3) / 1e9 / 80.0)
+            print(line, flush=True)
+        del sets
+        torch.cuda.empty_cache()
+
+
+STRIDES = [128 * MiB, 128 * MiB + 4096, 128 * MiB + 65536, 129 * MiB + 4096, 256 * MiB, 512 * MiB,
+           1024 * MiB, 1024 * MiB + 4096, 1024 * MiB + 65536, 1025 * MiB, 1026 * MiB + 8192, 1057 * MiB + 12288]
+CAPS = [8, 10, 12, 14, 16, 18, 21, 25, 0, -1]   # caps that whole LDS granules can express; -1 = the library's choice
+
+
+def table_stride(L, args):
+    """The inputs are slices of one allocation, `stride` bytes apart, so their addresses
+    alias differently in the HBM channel hash; per stride, percent of peak for several caps
+    on resident wavefronts per CU and for the library's own choice ("auto")."""
+    import torch
+    lib = L.lib()
+    k = args.k[0]
+    tdt = torch.bfloat16
+    esz = 2
+    nbytes = args.mib * MiB
+    n = nbytes // esz
+    cap0, loads0 = C.c_int(0), C.c_int(0)
+    L.check(lib.flagcxLocalGetTune(k, C.byref(cap0)))
+    L.check(lib.flagcxLocalGetTuneLoads(k, C.byref(loads0)))
+    bigs, outs = [], []
+    for _ in range(args.sets):
+        big = torch.empty((max(STRIDES) * (k - 1) + nbytes) // esz + 16, dtype=tdt, device="cuda")
+        big.view(torch.int16).random_(0, 1000)
+        bigs.append(big)
+        outs.append(torch.empty(n, dtype=tdt, device="cuda"))
+    print("k=%d bf16, %d MiB per input, %d buffer set(s), inputs in flight per wavefront in the cap columns: %s; "
+          "percent of 8 TB/s, (k+1)*bytes/time" % (k, args.mib, args.sets, "library's choice" if args.loads < 0 else args.loads))
+    print("%14s " % "stride" + " ".join("%7s" % ("cap %d" % c if c > 0 else "no cap" if c == 0 else "auto") for c in CAPS))
+    worst = {c: 100.0 for c in CAPS}
+    best = {c: 0.0 for c in CAPS}
+    try:
+        for stv in STRIDES:
+            srcs = [[big[j * stv // esz: j * stv // esz + n] for j in range(k)] for big in bigs]
+            cells = []
+            for cap in CAPS:
+                L.check(lib.flagcxLocalTune(k, cap))
+                L.check(lib.flagcxLocalTuneLoads(k, args.loads if cap >= 0 else -1))
+                ms = timed_sets_ms(lambda i: L.reduce(srcs[i], outs[i], L.RedOp.Sum), args.sets,
+                                   warmup=3 * args.sets, iters=20 * args.sets)
+                pct = (k + 1) * nbytes / (ms * 1e-3) / 1e9 / 80.0
+                worst[cap] = min(worst[cap], pct)
+                best[cap] = max(best[cap], pct)
+                cells.append("%7.1f" % pct)
+            print("%14d " % stv + " ".join(cells), flush=True)
+    finally:
+        L.check(lib.flagcxLocalTune(k, cap0.value))
+        L.check(lib.flagcxLocalTuneLoads(k, loads0.value))
+    print("%14s " % "worst..best" + " ".join("%3.0f..%-3.0f" % (worst[c], best[c]) for c in CAPS))
+
+
+# ----------------------------------------------------------------------- main
 
 def main():
     ap = argparse.ArgumentParser()
@@ -96,8 +589,7 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=32 * 1024 * 1024,
                     help="elements per input the CPU baseline reduces")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--cpu-configs", action="store_true",
-                    help="cpu_baseline also times the oracle on the C1 and C4 configurations")
+    ap.add_argument("--no-configs", action="store_true", help="skip the C1 / C3 / C4 / C5 rows")
     ap.add_argument("--allocator-layout", action="store_true",
                     help="inputs and output as separate torch allocations instead of placed in one")
     ap.add_argument("--rotate-sets", type=int, default=3, metavar="S",
@@ -106,6 +598,15 @@ def main():
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also run N flagcxLocalMemcpy launches of 256 MiB (a copy of known size "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--table", choices=["sweep", "sweep-rotate", "configs", "dtypes", "stride"],
+                    help="print one of the tables instead of the JSON line")
+    ap.add_argument("--min", type=int, default=1 << 10, help="sweep tables: smallest size")
+    ap.add_argument("--max", type=int, default=1 << 30, help="sweep tables: largest size")
+    ap.add_argument("--k", type=int, nargs="+", default=[8, 4, 2], help="dtypes / stride tables: inputs")
+    ap.add_argument("--mib", type=int, default=256, help="dtypes / stride tables: MiB per input")
+    ap.add_argument("--sets", type=int, default=2, help="dtypes / stride tables: buffer sets used in turn")
+    ap.add_argument("--loads", type=int, default=-1,
+                    help="stride table: inputs in flight per wavefront for the cap columns (-1: the library's choice)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs on ONE GPU (the k ranks are k HBM buffers on it); "
@@ -120,21 +621,20 @@ def main():
     torch.cuda.set_device(0)
     L.check(L.lib().flagcxLocalInit())
 
+    if args.table:
+        {"sweep": table_sweep, "sweep-rotate": table_sweep, "configs": table_configs, "dtypes": table_dtypes,
+         "stride": table_stride}[args.table](L, args)
+        return
+
     # The 8 input buffers and the output live in one allocation, at the addresses
     # flagcxLocalPlaceBuffers gives: equal offsets into them fall into different HBM
     # channel groups, which is how a caller that owns the ranks' staging buffers would
     # lay them out.  --allocator-layout takes nine separate torch allocations instead
     # (258 MiB apart on this allocator: all in one channel group).
     nbytes = N_ELEM * 2
-    if args.allocator_layout:
-        bufs = [torch.empty(N_ELEM, dtype=torch.bfloat16, device="cuda") for _ in range(K + 1)]
-        layout = "nine separate torch allocations"
-    else:
-        pool_bytes = (K + 1) * (nbytes + 128 * 1024)
-        pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
-        addrs = L.place_buffers(pool.data_ptr(), pool_bytes, nbytes, K + 1)
-        bufs = [pool[a - pool.data_ptr(): a - pool.data_ptr() + nbytes].view(torch.bfloat16) for a in addrs]
-        layout = "one allocation, buffers placed by flagcxLocalPlaceBuffers"
+    bufs, pool = placed(L, K + 1, N_ELEM, torch.bfloat16, args.allocator_layout)
+    layout = "nine separate torch allocations" if args.allocator_layout else \
+        "one allocation, buffers placed by flagcxLocalPlaceBuffers"
     # seeded synthetic inputs: N(0,1) per input from seeds 0..7, rounded to bf16
     inputs = bufs[:K]
     out = bufs[K]
@@ -171,28 +671,14 @@ def main():
     if args.rotate_sets >= 2:
         sets, keep = [bufs], []
         for _ in range(args.rotate_sets - 1):
-            if args.allocator_layout:
-                more = [torch.empty(N_ELEM, dtype=torch.bfloat16, device="cuda") for _ in range(K + 1)]
-            else:
-                p2 = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
-                keep.append(p2)
-                more = [p2[a - p2.data_ptr(): a - p2.data_ptr() + nbytes].view(torch.bfloat16)
-                        for a in L.place_buffers(p2.data_ptr(), pool_bytes, nbytes, K + 1)]
+            more, p2 = placed(L, K + 1, N_ELEM, torch.bfloat16, args.allocator_layout)
+            keep.append(p2)
             for j in range(K):
                 more[j].copy_(inputs[j])
             sets.append(more)
         nset = len(sets)
-        for i in range(2 * nset):
-            L.reduce(sets[i % nset][:K], sets[i % nset][K], L.RedOp.Sum)
-        torch.cuda.synchronize()
-        r0 = torch.cuda.Event(enable_timing=True)
-        r1 = torch.cuda.Event(enable_timing=True)
-        r0.record()
-        for i in range(args.steps):
-            L.reduce(sets[i % nset][:K], sets[i % nset][K], L.RedOp.Sum)
-        r1.record()
-        torch.cuda.synchronize()
-        rot_ms = r0.elapsed_time(r1) / args.steps
+        rot_ms = timed_sets_ms(lambda i: L.reduce(sets[i][:K], sets[i][K], L.RedOp.Sum), nset,
+                               warmup=2 * nset, iters=args.steps)
         same_out = all(torch.equal(sets[i][K].view(torch.int16), out.view(torch.int16)) for i in range(1, nset))
         rotating = {"sets": nset, "value": round(ALGO_BYTES / (rot_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
                     "frac": round(ALGO_BYTES / (rot_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
@@ -206,7 +692,6 @@ def main():
 
     # small-message latency: 2-input fp32 sum over 4 KiB buffers, arguments
     # marshalled once so the loop is one C call per launch
-    import ctypes as C
     a = torch.rand(1024, device="cuda")
     b = torch.rand(1024, device="cuda")
     c = torch.empty(1024, device="cuda")
@@ -219,18 +704,7 @@ def main():
     def small():
         return fn(ptrs, 2, cptr, 1024, f32, opsum, sref)
 
-    for _ in range(200):
-        small()
-    torch.cuda.synchronize()
-    n_lat = 2000
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(n_lat):
-        small()
-    e1.record()
-    torch.cuda.synchronize()
-    lat_stream_us = e0.elapsed_time(e1) * 1e3 / n_lat
+    lat_stream_us = timed_ms(small, warmup=200, iters=2000) * 1e3
     singles = []
     for _ in range(200):
         s0 = time.perf_counter()
@@ -247,9 +721,9 @@ def main():
         try:
             r = subprocess.run([perf_bin, "-b", "4096", "-e", "4096", "-n", "40"], capture_output=True, text=True,
                                timeout=120)
-            row = [l.split() for l in r.stdout.splitlines() if l.strip().startswith("4096")]
-            if r.returncode == 0 and row:
-                c_lat = {"back_to_back_per_launch": float(row[0][2]), "single_launch_to_sync_median": float(row[0][4])}
+            rw = [l.split() for l in r.stdout.splitlines() if l.strip().startswith("4096")]
+            if r.returncode == 0 and rw:
+                c_lat = {"back_to_back_per_launch": float(rw[0][2]), "single_launch_to_sync_median": float(rw[0][4])}
         except Exception as e:  # the figure is auxiliary: report why it is missing
             log("bench.py: C latency driver failed: %r" % (e,))
 
@@ -265,7 +739,9 @@ def main():
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "rotating_buffers": rotating,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES,
+                     "traffic_source": TRAFFIC_SOURCE + " (rocprofv3 counter runs of this same command, "
+                                                        "not measured by this run)",
                      "kernel": "reduceWaveKernel<bf16,sum,K=8,U=1>", "avg_launch_ms": round(kern_ms, 5),
                      "algorithmic_bytes_per_launch": ALGO_BYTES},
         "latency_us_4KiB": {"workload": "2-input fp32 sum, 4 KiB per buffer",
@@ -278,10 +754,8 @@ def main():
     if not args.no_cpu:
         bits = [t.view(torch.int16) for t in inputs]
         sample = min(args.cpu_sample, N_ELEM)
-        base, host, dst = cpu_baseline(bits, sample)
+        base, host, dst = cpu_headline(bits, sample)
         result["cpu_baseline"] = base
-        if args.cpu_configs:
-            base["other_configs"] = cpu_other_configs()
         # spot check of the GPU result against the oracle on the sample
         got = out[:sample].view(torch.int16).cpu().numpy().view(np.uint16)
         result["spot_check_vs_oracle"] = "bit-exact" if got.tobytes() == dst.tobytes() else "MISMATCH"
@@ -289,6 +763,33 @@ def main():
             log("bench.py: GPU result differs from the oracle on the sample")
             print(json.dumps(result))
             sys.exit(1)
+        del host, dst
+
+    del bufs, pool, inputs, out
+    torch.cuda.empty_cache()
+
+    if not args.no_configs:
+        cfg = {"method": "5 warm-up + 20 timed back-to-back passes per row, HIP events on the launch stream; "
+                         "C5 rows: median of 20 single launches, each between its own event pair; "
+                         "frac = GB/s / 8000; buffers placed by flagcxLocalPlaceBuffers unless "
+                         "--allocator-layout"}
+        c1_rows, (ca, cb, cout) = config_c1(L, args.allocator_layout)
+        cfg.update(c1_rows)
+        if not args.no_cpu:
+            c1_cpu, ha, hb = cpu_c1_reference_path()
+            result["cpu_baseline"]["c1_fp32_reference_path"] = c1_cpu
+            # the GPU's C1 output against the same sum on the host (fp32 add is exact either way)
+            L.reduce([ca, cb], cout, L.RedOp.Sum)
+            torch.cuda.synchronize()
+            ga, gb = ca.cpu().numpy(), cb.cpu().numpy()
+            cfg["C1_same_buffers"]["bit_exact_vs_host_sum"] = bool(np.array_equal(cout.cpu().numpy(), ga + gb))
+            del ha, hb
+        del ca, cb, cout
+        torch.cuda.empty_cache()
+        cfg.update(config_c3(L, full=False, separate=args.allocator_layout))
+        cfg.update(config_c4(L, args.allocator_layout))
+        cfg.update(config_c5(L))
+        result["configs"] = cfg
 
     print(json.dumps(result))
 
