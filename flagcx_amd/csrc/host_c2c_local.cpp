@@ -22,9 +22,12 @@
 // commOp values: LocCpy copies send[sendOffset..) to recv[recvOffset..); LocRed
 // sets recv[recvOffset..) = OP(send[sendOffset..), recv[recvOffset..)).
 //
-// Not replayed (flagcxNotSupported): Send/Recv homo functions of homoType 1, which
-// need the planner's inter-rank buffer lists (c2c_algo.cc:386-400,434-452), and
-// AlltoAllv.
+// Send / Recv homo functions (c2c_algo.cc:364-463) are replayed for all three
+// homoTypes; for homoType 1 the planner's inter-rank buffer list, which the plan
+// document does not carry, is rebuilt from the rank's hetero receives (the list's
+// isRecv_ entries are exactly those, c2c_algo.cc:386-400,434-452).
+// Not replayed (flagcxNotSupported): AlltoAllv, whose counts and displacements are
+// call arguments, not part of a plan.
 #include "../../include/flagcx_amd.h"
 
 #include <cstdio>
@@ -80,6 +83,16 @@ struct Node {
   size_t size(const char *n) const {
     const Node *c = child(n);
     return c ? (size_t)strtoull(c->text.c_str(), nullptr, 10) : 0;
+  }
+  // the name of the first child (searched to any depth) among `fields` that holds a
+  // negative number: offsets and counts are sizes (readSizeTag, c2c_ir.h:55-60)
+  const char *negativeSize(const char *const *fields, int nfields) const {
+    for (auto &k : kids) {
+      for (int i = 0; i < nfields; i++)
+        if (k.name == fields[i] && !k.text.empty() && k.text[0] == '-') return fields[i];
+      if (const char *deep = k.negativeSize(fields, nfields)) return deep;
+    }
+    return nullptr;
   }
 };
 
@@ -197,6 +210,8 @@ struct flagcxLocalPlan {
   int commOp = flagcxCommNoOp, redOp = flagcxSum;
   std::vector<RankPlan> ranks;
   int algorithm = 2; // flagcxAlgoInput: what importXml sets (c2c_algo.h:15-19, c2c_algo.cc:974)
+  size_t defaultChunks = 0; // nChunks of documents that carry none (flagcxLocalPlanSetChunks)
+  int eachNicPerRank = 0, multiNic = 0; // as the planner's constructor sets them (c2c_algo.cc:636-672)
   bool loaded = false;
   char err[256] = "";
 };
@@ -247,7 +262,12 @@ static flagcxResult_t gatherBlocks(char *dst, const std::vector<const void *> &s
   return flagcxSuccess;
 }
 
-// One homo function slot (step s, index i of one table) across all ranks.
+static flagcxResult_t runSendRecv(flagcxLocalPlan *p, int cl, const std::vector<const HomoFunc *> &fn, const Bufs &b,
+                                  size_t ts, int root, flagcxStream_t stream);
+
+// One homo function slot (step s, index i of one table) across all ranks.  `root`
+// is the collective's root as a rank of its cluster, globalrank2homorank[root]
+// (c2c_algo.cc:2147,2170).
 static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const HomoFunc *> &fn, const Bufs &b,
                                   flagcxDataType_t dt, int root, flagcxStream_t stream) {
   const size_t ts = flagcxLocalGetDataTypeSize(dt);
@@ -280,6 +300,10 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
           LCHECK(flagcxLocalReduce(srcs, 2, d, f->count_, dt, (flagcxRedOp_t)p->redOp, stream));
         }
       }
+      continue;
+    }
+    if (op == flagcxCommOpSend || op == flagcxCommOpRecv) {
+      LCHECK(runSendRecv(p, cl, fn, b, ts, root, stream));
       continue;
     }
     // the communicator the reference would use: homoInterComm for homoType 1, else homo_comm
@@ -365,7 +389,8 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
   return flagcxSuccess;
 }
 
-static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream);
+static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream,
+                                 const std::vector<char> *only = nullptr);
 
 static flagcxResult_t runHomoStep(flagcxLocalPlan *p, std::vector<std::vector<HomoFunc>> RankPlan::*table, int s,
                                   const Bufs &b, flagcxDataType_t dt, int root, flagcxStream_t stream,
@@ -433,16 +458,91 @@ static size_t heteroWidth(flagcxLocalPlan *p, int s) {
   return w;
 }
 
-static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream) {
+// The refresh function of every rank (only: of the ranks marked).
+static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream,
+                                 const std::vector<char> *only) {
   for (int r = 0; r < p->nranks; r++) {
+    if (only && !(*only)[r]) continue;
     const RefreshFunc &f = p->ranks[r].refreshFunc_;
-    // bufftype -1 resolves to recv (1) without scratch, scratch (2) with it (c2c_algo.cc:2156-2164)
+    // bufftype -1 resolves to recv (1) without scratch, scratch (2) with it, and under the
+    // pipeline algorithm a reduce-type collective starts at its cluster's part (c2c_algo.cc:2156-2164)
     int bt = f.bufftype_;
-    if (bt == -1) bt = (b.scratch && b.scratch[r]) ? 2 : 1;
+    size_t start = f.start_;
+    if (bt == -1) {
+      bt = (b.scratch && b.scratch[r]) ? 2 : 1;
+      if ((p->commOp == flagcxCommOpReduceScatter || p->commOp == flagcxCommOpAllReduce) && p->algorithm == 1) {
+        size_t clusterOffset = 0;
+        for (int c = 0; c < p->clusterOf[r]; c++) clusterOffset += p->clusterRanks[c].size();
+        start = clusterOffset * p->totalCount / (size_t)p->nranks;
+      }
+    }
     void *buff = bt == 1 ? b.recv[r] : (b.scratch ? b.scratch[r] : nullptr);
     if (f.totalCount_ == 0) continue;
     if (!buff) return planFail(p, flagcxInvalidArgument, "refresh needs a scratch buffer%s", "");
-    LCHECK(flagcxLocalRefresh(buff, f.start_, f.offset_, f.count_, f.totalCount_, dt, (flagcxRedOp_t)f.redOp_, stream));
+    LCHECK(flagcxLocalRefresh(buff, start, f.offset_, f.count_, f.totalCount_, dt, (flagcxRedOp_t)f.redOp_, stream));
+  }
+  return flagcxSuccess;
+}
+
+// Send / Recv homo functions of one cluster in one slot (c2c_algo.cc:364-463).  A
+// send is carried out when the receiving rank holds the matching Recv function:
+//   homoType 0: the root sends [sendOffset, +count) to every other inter-rank,
+//               which receives at its recvOffset;
+//   homoType 1: inter-ranks 1.. send to inter-rank 0 what they received from other
+//               clusters, piece by piece at the pieces' own offsets;
+//   homoType 2: inter-rank 0 sends to the root unless it is the root itself.
+// Roots are ranks inside the cluster.
+static flagcxResult_t runSendRecv(flagcxLocalPlan *p, int cl, const std::vector<const HomoFunc *> &fn, const Bufs &b,
+                                  size_t ts, int root, flagcxStream_t stream) {
+  const std::vector<int> &members = p->clusterRanks[cl], &inters = p->clusterInterRanks[cl];
+  auto recvOf = [&](int r) -> const HomoFunc * {
+    const HomoFunc *g = fn[r];
+    return (g && g->commOp_ == flagcxCommOpRecv) ? g : nullptr;
+  };
+  for (int r : members) {
+    const HomoFunc *f = fn[r];
+    if (!f || f->commOp_ != flagcxCommOpSend) continue;
+    const int rt = f->rootRank_ == -1 ? root : f->rootRank_;
+    if (rt < 0 || rt >= (int)members.size())
+      return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
+    char *src = pick(b, r, f->sendType_);
+    if (!src) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+    if (f->homoType_ == 0) {
+      if (p->homoRank[r] != rt) continue;
+      for (int peer : inters) {
+        const HomoFunc *g = recvOf(peer);
+        if (peer == r || !g || p->homoRank[peer] == rt) continue;
+        char *dst = pick(b, peer, g->recvType_ == 1 ? 1 : 2);
+        if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+        LCHECK(flagcxLocalMemcpy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts, stream));
+      }
+    } else if (f->homoType_ == 1) {
+      if (p->homoInterRank[r] <= 0 || inters.empty()) continue;
+      const HomoFunc *g = recvOf(inters[0]);
+      if (!g) continue;
+      char *dst = pick(b, inters[0], g->recvType_ == 1 ? 1 : 2);
+      if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+      // what rank r received from other clusters: every receive of its hetero functions
+      std::vector<std::pair<size_t, size_t>> pieces;
+      for (auto &step : p->ranks[r].heteroFuncSteps_)
+        for (auto &h : step)
+          for (auto &o : h.p2pOps_) {
+            if (!o.isRecv_) continue;
+            bool seen = false;
+            for (auto &q : pieces) seen = seen || (q.first == o.offset_ && q.second == o.count_);
+            if (!seen) pieces.push_back({o.offset_, o.count_});
+          }
+      for (auto &q : pieces)
+        LCHECK(flagcxLocalMemcpy(dst + q.first * ts, src + q.first * ts, q.second * ts, stream));
+    } else if (f->homoType_ == 2) {
+      if (p->homoInterRank[r] != 0 || p->homoRank[r] == rt) continue;
+      const int peer = members[rt];
+      const HomoFunc *g = recvOf(peer);
+      if (!g) continue;
+      char *dst = pick(b, peer, g->recvType_ == 1 ? 1 : 2);
+      if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+      LCHECK(flagcxLocalMemcpy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts, stream));
+    }
   }
   return flagcxSuccess;
 }
@@ -483,8 +583,30 @@ flagcxResult_t flagcxLocalPlanCreate(flagcxLocalPlan **plan, int nranks, const i
       p->clusterInterRanks[cl].push_back(r);
     }
   }
+  // multiNic_ / eachNicPerRank_ of the planner's constructor (c2c_algo.cc:636-672)
+  const bool reduceType = p->commOp == flagcxCommOpAllReduce || p->commOp == flagcxCommOpReduceScatter ||
+                          p->commOp == flagcxCommOpReduce;
+  p->multiNic = reduceType ? 1 : 0;
+  p->eachNicPerRank = 1;
+  for (int cl = 0; cl < ncl; cl++) {
+    const size_t inter = p->clusterInterRanks[cl].size();
+    if (reduceType && inter == 1) p->multiNic = 0;
+    if (!reduceType && inter != 1) p->multiNic = 1;
+    if (inter != p->clusterRanks[cl].size()) p->eachNicPerRank = 0;
+  }
+  for (int cl = 0; cl < ncl; cl++)
+    if (p->clusterInterRanks[cl].size() > totalCount) p->multiNic = 0;
   p->ranks.resize(nranks);
   *plan = p;
+  return flagcxSuccess;
+}
+
+// Number of chunks of plan documents that carry no <nChunks> (those written by
+// flagcx/tools/algorithm.py); offsets and counts of a document are in units of
+// totalCount / nChunks elements (c2c_algo.cc:989).
+flagcxResult_t flagcxLocalPlanSetChunks(flagcxLocalPlan *plan, size_t nchunks) {
+  if (!plan || nchunks == 0) return flagcxInvalidArgument;
+  plan->defaultChunks = nchunks;
   return flagcxSuccess;
 }
 
@@ -522,9 +644,19 @@ flagcxResult_t flagcxLocalPlanImportXml(flagcxLocalPlan *p, const char *prefix) 
     if (pos == std::string::npos || !parseNode(text, pos, rootNode) || rootNode.name != "FlagcxC2cPlanner")
       return planFail(p, flagcxInvalidArgument, "%s is not a FlagcxC2cPlanner document", filename);
     RankPlan &rp = p->ranks[r];
-    rp.nchunks_ = rootNode.size("nChunks");
+    // documents written by the reference's plan DSL carry no <nChunks>
+    // (flagcx/tools/algorithm.py:160-181); exportXml always writes it (c2c_algo.cc:1058)
+    rp.nchunks_ = rootNode.child("nChunks") ? rootNode.size("nChunks") : p->defaultChunks;
+    if (rp.nchunks_ == 0 && !rootNode.child("nChunks"))
+      return planFail(p, flagcxInvalidArgument, "%s has no <nChunks>: say how many chunks it counts in (flagcxLocalPlanSetChunks)",
+                      filename);
     if (rp.nchunks_ == 0 || p->totalCount % rp.nchunks_)
       return planFail(p, flagcxInvalidArgument, "%s: nChunks must divide the total count", filename);
+    static const char *const kSizes[] = {"nChunks", "start", "offset", "count", "totalCount", "sendOffset", "recvOffset"};
+    if (const char *neg = rootNode.negativeSize(kSizes, 7)) {
+      snprintf(p->err, sizeof(p->err), "%s: negative <%s>: offsets and counts are sizes", filename, neg);
+      return flagcxInvalidArgument;
+    }
     const size_t cs = p->totalCount / rp.nchunks_; // chunksize = totalCount_ / nchunks_ (c2c_algo.cc:989)
     rp.nSeqPreSteps_ = (int)rootNode.num("nSeqPreSteps");
     rp.nPipePreSteps_ = (int)rootNode.num("nPipePreSteps");
@@ -636,25 +768,42 @@ flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan *p, const void *const *sen
     char *scratch = scratchbuffs ? (char *)scratchbuffs[r] : nullptr;
     recvTmp[r] = scratch ? scratch : (char *)recvbuffs[r];
     const bool fromSend = p->commOp == flagcxCommOpAlltoAll || p->commOp == flagcxCommOpAlltoAllv ||
-                          (p->commOp == flagcxCommOpScatter && r == root);
+                          (p->commOp == flagcxCommOpScatter && r == root) ||
+                          (p->commOp == flagcxCommOpAllGather && p->eachNicPerRank && p->multiNic);
     sendTmp[r] = fromSend ? (char *)const_cast<void *>(sendbuffs[r]) : recvTmp[r];
   }
+  // what the homo functions get as root: the root's rank inside its cluster (c2c_algo.cc:2147,2170)
+  const int homoRoot = (root >= 0 && root < p->nranks) ? p->homoRank[root] : root;
   const bool anyPipe = c.nPipePreSteps_ > 0 || c.nPipePostSteps_ > 0;
   // when the reference refreshes around sequential steps (c2c_algo.cc:2205-2208,2226-2229,2276-2279)
   const bool refreshSeq = p->algorithm == 0 || !anyPipe;
   const bool refreshAfterInter = p->algorithm == 1 && anyPipe;
+  // ranks whose own homoInter table holds a function i in step hs: every rank decides
+  // `homoInterFuncSteps_[s].size() > i` for itself (c2c_algo.cc:2181,2219,2258)
+  std::vector<char> has(p->nranks);
+  auto interAt = [&](int hs, size_t i) {
+    bool any = false;
+    for (int r = 0; r < p->nranks; r++) {
+      auto &t = p->ranks[r].homoInterFuncSteps_;
+      has[r] = hs < (int)t.size() && i < t[hs].size();
+      any = any || has[r];
+    }
+    return any;
+  };
 
   // sequential preHomoFunc steps
   for (int s = 0; s < c.nSeqPreSteps_; s++)
-    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, s, b, datatype, root, stream));
+    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, s, b, datatype, homoRoot, stream));
   LCHECK(runRefresh(p, b, datatype, stream));
   // pipelined preHomoFunc + heteroFunc steps
   for (int s = 0; s < c.nPipePreSteps_; s++) {
-    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, c.nSeqPreSteps_ + s, b, datatype, root, stream));
+    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, c.nSeqPreSteps_ + s, b, datatype, homoRoot, stream));
     for (size_t i = 0; i < heteroWidth(p, s); i++) {
       LCHECK(runHeteroSlot(p, s, (int)i, sendTmp, recvTmp, datatype, stream));
-      LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, s, b, datatype, root, stream, (int)i));
-      LCHECK(runRefresh(p, b, datatype, stream));
+      if (interAt(s, i)) {
+        LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, s, b, datatype, homoRoot, stream, (int)i));
+        LCHECK(runRefresh(p, b, datatype, stream, &has));
+      }
     }
   }
   // sequential heteroFunc steps
@@ -663,22 +812,25 @@ flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan *p, const void *const *sen
     for (size_t i = 0; i < heteroWidth(p, hs); i++) {
       if (refreshSeq) LCHECK(runRefresh(p, b, datatype, stream));
       LCHECK(runHeteroSlot(p, hs, (int)i, sendTmp, recvTmp, datatype, stream));
-      LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, root, stream, (int)i));
-      if (refreshAfterInter) LCHECK(runRefresh(p, b, datatype, stream));
+      if (interAt(hs, i)) {
+        LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, homoRoot, stream, (int)i));
+        if (refreshAfterInter) LCHECK(runRefresh(p, b, datatype, stream, &has));
+      }
     }
   }
   // pipelined heteroFunc + postHomoFunc steps
   for (int s = 0; s < c.nPipePostSteps_; s++) {
-    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, s, b, datatype, root, stream));
+    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, s, b, datatype, homoRoot, stream));
     const int hs = c.nPipePreSteps_ + c.nSeqInterSteps_ + s;
     for (size_t i = 0; i < heteroWidth(p, hs); i++) {
       LCHECK(runHeteroSlot(p, hs, (int)i, sendTmp, recvTmp, datatype, stream));
-      LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, root, stream, (int)i));
+      if (interAt(hs, i))
+        LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, homoRoot, stream, (int)i));
     }
   }
   // sequential postHomoFunc steps
   for (int s = 0; s < c.nSeqPostSteps_; s++)
-    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, c.nPipePostSteps_ + s, b, datatype, root, stream, -1,
+    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, c.nPipePostSteps_ + s, b, datatype, homoRoot, stream, -1,
                        refreshSeq));
   return flagcxSuccess;
 }

@@ -125,7 +125,7 @@ EXPORTS = [
     "flagcxLocalRingReduceScatter",
     "flagcxLocalGetDeviceAdaptor", "flagcxLocalDeviceAdaptorLayout",
     "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
-    "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
+    "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanSetChunks", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
@@ -194,6 +194,7 @@ def lib():
         L.flagcxLocalPlanImportXml.argtypes = [vp, C.c_char_p]
         L.flagcxLocalPlanExportXml.argtypes = [vp, C.c_char_p]
         L.flagcxLocalPlanSetAlgorithm.argtypes = [vp, i]
+        L.flagcxLocalPlanSetChunks.argtypes = [vp, sz]
         L.flagcxLocalPlanExecute.argtypes = [vp, pp, pp, pp, i, i, sp]
         L.flagcxLocalPlanGetLastError.restype = C.c_char_p
         L.flagcxLocalPlanGetLastError.argtypes = [vp]
@@ -397,6 +398,9 @@ class Plan:
 
     def export_xml(self, prefix):
         self._check(lib().flagcxLocalPlanExportXml(self._h, prefix.encode()))
+
+    def set_chunks(self, nchunks):
+        self._check(lib().flagcxLocalPlanSetChunks(self._h, nchunks))
 
     def set_algorithm(self, algo):
         self._check(lib().flagcxLocalPlanSetAlgorithm(self._h, algo))

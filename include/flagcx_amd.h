@@ -523,8 +523,13 @@ flagcxResult_t flagcxLocalStagedReduceScatterNoAlloc(const void *const *sendbuff
  * flagcxC2cPlanner::execute does (c2c_algo.cc:2142-2290).  Homo functions
  * (flagcxC2cHomoFunc::run, c2c_algo.cc:286-511) run on the ranks of a cluster
  * (homoType 1: on its inter-ranks) with the local reduce / copy kernels in place
- * of the vendor CCL, folding in homo-rank order; hetero P2P ops become device
- * copies between the ranks' buffers; the refresh function is flagcxLocalRefresh.
+ * of the vendor CCL, folding in homo-rank order; Send / Recv homo functions of all
+ * three homoTypes and hetero P2P ops become device copies between the ranks'
+ * buffers; the refresh function is flagcxLocalRefresh.  `root` of Execute is a
+ * global rank and reaches the homo functions as its rank inside its cluster, like
+ * globalrank2homorank[root] (c2c_algo.cc:2147,2170).  AlltoAllv is
+ * flagcxNotSupported (its counts are call arguments, not part of a plan); a
+ * document with negative offsets or counts is flagcxInvalidArgument at import.
  * commOp 12 (LocCpy) and 13 (LocRed), reserved by the reference's plan DSL
  * (flagcx/tools/utils.py:43-44), are rank-local copy and
  * recv = OP(send, recv).  Host-side errors of a plan are reported through
@@ -543,6 +548,11 @@ flagcxResult_t flagcxLocalPlanDestroy(flagcxLocalPlan_t plan);
 /* Reads / writes <prefix>_<rank>.xml for every rank. */
 flagcxResult_t flagcxLocalPlanImportXml(flagcxLocalPlan_t plan, const char *prefix);
 flagcxResult_t flagcxLocalPlanExportXml(flagcxLocalPlan_t plan, const char *prefix);
+/* Number of chunks of plan documents that carry no <nChunks> (those written by the
+ * reference's plan DSL, flagcx/tools/algorithm.py:160-181; exportXml always writes
+ * it, c2c_algo.cc:1058): a document's offsets and counts are in units of
+ * totalCount / nChunks elements.  Call before ImportXml. */
+flagcxResult_t flagcxLocalPlanSetChunks(flagcxLocalPlan_t plan, size_t nchunks);
 /* 0 sequential, 1 pipeline, 2 input (default after import). */
 flagcxResult_t flagcxLocalPlanSetAlgorithm(flagcxLocalPlan_t plan, int algorithm);
 /* Host arrays of one device pointer per rank; scratchbuffs may be NULL when the

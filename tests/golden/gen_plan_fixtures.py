@@ -1,0 +1,157 @@
+#!/usr/bin/env python3
+"""Writes the C2C plan fixtures under tests/golden/plans/ with the reference's own
+plan DSL (flagcx/tools/algorithm.py, standard library only), so that the importer
+of flagcxLocalPlanImportXml is tested on files its own author did not format.
+
+Run in the build container only (the reference tree is not on the GPU box):
+
+    python tests/golden/gen_plan_fixtures.py [/root/reference]
+
+The fixtures are data: plan documents, no reference code.  Three sets:
+
+  test_{0..7}.xml        the workflow of flagcx/tools/test.py run as it stands.  Its
+                         cluster-1 half addresses buffers with `rank - 4` where rank
+                         runs 0..3, so those documents hold negative offsets and
+                         global ranks as roots: they pin the DSL's layout (tag order,
+                         pretty-printer whitespace, no <nChunks>, <Step/> for an empty
+                         step) and must be refused at execution, not replayed.
+  allreduce8_{0..7}.xml  the same workflow with the cluster-1 half written out as
+                         its cluster-0 half reads (offsets rank, rank + 4; homo ranks
+                         as roots): an 8-rank all-reduce over 2 clusters of 4,
+                         set_pipeline(1, 0, 1, 1, 1), refresh per rank.
+  allgather4_{0..3}.xml  the all-gather that flagcxC2cPlanner::findStrategy lays out
+                         for 2 clusters of 2 where every rank is an inter-rank
+                         (flagcx/core/c2c_algo.cc:1494-1537, 1668-1690, 1824-1866):
+                         hetero sends read the user send buffer.
+"""
+import os
+import runpy
+import shutil
+import sys
+import tempfile
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+TOOLS = os.path.join(REF, "flagcx", "tools")
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "plans")
+
+
+def reference_example(outdir):
+    """flagcx/tools/test.py, unchanged: it writes output/test_<rank>.xml."""
+    work = tempfile.mkdtemp()
+    os.makedirs(os.path.join(work, "output"))
+    cwd = os.getcwd()
+    os.chdir(work)
+    try:
+        runpy.run_path(os.path.join(TOOLS, "test.py"), run_name="__main__")
+    finally:
+        os.chdir(cwd)
+    for r in range(8):
+        shutil.copy(os.path.join(work, "output", "test_%d.xml" % r), os.path.join(outdir, "test_%d.xml" % r))
+    shutil.rmtree(work)
+
+
+def allreduce8(outdir):
+    from algorithm import (BuffRef, Collective, FlagcxWorkflow, Param, Primitive, RedOp, Stage, add_opr, init_buffer,
+                           set_pipeline, set_refresh, to_xml)
+    with FlagcxWorkflow("allreduce8", Collective.AllReduce, [], [], 8):
+        send, recv = {}, {}
+        for rank in range(8):
+            send[rank] = init_buffer(rank, 0, 8)
+            recv[rank] = init_buffer(rank, 1, 8)
+        set_pipeline(1, 0, 1, 1, 1)
+        for rank in range(8):
+            set_refresh(rank, 1, rank // 4 * 4, rank % 4, 1, 4, RedOp.sum)
+        for cl in range(2):
+            for h in range(4):
+                rank = 4 * cl + h
+                other = 4 * (1 - cl)
+                mine = 4 * cl
+                # pre: the cluster reduce-scatters both halves of the send buffer
+                for half in (0, 4):
+                    add_opr(rank_=rank, stage_=Stage.PreHomoFunc, step_=0,
+                            params_={Param.send_buff: BuffRef(send[rank], half, 4),
+                                     Param.recv_buff: BuffRef(recv[rank], half + h, 1),
+                                     Param.count: 1, Param.homo_type: 0, Param.comm_op: Primitive.ReduceScatter})
+                # hetero step 0: the partial sum of the other cluster's chunk goes over, one of ours comes in
+                add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=0,
+                        params_={Param.peer_or_root_rank: other + (h + 1) % 4, Param.send_offset: other + h,
+                                 Param.recv_offset: -1, Param.count: 1})
+                add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=0,
+                        params_={Param.peer_or_root_rank: other + (h + 3) % 4, Param.send_offset: -1,
+                                 Param.recv_offset: mine + (h + 3) % 4, Param.count: 1})
+                # hetero step 1: the finished chunks are exchanged pairwise
+                add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=1,
+                        params_={Param.peer_or_root_rank: other + h, Param.send_offset: mine + h,
+                                 Param.recv_offset: -1, Param.count: 1})
+                add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=1,
+                        params_={Param.peer_or_root_rank: other + h, Param.send_offset: -1,
+                                 Param.recv_offset: other + h, Param.count: 1})
+                # homo inter: own partial + the one received, scattered back to its owner
+                add_opr(rank_=rank, stage_=Stage.HomoInterFunc, step_=0,
+                        params_={Param.send_buff: BuffRef(recv[rank], mine, 1),
+                                 Param.recv_buff: BuffRef(recv[rank], mine + h, 1),
+                                 Param.count: 1, Param.homo_type: 2, Param.comm_op: Primitive.ReduceScatter})
+                add_opr(rank_=rank, stage_=Stage.HomoInterFunc, step_=1, params_=None)
+                # post: broadcast the cluster's own chunks, then the other cluster's
+                for step, base in ((0, mine), (1, other)):
+                    for root in range(4):
+                        add_opr(rank_=rank, stage_=Stage.PostHomoFunc, step_=step,
+                                params_={Param.peer_or_root_rank: root,
+                                         Param.send_buff: BuffRef(recv[rank], base + root, 1),
+                                         Param.recv_buff: BuffRef(recv[rank], base + root, 1),
+                                         Param.count: 1, Param.homo_type: 2, Param.comm_op: Primitive.Broadcast})
+        for rank in range(8):
+            to_xml(rank_=rank, path_=outdir)
+
+
+def allgather4(outdir):
+    from algorithm import (BuffRef, Collective, FlagcxWorkflow, Param, Primitive, RedOp, Stage, add_opr, init_buffer,
+                           set_pipeline, set_refresh, to_xml)
+    with FlagcxWorkflow("allgather4", Collective.AllGather, [], [], 4):
+        send, recv = {}, {}
+        for rank in range(4):
+            send[rank] = init_buffer(rank, 0, 1)
+            recv[rank] = init_buffer(rank, 1, 4)
+        set_pipeline(1, 0, 1, 0, 1)
+        for rank in range(4):
+            # flagcxC2cRefreshFunc(0, 0, totalCount_, redOp_) with redOp nop: nothing is cleared
+            set_refresh(rank, -1, 0, 0, 0, 4, RedOp.nop)
+        for cl in range(2):
+            for h in range(2):
+                rank, peer = 2 * cl + h, 2 * (1 - cl) + h
+                # pre: all-gather inside the cluster, send[0] -> recv[clusterOffset + homo rank]
+                add_opr(rank_=rank, stage_=Stage.PreHomoFunc, step_=0,
+                        params_={Param.send_buff: BuffRef(send[rank], 0, 1), Param.recv_buff: BuffRef(recv[rank], 2 * cl, 1),
+                                 Param.count: 1, Param.homo_type: 0, Param.comm_op: Primitive.AllGather})
+                # hetero: own block, from offset 0 of the SEND buffer, to the rank of the same homo index
+                add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=0,
+                        params_={Param.peer_or_root_rank: peer, Param.send_offset: 0, Param.recv_offset: -1, Param.count: 1})
+                add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=0,
+                        params_={Param.peer_or_root_rank: peer, Param.send_offset: -1, Param.recv_offset: peer, Param.count: 1})
+                add_opr(rank_=rank, stage_=Stage.HomoInterFunc, step_=0,
+                        params_={Param.send_type: 0, Param.recv_type: 1, Param.send_offset: 0, Param.recv_offset: 0,
+                                 Param.count: 4, Param.homo_type: 1, Param.comm_op: Primitive.Nop})
+                # post: every inter-rank broadcasts the block it received
+                for root in range(2):
+                    blk = 2 * (1 - cl) + root
+                    add_opr(rank_=rank, stage_=Stage.PostHomoFunc, step_=0,
+                            params_={Param.peer_or_root_rank: root, Param.send_buff: BuffRef(recv[rank], blk, 1),
+                                     Param.recv_buff: BuffRef(recv[rank], blk, 1), Param.count: 1, Param.homo_type: 2,
+                                     Param.comm_op: Primitive.Broadcast})
+        for rank in range(4):
+            to_xml(rank_=rank, path_=outdir)
+
+
+def main():
+    if not os.path.isdir(TOOLS):
+        sys.exit("reference tree not found at %s" % REF)
+    sys.path.insert(0, TOOLS)
+    os.makedirs(OUT, exist_ok=True)
+    reference_example(OUT)
+    allreduce8(OUT)
+    allgather4(OUT)
+    print("wrote", sorted(os.listdir(OUT)))
+
+
+if __name__ == "__main__":
+    main()
