@@ -18,6 +18,7 @@
 #include "../../include/flagcx_amd.h"
 
 #include <hip/hip_runtime.h>
+#include <sched.h>
 
 #include <vector>
 
@@ -222,7 +223,14 @@ flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing *r, flagcxLocalR
   size_t copied = 0, handed = 0; // steps whose copy is issued / whose reduce is enqueued
   uint64_t lastTicket = 0, consumed = 0;
   while (handed < nsteps) {
-    RCHECK(flagcxLocalReduceFifoQuery(fifo, nullptr, &consumed, nullptr));
+    const size_t copiedBefore = copied, handedBefore = handed;
+    int state = 0;
+    RCHECK(flagcxLocalReduceFifoQuery(fifo, nullptr, &consumed, &state));
+    // a consumer that has left for good (stopped, or timed out on its spin bound)
+    // frees no more slots: give up instead of waiting for `consumed` to move
+    if (state != FLAGCX_LOCAL_REDUCE_FIFO_RUNNING && state != FLAGCX_LOCAL_REDUCE_FIFO_PARKED && handed > 0 &&
+        consumed < lastTicket)
+      return flagcxInternalError;
     // issue copies into free slots (sendHead side), a group of steps per launch and event
     while (copied < nsteps) {
       const size_t m = groupAt(r, nranks - 1, copied, nsteps, size);
@@ -256,6 +264,7 @@ flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing *r, flagcxLocalR
       ticket[handed % depth] = lastTicket;
       handed++;
     }
+    if (copied == copiedBefore && handed == handedBefore) sched_yield(); // nothing moved: let the copies and the consumer run
   }
   return flagcxLocalReduceFifoWait(fifo, lastTicket);
 }

@@ -139,3 +139,52 @@ def test_ring_rejects_bad_arguments(L):
     ptrs = (C.c_void_p * 3)(mem.data_ptr(), mem.data_ptr(), mem.data_ptr())
     assert lib.flagcxLocalRingReduceScatter(h, ptrs, 3, 0, mem.data_ptr(), 16, 7, 0, C.byref(st), C.byref(st)) == inv
     assert lib.flagcxLocalRingDestroy(h) == 0
+
+
+def test_ring_fifo_returns_when_the_consumer_has_left(L):
+    """A consumer that gives up on its spin bound while the host still waits for ring
+    slots: the call returns an error instead of waiting for `consumed` to move, every
+    kernel having ended normally, and the same queue works again after a restart.
+    (With a spin bound of one poll the consumer leaves at the first entry it cannot
+    finish between two polls; should it get through all the same, the bytes are right.)"""
+    import torch
+    dt, op, nranks, rcount, chunk, steps = O.FP32, O.SUM, 4, 4096 * 64, 4096, 2
+    ts = O.type_size(dt)
+    send_h = make_inputs(dt, nranks, nranks * rcount, seed=99, op=op)
+    send = [to_dev(h) for h in send_h]
+    ring_mem = torch.empty(steps * (nranks - 1) * chunk, dtype=torch.uint8, device="cuda")
+    ring = L.Ring(ring_mem, nranks - 1, chunk, steps)
+    ta, tb, sa, sb = streams(L)
+    out = dev_empty(rcount, ts, fill=0)
+    rc, want = O.reduce_scatter_rank(send_h, 1, rcount, dt, op)
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(8, nranks, dt, op)
+    q.set_linger(0)
+    try:
+        L.lib().flagcxLocalSetMaxSpinCount(1)
+        q.start()
+        try:
+            ring.reduce_scatter_fifo(q, send, 1, out, sa)
+            left = False
+        except L.FlagcxError:
+            left = True
+        torch.cuda.synchronize()              # returns: no kernel is left spinning
+        if left:
+            assert q.query()[2] == 3          # timed out
+            try:
+                q.stop()
+            except L.FlagcxError:
+                pass                          # reports the entries that were not reached
+        else:
+            q.stop()
+            assert same(from_dev(out, send_h[0].dtype), want, nan_class=True, dtype=dt)
+        L.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+        out.zero_()
+        torch.cuda.synchronize()
+        with q:
+            ring.reduce_scatter_fifo(q, send, 1, out, sa)
+        assert same(from_dev(out, send_h[0].dtype), want, nan_class=True, dtype=dt)
+    finally:
+        L.lib().flagcxLocalSetMaxSpinCount(-1)
+        q.close()
+        ring.close()
