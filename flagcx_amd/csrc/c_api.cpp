@@ -3,11 +3,11 @@
 // Thin by design: validate on the host exactly what the kernels and their grids
 // assume (pointers, alignment, overlap, enum ranges), resolve the stream handle,
 // launch.  No allocation, no hipSetDevice, no global mutable state beyond the
-// immutable device-property cache and the launch-shape table.
+// device-property cache, which is written once; the launch-shape tables are
+// constants and their overrides (flagcxLocalTune*) belong to the calling thread.
 #include "../../include/flagcx_amd.h"
 #include "launch.h"
 
-#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -36,9 +36,15 @@ static flagcxResult_t fromHip(int err, const char *what) {
 }
 
 // ----------------------------------------------------------- device facts
-static DeviceInfo gInfo{256, 160 * 1024};
+static DeviceInfo gInfo{256, 160 * 1024, true, true};
 static std::once_flag gInfoOnce;
 static int gInfoErr = 0;
+
+// Never launched: only asked how many copies of it fit on a CU with a given LDS
+// reservation, to see whether this device hands LDS out the way ldsReservation assumes.
+static __global__ void __launch_bounds__(64) ldsProbeKernel(int *p) {
+  if (p) *p = 0;
+}
 
 const DeviceInfo &deviceInfo() {
   std::call_once(gInfoOnce, [] {
@@ -47,6 +53,25 @@ const DeviceInfo &deviceInfo() {
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e == hipSuccess && cus > 0) gInfo.numCU = cus; else gInfoErr = (int)e;
     gInfo.ldsPerCU = 160 * 1024; // gfx950: 160 KiB of LDS per CU
+    if (e != hipSuccess) return;
+    // The caps on resident wavefronts per CU are expressed as LDS reservations in
+    // whole 1280-byte granules, 128 to a CU.  If this device answers differently for
+    // three of them (another LDS size or granule, a partition mode that changes it),
+    // no cap is applied at all: the kernels are correct with any occupancy.
+    gInfo.ldsPerCU = 160 * 1024;
+    for (int w : {8, 14, 25}) {
+      const int granules = (gInfo.ldsPerCU / 1280) / (w + 1) + 1;
+      int fit = 0;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, ldsProbeKernel, 64, (size_t)granules * 1280) != hipSuccess ||
+          fit != w)
+        gInfo.ldsCaps = false;
+    }
+    (void)hipGetLastError();
+    // The channel-group model behind the choice between the `spread` and `aliased`
+    // columns was fitted on the whole device (256 CUs, one memory partition); on
+    // anything else every launch takes the `aliased` column, which runs within a few
+    // percent of the best for any layout.
+    gInfo.fittedLayout = gInfo.numCU == 256;
   });
   return gInfo;
 }
@@ -78,25 +103,30 @@ static const int kLoadsLarge[9] = {0, 0, 1, 1, 2, 2, 2, 2, 2};
 static const int kWavesLarge[9] = {0, 0, 25, 21, 14, 16, 14, 14, 14};
 static const uint64_t kNever = ~0ull;
 static const uint64_t kMinTilesLarge[9] = {kNever, kNever, 131072, 131072, 131072, 16384, 16384, 16384, 16384};
-// explicit settings (flagcxLocalTune, flagcxLocalTuneLoads); -1 = choose as above
-static std::atomic<int> gWaves[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
-static std::atomic<int> gLoads[9] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
+// explicit settings of the calling thread (flagcxLocalTune, flagcxLocalTuneLoads);
+// -1 = choose as above.  Per thread: a caller that fixes the launch shape for its
+// own call sites does not change what other threads' launches do.
+struct TuneOverrides {
+  int waves[9] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
+  int loads[9] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
+};
+static thread_local TuneOverrides tlsTune;
 
 int loadsInFlightFor(int k, uint64_t tiles) {
   if (k < 2 || k > 8) return 0;
-  const int set = gLoads[k].load(std::memory_order_relaxed);
+  const int set = tlsTune.loads[k];
   if (set >= 0) return set < k ? set : 0;
   return tiles >= kMinTilesLarge[k] ? kLoadsLarge[k] : 0;
 }
-int tunedLoadsInFlight(int k) { return (k >= 0 && k <= 8) ? gLoads[k].load(std::memory_order_relaxed) : -1; }
+int tunedLoadsInFlight(int k) { return (k >= 0 && k <= 8) ? tlsTune.loads[k] : -1; }
 void setLoadsInFlight(int k, int loads) {
-  if (k >= 0 && k <= 8) gLoads[k].store(loads, std::memory_order_relaxed);
+  if (k >= 0 && k <= 8) tlsTune.loads[k] = loads;
 }
 
 int wavesPerCUFor(int k, bool spread, int inflight) {
   if (k < 0) k = 0;
   if (k > 8) k = 8;
-  const int set = gWaves[k].load(std::memory_order_relaxed);
+  const int set = tlsTune.waves[k];
   if (set >= 0) return set;
   if (k >= 2 && inflight > 0) {
     // the product of wavefronts and inputs in flight is what has to cover the latency
@@ -105,9 +135,9 @@ int wavesPerCUFor(int k, bool spread, int inflight) {
   }
   return spread ? kWavesSpread[k] : kWavesAliased[k];
 }
-int tunedWavesPerCU(int k) { return (k >= 0 && k <= 8) ? gWaves[k].load(std::memory_order_relaxed) : -1; }
+int tunedWavesPerCU(int k) { return (k >= 0 && k <= 8) ? tlsTune.waves[k] : -1; }
 void setWavesPerCU(int k, int waves) {
-  if (k >= 0 && k <= 8) gWaves[k].store(waves, std::memory_order_relaxed);
+  if (k >= 0 && k <= 8) tlsTune.waves[k] = waves;
 }
 
 // Which of 32 channel groups a KiB of HBM belongs to on MI355X, as far as the
@@ -124,6 +154,7 @@ static inline unsigned channelGroupOf(const void *p) {
 
 bool inputsSpread(const void *const *src, int k) {
   if (k < 4) return true; // one table value serves both cases
+  if (!deviceInfo().fittedLayout) return false;
   const int n = k < 8 ? k : 8;
   uint32_t seen = 0;
   int distinct = 0, middle = 0;
@@ -143,7 +174,7 @@ int ldsReservation(int waves) {
   // LDS is handed out in granules of 1280 bytes, 128 of them per CU: reserve the
   // smallest whole number of granules with which no more than `waves` workgroups
   // fit (exactly `waves` for 8, 9, 10, 11, 12, 14, 16, 18, 21, 25, 32).
-  if (waves <= 0 || waves >= 32) return 0;
+  if (waves <= 0 || waves >= 32 || !deviceInfo().ldsCaps) return 0;
   const int granules = deviceInfo().ldsPerCU / 1280;
   int each = granules / (waves + 1) + 1;
   int bytes = each * 1280;
@@ -378,7 +409,7 @@ flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU) {
 
 flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight) {
   if (nranks < 2 || nranks > 8 || inputsInFlight < -1 || inputsInFlight > 3)
-    return fail(flagcxInvalidArgument, "flagcxLocalTuneLoads: nranks %d (4..8) / inputsInFlight %d (-1..3) out of range", nranks,
+    return fail(flagcxInvalidArgument, "flagcxLocalTuneLoads: nranks %d (2..8) / inputsInFlight %d (-1..3) out of range", nranks,
                 inputsInFlight);
   setLoadsInFlight(nranks, inputsInFlight);
   return flagcxSuccess;
@@ -386,7 +417,7 @@ flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight) {
 
 flagcxResult_t flagcxLocalGetTuneLoads(int nranks, int *inputsInFlight) {
   if (nranks < 2 || nranks > 8 || !inputsInFlight)
-    return fail(flagcxInvalidArgument, "flagcxLocalGetTuneLoads: nranks %d out of range (4..8) or NULL result", nranks);
+    return fail(flagcxInvalidArgument, "flagcxLocalGetTuneLoads: nranks %d out of range (2..8) or NULL result", nranks);
   *inputsInFlight = tunedLoadsInFlight(nranks);
   return flagcxSuccess;
 }

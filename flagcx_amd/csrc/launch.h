@@ -22,7 +22,9 @@ struct ReduceCall {
 // Cached per-process facts about the device the library runs on.
 struct DeviceInfo {
   int numCU;
-  int ldsPerCU; // bytes
+  int ldsPerCU;      // bytes
+  bool ldsCaps;      // LDS reservations cap the wavefronts per CU the way ldsReservation assumes
+  bool fittedLayout; // the device the channel-group model was fitted on (whole MI355X)
 };
 const DeviceInfo &deviceInfo();
 

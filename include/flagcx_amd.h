@@ -154,7 +154,11 @@ flagcxResult_t flagcxLocalPlaceBuffers(void *pool, size_t poolbytes, size_t byte
  * Launches that ask for all inputs at once look at whether the inputs' addresses
  * fall into different HBM channel groups (few wavefronts are best) or collide
  * (more are needed); with a limit the layout of the inputs hardly matters.
- * Process-wide. */
+ * The settings belong to the calling thread: they shape the launches that thread
+ * makes afterwards and nobody else's.  flagcxLocalInit checks once that the device
+ * hands out LDS the way the caps assume (else no cap is applied) and that it is the
+ * whole 256-CU device the channel-group model was fitted on (else every launch takes
+ * the layout-independent choice). */
 flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU);
 flagcxResult_t flagcxLocalGetTune(int nranks, int *wavesPerCU);
 flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight);

@@ -85,3 +85,41 @@ def test_last_error_is_per_thread():
     b.join()
     assert b"sendbuffs is NULL" in seen["bad"]
     assert seen["clean"] == b""
+
+
+def test_tuning_overrides_belong_to_the_calling_thread():
+    """flagcxLocalTune / flagcxLocalTuneLoads shape the launches of the thread that set
+    them: another thread still sees (and launches with) the library's own choice."""
+    import ctypes as C
+    from flagcx_amd import local as L
+    lib = L.lib()
+    seen = {}
+    ready, done = threading.Event(), threading.Event()
+
+    def tuner():
+        assert lib.flagcxLocalTune(8, 25) == 0 and lib.flagcxLocalTuneLoads(8, 1) == 0
+        w, l = C.c_int(-2), C.c_int(-2)
+        assert lib.flagcxLocalGetTune(8, C.byref(w)) == 0 and lib.flagcxLocalGetTuneLoads(8, C.byref(l)) == 0
+        seen["tuner"] = (w.value, l.value)
+        ready.set()
+        done.wait(30)
+        # still set here after the other thread has looked and set its own
+        assert lib.flagcxLocalGetTune(8, C.byref(w)) == 0 and lib.flagcxLocalGetTuneLoads(8, C.byref(l)) == 0
+        seen["tuner_after"] = (w.value, l.value)
+
+    def other():
+        ready.wait(30)
+        w, l = C.c_int(-2), C.c_int(-2)
+        assert lib.flagcxLocalGetTune(8, C.byref(w)) == 0 and lib.flagcxLocalGetTuneLoads(8, C.byref(l)) == 0
+        seen["other"] = (w.value, l.value)
+        assert lib.flagcxLocalTune(8, 10) == 0
+        done.set()
+
+    a, b = threading.Thread(target=tuner), threading.Thread(target=other)
+    a.start()
+    b.start()
+    a.join(60)
+    b.join(60)
+    assert seen == {"tuner": (25, 1), "other": (-1, -1), "tuner_after": (25, 1)}
+    w = C.c_int(-2)
+    assert lib.flagcxLocalGetTune(8, C.byref(w)) == 0 and w.value == -1     # and the main thread was never touched
