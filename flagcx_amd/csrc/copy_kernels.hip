@@ -131,7 +131,7 @@ static int launchCopyT(const CopyParams &p, const ListParams &l, bool vector, un
     uint64_t gx = (p.body + tileBytes - 1) / tileBytes;
     if (gx < 1) gx = 1;
     if (gx > kMaxGridX) gx = kMaxGridX;
-    const int lds = ldsReservation(wavesPerCUFor(0));
+    const int lds = ldsReservation(launchShapeFor(0, 0).waves);
     if (LIST == 0)
       copyWaveKernel<kCopyUnroll><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), lds, stream>>>(p);
     else

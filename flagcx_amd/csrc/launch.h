@@ -24,18 +24,18 @@ struct DeviceInfo {
   int numCU;
   int ldsPerCU;      // bytes
   bool ldsCaps;      // LDS reservations cap the wavefronts per CU the way ldsReservation assumes
-  bool fittedLayout; // the device the channel-group model was fitted on (whole MI355X)
 };
 const DeviceInfo &deviceInfo();
 
-// Resident single-wave workgroups per CU for a k-input reduce (k = 0: copies);
-// `spread`: the inputs' addresses fall into different HBM channel groups.
-int wavesPerCUFor(int k, bool spread = true, int inflight = 0);
-// inputs whose loads a wavefront keeps in flight (0 = all) in a launch of `tiles` KiB per input
-int loadsInFlightFor(int k, uint64_t tiles);
+// Launch shape of a k-input reduce (k = 0: copies) of `tiles` KiB per input: inputs
+// whose loads a wavefront keeps in flight (0 = all) and resident one-wave workgroups
+// per CU (0 = no cap); the calling thread's flagcxLocalTune* settings applied.
+struct LaunchShape {
+  int loads, waves;
+};
+LaunchShape launchShapeFor(int k, uint64_t tiles);
 void setWavesPerCU(int k, int waves);
 int tunedWavesPerCU(int k); // the explicit setting, or -1
-bool inputsSpread(const void *const *src, int k);
 
 // LDS bytes to reserve per workgroup so that at most `waves` one-wave workgroups
 // fit on a CU.  0 when no cap is wanted.

@@ -83,11 +83,11 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   // a limit on the inputs in flight per wavefront trades latency per wavefront for
   // DRAM efficiency: by default only where the launch runs many rounds of resident
   // wavefronts
-  const int inflight = loadsInFlightFor(K, tiles);
-  p.inflight = inflight;
+  const LaunchShape shape = launchShapeFor(K, tiles);
+  p.inflight = shape.loads;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  const int lds = ldsReservation(wavesPerCUFor(K, inflight ? true : inputsSpread(c.src, K), inflight));
+  const int lds = ldsReservation(shape.waves);
   reduceWaveKernel<elem_t, OP, K, U><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
   return (int)hipGetLastError();
 }
@@ -117,7 +117,7 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   // inputs, whatever their layout.
   static const int kWavesUnaligned[9] = {0, 0, 25, 25, 21, 21, 16, 14, 14};
   int waves = c.k > 8 ? tunedWavesPerCU(8) : -1;
-  if (c.k <= 8) waves = (!s.vector && tunedWavesPerCU(c.k) < 0) ? kWavesUnaligned[c.k] : wavesPerCUFor(c.k, inputsSpread(c.src, c.k));
+  if (c.k <= 8) waves = (!s.vector && tunedWavesPerCU(c.k) < 0) ? kWavesUnaligned[c.k] : launchShapeFor(c.k, tiles).waves;
   else if (waves < 0) waves = c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
   const int lds = ldsReservation(waves);
   if (s.vector)
@@ -167,9 +167,9 @@ static int launchBatchFixed(const ReduceCall *calls, const Split *splits, int n)
       totalTiles += tiles;
     }
     if (maxTiles > kMaxGrid) maxTiles = kMaxGrid;
-    const int inflight = loadsInFlightFor(K, totalTiles);
-    for (int i = 0; i < m; i++) bp.seg[i].inflight = inflight;
-    const int lds = ldsReservation(wavesPerCUFor(K, inputsSpread(calls[base].src, K), inflight));
+    const LaunchShape shape = launchShapeFor(K, totalTiles);
+    for (int i = 0; i < m; i++) bp.seg[i].inflight = shape.loads;
+    const int lds = ldsReservation(shape.waves);
     reduceBatchKernel<elem_t, OP, K, U>
         <<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, calls[0].stream>>>(bp);
     const int err = (int)hipGetLastError();

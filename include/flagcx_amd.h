@@ -149,16 +149,13 @@ flagcxResult_t flagcxLocalPlaceBuffers(void *pool, size_t poolbytes, size_t byte
  * the values measured on MI355X.
  * TuneLoads: of how many of its `nranks` inputs (2..8) a wavefront keeps the loads
  * in flight before it asks for the next: 1..3, 0 = all of them at once, -1 (the
- * default) = two (one with two or three inputs) in large launches - 16 MiB per
- * input and more, 128 MiB with up to four inputs - and all at once below.
- * Launches that ask for all inputs at once look at whether the inputs' addresses
- * fall into different HBM channel groups (few wavefronts are best) or collide
- * (more are needed); with a limit the layout of the inputs hardly matters.
+ * default) = by size: all at once with 18-25 wavefronts per CU in small launches,
+ * one or two from 16-96 MiB per input on (from 16 MiB with five and more inputs,
+ * 32 MiB with three or four, 96 MiB with two), where 14-25 wavefronts per CU each
+ * waiting for its previous input keep DRAM busier than bursts of all inputs.
  * The settings belong to the calling thread: they shape the launches that thread
  * makes afterwards and nobody else's.  flagcxLocalInit checks once that the device
- * hands out LDS the way the caps assume (else no cap is applied) and that it is the
- * whole 256-CU device the channel-group model was fitted on (else every launch takes
- * the layout-independent choice). */
+ * hands out LDS the way the caps assume (else no cap is applied). */
 flagcxResult_t flagcxLocalTune(int nranks, int wavesPerCU);
 flagcxResult_t flagcxLocalGetTune(int nranks, int *wavesPerCU);
 flagcxResult_t flagcxLocalTuneLoads(int nranks, int inputsInFlight);
