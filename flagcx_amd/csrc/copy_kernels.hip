@@ -6,8 +6,8 @@
 // 1 KiB request and a tile is U consecutive KiB of one chunk.  blockIdx.y walks
 // chunks (or list entries), blockIdx.x walks tiles inside a chunk.  Buffer
 // descriptors are clipped to the tile, so ragged chunk ends need no branches.
-// A contiguous copy whose two sides differ modulo 16 is tiled on the destination
-// and reads its source with unaligned 16-byte loads; strided forms whose chunk
+// A contiguous copy whose two sides differ modulo 16 goes to the one-input reduce
+// kernel for misaligned sources (aligned loads, lane shifts); strided forms whose chunk
 // sizes or strides are not multiples of 16 go through an element path at the
 // widest width every address shares.
 // HBM bound: 2 bytes of traffic per payload byte (1 for fills); no LDS, no MFMA.
@@ -77,29 +77,6 @@ __global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p) {
 template <int U, int LIST>
 __global__ void __launch_bounds__(64) copyWaveListKernel(CopyParams p, ListParams l) {
   copyWaveBody<U, LIST>(p, &l);
-}
-
-// One contiguous run whose two sides sit at different offsets modulo 16: tiled on
-// the destination (aligned stores), source read with unaligned 16-byte loads.
-__global__ void __launch_bounds__(64) copyWaveUnalignedKernel(CopyParams p, const char *src0, char *dst0) {
-  const uint64_t nvec = p.body / 16;
-  const uint64_t ntiles = (nvec + 63) / 64;
-  const char *s = src0 + p.head;
-  char *d = dst0 + p.head;
-  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const uint64_t i = t * 64 + threadIdx.x;
-    if (i < nvec) {
-      const u32x4 v = __builtin_nontemporal_load((const u32x4_unaligned *)(s + i * 16));
-      *(u32x4 *)(d + i * 16) = v;
-    }
-  }
-  if (blockIdx.x == gridDim.x - 1) {
-    const uint64_t edge = p.head + p.tail;
-    if (threadIdx.x < edge) {
-      const uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.body + (threadIdx.x - p.head);
-      dst0[i] = src0[i];
-    }
-  }
 }
 
 // Element path: W-byte units, chunk by chunk.
@@ -205,11 +182,16 @@ int launchCopy2D(const Copy2D &c) {
     p.tail = c.chunkBytes - head - p.body;
     vector = sameMis;
     if (!vector) {
-      uint64_t gx = (p.body / 16 + 63) / 64;
-      if (gx < 1) gx = 1;
-      if (gx > kMaxGridX) gx = kMaxGridX;
-      copyWaveUnalignedKernel<<<dim3((unsigned)gx), dim3(64), 0, c.stream>>>(p, src0, dst0);
-      return (int)hipGetLastError();
+      // the two sides sit at different offsets modulo 16: a one-input byte "reduce",
+      // which reads the source with aligned loads and puts it in place with lane shifts
+      ReduceCall r;
+      r.src[0] = src0;
+      r.dst = dst0;
+      r.count = c.chunkBytes;
+      r.k = 1;
+      r.op = 0; // sum of one input: the input
+      r.stream = c.stream;
+      return reduceLauncherFor(1 /* flagcxUint8 */)(r);
     }
   } else {
     vector = allAligned && (c.chunkBytes & 15u) == 0;

@@ -375,4 +375,121 @@ __global__ void __launch_bounds__(64) reduceWaveUnalignedKernel(ReduceParams<FLA
   }
 }
 
+// ------------------------------------------------- sources at other offsets
+// The same sources read with ALIGNED 16-byte loads and put in place with lane
+// shifts.  The output is tiled like the aligned kernel (64 vectors of 16 bytes per
+// wavefront and tile, after p.head elements); output vector v of source j needs
+// bytes [16 v + d_j, 16 v + d_j + 16) counted from the source's aligned base, i.e.
+// the top of aligned granule v and the bottom of granule v + 1, where d_j = the
+// source's offset inside a 16-byte line minus the destination's.  Lane i loads
+// granule 64 t + i of every source, takes granule 64 t + i + 1 from lane i + 1, and
+// lane 63 takes it from lane 0 of the NEXT tile, which the same wavefront has
+// already asked for: a wavefront walks R consecutive tiles, one tile ahead with its
+// loads, so every granule is fetched once (plus one granule per R tiles), where
+// unaligned 16-byte loads touch a ninth cache line per KiB, and in another XCD's L2
+// than the wavefront that fetches the rest of that line.
+// Descriptors are clipped to the granules that hold source bytes, so nothing
+// outside a source's own 16-byte lines is ever read.
+template <int K>
+struct ShiftParams {
+  const void *base[K]; // source address rounded down to 16, at the first body element
+  uint32_t shift[K];   // d_j in bytes, 0..15 (a multiple of the element size)
+  uint64_t granules[K]; // aligned 16-byte granules of source j that hold body bytes
+  const void *src[K];  // original pointers (head and tail elements)
+  void *dst;
+  uint64_t nvec, head, tail;
+  int32_t tilesPerWave;
+};
+
+// bytes [4 Q + b, 4 Q + b + 16) of the 32 bytes (lo, hi).  Q is a template argument
+// and the caller branches on it (it is wave-uniform): with a run-time register index
+// the compiler moves the eight words into LDS and indexes them there.
+template <int Q>
+__device__ __forceinline__ u32x4 funnel16q(const u32x4 lo, const u32x4 hi, uint32_t b) {
+  const uint32_t w0 = Q == 0 ? lo[0] : Q == 1 ? lo[1] : Q == 2 ? lo[2] : lo[3];
+  const uint32_t w1 = Q == 0 ? lo[1] : Q == 1 ? lo[2] : Q == 2 ? lo[3] : hi[0];
+  const uint32_t w2 = Q == 0 ? lo[2] : Q == 1 ? lo[3] : Q == 2 ? hi[0] : hi[1];
+  const uint32_t w3 = Q == 0 ? lo[3] : Q == 1 ? hi[0] : Q == 2 ? hi[1] : hi[2];
+  const uint32_t w4 = Q == 0 ? hi[0] : Q == 1 ? hi[1] : Q == 2 ? hi[2] : hi[3];
+  u32x4 r;
+  r[0] = __builtin_amdgcn_alignbyte(w1, w0, b);
+  r[1] = __builtin_amdgcn_alignbyte(w2, w1, b);
+  r[2] = __builtin_amdgcn_alignbyte(w3, w2, b);
+  r[3] = __builtin_amdgcn_alignbyte(w4, w3, b);
+  return r;
+}
+__device__ __forceinline__ u32x4 funnel16(const u32x4 lo, const u32x4 hi, uint32_t q, uint32_t b) {
+  switch (q) {
+    case 0: return funnel16q<0>(lo, hi, b);
+    case 1: return funnel16q<1>(lo, hi, b);
+    case 2: return funnel16q<2>(lo, hi, b);
+    default: return funnel16q<3>(lo, hi, b);
+  }
+}
+
+template <typename T, int OP, int K>
+__global__ void __launch_bounds__(64) reduceWaveShiftKernel(ShiftParams<K> p) {
+  constexpr int N = 16 / sizeof(T);
+  const uint32_t lane = threadIdx.x;
+  const uint64_t ntiles = (p.nvec + 63) / 64;
+  const uint64_t R = (uint64_t)p.tilesPerWave;
+  const uint64_t headBytes = p.head * sizeof(T);
+  for (uint64_t t0 = (uint64_t)blockIdx.x * R; t0 < ntiles; t0 += (uint64_t)gridDim.x * R) {
+    const uint64_t tEnd = t0 + R < ntiles ? t0 + R : ntiles;
+    // Granules of a tile: a descriptor from granule 64 t on, clipped to the source's own
+    // granules and to `want` of them: 64 for a tile of this walk, 1 for the tile after
+    // the walk (only its first granule is needed, by lane 63 of the last tile), 0 beyond.
+    auto loadTile = [&](u32x4 (&out)[K], uint64_t t) {
+      const uint64_t want = t < tEnd ? 64 : t == tEnd ? 1 : 0;
+#pragma unroll
+      for (int j = 0; j < K; j++) {
+        const uint64_t g0 = t * 64;
+        const uint64_t left = p.granules[j] > g0 ? p.granules[j] - g0 : 0;
+        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)((const char *)p.base[j] + g0 * 16), 0, (uint32_t)(left < want ? left : want) * 16u, kRsrcFlags);
+        out[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16u, 0, kLoadAux);
+      }
+    };
+    u32x4 cur[K], nxt[K];
+    loadTile(cur, t0);
+    loadTile(nxt, t0 + 1);
+    for (uint64_t t = t0; t < tEnd; t++) {
+      u32x4 in[K];
+#pragma unroll
+      for (int j = 0; j < K; j++) {
+        u32x4 hi;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+          const uint32_t fromNext = __builtin_amdgcn_readfirstlane(nxt[j][d]); // lane 0 of the next tile
+          // wave_shl:1 - lane i reads lane i + 1; lane 63 has no source lane and keeps `old`
+          hi[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)fromNext, (int)cur[j][d], 0x130, 0xf, 0xf, false);
+        }
+        in[j] = funnel16(cur[j], hi, p.shift[j] >> 2, p.shift[j] & 3u);
+      }
+      // the tile after next is asked for before this one is folded: its loads are in
+      // flight during the arithmetic (the registers of `cur` are free from here on)
+      loadTile(cur, t + 2);
+      const uint64_t off = t * 1024;
+      const uint64_t left = p.nvec * 16 - off;
+      __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
+          (void *)((char *)p.dst + headBytes + off), 0, left < 1024 ? (uint32_t)left : 1024u, kRsrcFlags);
+      __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, lane * 16u, 0, kStoreAux);
+#pragma unroll
+      for (int j = 0; j < K; j++) {
+        const u32x4 tmp = nxt[j];
+        nxt[j] = cur[j];
+        cur[j] = tmp;
+      }
+    }
+  }
+  // head and tail elements (fewer than 2*N <= 32): last workgroup, one lane each
+  if (blockIdx.x == gridDim.x - 1) {
+    const uint64_t edge = p.head + p.tail;
+    if (threadIdx.x < edge) {
+      uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
+      foldScalar<T, OP>(p.src, K, p.dst, i);
+    }
+  }
+}
+
 } // namespace flagcx_amd

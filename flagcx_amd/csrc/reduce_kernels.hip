@@ -111,14 +111,10 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   // 10, more want 8 (85-86 %).  An explicit flagcxLocalTune(8, n) overrides.
   // (A limit on the inputs in flight, as the kernels for up to eight inputs have
   // it, gains nothing here: within one percent for 9..32 inputs.)
-  // Sources at another offset modulo 16 than the output (up to eight of them come
-  // here too) are bound by the unaligned loads themselves, 68-78 % of peak, and
-  // want more wavefronts to get there: measured 25, 21, 14 per CU for 2, 4, 8
-  // inputs, whatever their layout.
-  static const int kWavesUnaligned[9] = {0, 0, 25, 25, 21, 21, 16, 14, 14};
-  int waves = c.k > 8 ? tunedWavesPerCU(8) : -1;
-  if (c.k <= 8) waves = (!s.vector && tunedWavesPerCU(c.k) < 0) ? kWavesUnaligned[c.k] : launchShapeFor(c.k, tiles).waves;
-  else if (waves < 0) waves = c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
+  // More than eight sources at another offset modulo 16 than the output are read
+  // with unaligned 16-byte loads (up to eight take the lane-shift kernel above).
+  int waves = tunedWavesPerCU(8);
+  if (waves < 0) waves = c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
   const int lds = ldsReservation(waves);
   if (s.vector)
     reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
@@ -127,9 +123,56 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   return (int)hipGetLastError();
 }
 
+// Sources at another offset modulo 16 than the output, up to eight of them: aligned
+// loads put in place with lane shifts, a wavefront walking consecutive tiles.
+template <int OP, int K>
+static int launchShift(const ReduceCall &c, const Split &s) {
+  ShiftParams<K> p;
+  const uint64_t headBytes = s.head * sizeof(elem_t);
+  for (int j = 0; j < K; j++) {
+    const uintptr_t first = (uintptr_t)c.src[j] + headBytes;
+    p.base[j] = (const void *)(first & ~(uintptr_t)15);
+    p.shift[j] = (uint32_t)(first & 15u);
+    p.granules[j] = s.nvec + (p.shift[j] ? 1 : 0);
+    p.src[j] = c.src[j];
+  }
+  p.dst = c.dst;
+  p.nvec = s.nvec;
+  p.head = s.head;
+  p.tail = s.tail;
+  const uint64_t tiles = (s.nvec + 63) / 64;
+  // Two tiles per wavefront: the look-ahead granule costs one extra 16-byte load per
+  // two KiB of every source, and the wavefront is short-lived enough for the
+  // dispatcher to keep the tiles in work dense (4 and 8 tiles measured 2-6 points of
+  // peak lower for 256 MiB inputs).  Wavefronts per CU measured best at 25 / 21 / 16
+  // for up to 3 / 4 / more inputs (bf16, 64 and 256 MiB per input: 73-78, 75-77 and
+  // 70-74 % of peak, against 68-72 % with unaligned 16-byte loads).
+  constexpr int walk = 2;
+  p.tilesPerWave = walk;
+  uint64_t grid = (tiles + (uint64_t)walk - 1) / (uint64_t)walk;
+  if (grid < 1) grid = 1;
+  if (grid > kMaxGrid) grid = kMaxGrid;
+  const int tuned = tunedWavesPerCU(K);
+  const int lds = ldsReservation(tuned >= 0 ? tuned : K <= 3 ? 25 : K == 4 ? 21 : 16);
+  reduceWaveShiftKernel<elem_t, OP, K><<<dim3((unsigned)grid), dim3(64), lds, c.stream>>>(p);
+  return (int)hipGetLastError();
+}
+
 template <int OP>
 static int launchOp(const ReduceCall &c) {
   const Split s = splitFor(c);
+  if (!s.vector && c.k <= 8) {
+    switch (c.k) {
+      case 1: return launchShift<OP, 1>(c, s);
+      case 2: return launchShift<OP, 2>(c, s);
+      case 3: return launchShift<OP, 3>(c, s);
+      case 4: return launchShift<OP, 4>(c, s);
+      case 5: return launchShift<OP, 5>(c, s);
+      case 6: return launchShift<OP, 6>(c, s);
+      case 7: return launchShift<OP, 7>(c, s);
+      default: return launchShift<OP, 8>(c, s);
+    }
+  }
   if (!s.vector || c.k > 8) return launchAny<OP>(c, s);
   switch (c.k) {
     case 1: return launchFixed<OP, 1>(c, s);
