@@ -188,3 +188,24 @@ def test_ring_fifo_returns_when_the_consumer_has_left(L):
         L.lib().flagcxLocalSetMaxSpinCount(-1)
         q.close()
         ring.close()
+
+
+@pytest.mark.parametrize("size,chunk,steps", [(4096 * 9 + 5, 4096, 4), (1 << 20, 65536, 16)])
+def test_ring_send_recv_through_a_host_bounce_buffer(L, size, chunk, steps):
+    """The socket transport's variant of the staging steps (flagcx/core/net.cc:153-161,
+    298-306): the ring is pinned host memory, so the producer's copies are device-to-host
+    and the consumer's host-to-device, done by the same copy kernels over PCIe."""
+    import torch
+    ring_mem = torch.empty(steps * chunk, dtype=torch.uint8, pin_memory=True)
+    ring = L.Ring(ring_mem, 1, chunk, steps)
+    h = np.random.default_rng(size).integers(0, 256, size, dtype=np.uint8)
+    src = to_dev(h)
+    dst = torch.full((size + 16,), 0x5A, dtype=torch.uint8, device="cuda")
+    ta, tb, sa, sb = streams(L)
+    torch.cuda.synchronize()
+    ring.send_recv(dst.data_ptr(), src.data_ptr(), size, sa, sb)
+    tb.synchronize()
+    ta.synchronize()
+    got = from_dev(dst, np.uint8)
+    assert same(got[:size], h) and (got[size:] == 0x5A).all()
+    ring.close()
