@@ -212,6 +212,8 @@ struct flagcxLocalPlan {
   int algorithm = 2; // flagcxAlgoInput: what importXml sets (c2c_algo.h:15-19, c2c_algo.cc:974)
   size_t defaultChunks = 0; // nChunks of documents that carry none (flagcxLocalPlanSetChunks)
   int eachNicPerRank = 0, multiNic = 0; // as the planner's constructor sets them (c2c_algo.cc:636-672)
+  // AlltoAllv: row r of each matrix is the array rank r hands to execute() (c2c_algo.cc:2042-2046,2083-2094)
+  std::vector<size_t> sendCounts, sDispls, recvCounts, rDispls;
   bool loaded = false;
   char err[256] = "";
 };
@@ -304,6 +306,37 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
     }
     if (op == flagcxCommOpSend || op == flagcxCommOpRecv) {
       LCHECK(runSendRecv(p, cl, fn, b, ts, root, stream));
+      continue;
+    }
+    if (op == flagcxCommOpAlltoAllv) {
+      // every member sends to and receives from the members of its own cluster, counts and
+      // displacements from the caller's arrays, buffers without offsets (c2c_algo.cc:482-508)
+      const size_t n = (size_t)p->nranks;
+      if (p->sendCounts.empty())
+        return planFail(p, flagcxInvalidArgument, "AlltoAllv needs counts and displacements (flagcxLocalPlanSetAlltoAllv)%s", "");
+      for (int r : mem) {
+        const HomoFunc *f = fn[r];
+        char *src = pick(b, r, f->sendType_);
+        if (!src) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+        for (int i : p->clusterRanks[cl]) {
+          const size_t cnt = p->sendCounts[r * n + i];
+          const HomoFunc *g = fn[i];
+          const bool recvs = g && g->commOp_ == op && !(g->homoType_ == 1 && p->homoInterRank[i] == -1);
+          if (cnt != (recvs ? p->recvCounts[i * n + r] : 0))
+            return planFail(p, flagcxInvalidUsage, "AlltoAllv: rank %s%lld sends to rank %lld what that rank does not receive", "", r, i);
+          if (!cnt) continue;
+          char *dst = pick(b, i, g->recvType_ == 1 ? 1 : 2);
+          if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+          LCHECK(flagcxLocalMemcpy(dst + p->rDispls[i * n + r] * ts, src + p->sDispls[r * n + i] * ts, cnt * ts, stream));
+        }
+      }
+      // a receive nobody sends would hang the reference
+      for (int i : mem)
+        for (int r : p->clusterRanks[cl]) {
+          const bool sends = fn[r] && fn[r]->commOp_ == op && !(fn[r]->homoType_ == 1 && p->homoInterRank[r] == -1);
+          if (p->recvCounts[i * n + r] && !sends)
+            return planFail(p, flagcxInvalidUsage, "AlltoAllv: rank %s%lld receives from rank %lld what that rank does not send", "", i, r);
+        }
       continue;
     }
     // the communicator the reference would use: homoInterComm for homoType 1, else homo_comm
@@ -607,6 +640,24 @@ flagcxResult_t flagcxLocalPlanCreate(flagcxLocalPlan **plan, int nranks, const i
 flagcxResult_t flagcxLocalPlanSetChunks(flagcxLocalPlan *plan, size_t nchunks) {
   if (!plan || nchunks == 0) return flagcxInvalidArgument;
   plan->defaultChunks = nchunks;
+  return flagcxSuccess;
+}
+
+// Counts and displacements (in elements) of an AlltoAllv: four nranks x nranks matrices,
+// row r = the arrays rank r passes to flagcxC2cPlanner::execute (c2c_algo.cc:2042-2046).
+// The hetero functions of the plan carry the cross-cluster pieces themselves
+// (c2c_algo.cc:1618-1630); the homo function reads these for the pieces inside a cluster.
+flagcxResult_t flagcxLocalPlanSetAlltoAllv(flagcxLocalPlan *p, const size_t *sendCounts, const size_t *sDispls,
+                                           const size_t *recvCounts, const size_t *rDispls) {
+  if (!p) return flagcxInvalidArgument;
+  // c2c_algo.cc:2083-2089
+  if (!sendCounts || !sDispls || !recvCounts || !rDispls)
+    return planFail(p, flagcxInvalidArgument, "sendrecv counts and displacements need to be set for AlltoAllv%s", "");
+  const size_t n = (size_t)p->nranks * (size_t)p->nranks;
+  p->sendCounts.assign(sendCounts, sendCounts + n);
+  p->sDispls.assign(sDispls, sDispls + n);
+  p->recvCounts.assign(recvCounts, recvCounts + n);
+  p->rDispls.assign(rDispls, rDispls + n);
   return flagcxSuccess;
 }
 

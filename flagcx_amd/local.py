@@ -125,7 +125,7 @@ EXPORTS = [
     "flagcxLocalRingReduceScatter",
     "flagcxLocalGetDeviceAdaptor", "flagcxLocalDeviceAdaptorLayout",
     "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
-    "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanSetChunks", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
+    "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanSetChunks", "flagcxLocalPlanSetAlltoAllv", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
@@ -195,6 +195,8 @@ def lib():
         L.flagcxLocalPlanExportXml.argtypes = [vp, C.c_char_p]
         L.flagcxLocalPlanSetAlgorithm.argtypes = [vp, i]
         L.flagcxLocalPlanSetChunks.argtypes = [vp, sz]
+        szp = C.POINTER(C.c_size_t)
+        L.flagcxLocalPlanSetAlltoAllv.argtypes = [vp, szp, szp, szp, szp]
         L.flagcxLocalPlanExecute.argtypes = [vp, pp, pp, pp, i, i, sp]
         L.flagcxLocalPlanGetLastError.restype = C.c_char_p
         L.flagcxLocalPlanGetLastError.argtypes = [vp]
@@ -401,6 +403,16 @@ class Plan:
 
     def set_chunks(self, nchunks):
         self._check(lib().flagcxLocalPlanSetChunks(self._h, nchunks))
+
+    def set_alltoallv(self, send_counts, s_displs, recv_counts, r_displs):
+        """Four nranks x nranks matrices (nested lists), row r = rank r's arrays, in elements."""
+        def flat(m):
+            if m is None:
+                return None
+            v = [int(x) for row in m for x in row]
+            return (C.c_size_t * len(v))(*v)
+        self._check(lib().flagcxLocalPlanSetAlltoAllv(self._h, flat(send_counts), flat(s_displs), flat(recv_counts),
+                                                      flat(r_displs)))
 
     def set_algorithm(self, algo):
         self._check(lib().flagcxLocalPlanSetAlgorithm(self._h, algo))

@@ -554,6 +554,15 @@ flagcxResult_t flagcxLocalPlanExportXml(flagcxLocalPlan_t plan, const char *pref
  * it, c2c_algo.cc:1058): a document's offsets and counts are in units of
  * totalCount / nChunks elements.  Call before ImportXml. */
 flagcxResult_t flagcxLocalPlanSetChunks(flagcxLocalPlan_t plan, size_t nchunks);
+/* Counts and displacements of an AlltoAllv, in elements: four nranks x nranks
+ * matrices, row r = the arrays rank r passes to flagcxC2cPlanner::execute
+ * (flagcx/core/c2c_algo.cc:2042-2046; NULL -> flagcxInvalidArgument as
+ * c2c_algo.cc:2083-2089).  The plan's hetero functions carry the cross-cluster
+ * pieces (c2c_algo.cc:1618-1630); its AlltoAllv homo function moves the pieces
+ * inside a cluster from these arrays (c2c_algo.cc:482-508).  Call before Execute. */
+flagcxResult_t flagcxLocalPlanSetAlltoAllv(flagcxLocalPlan_t plan, const size_t *sendCounts,
+                                           const size_t *sDispls, const size_t *recvCounts,
+                                           const size_t *rDispls);
 /* 0 sequential, 1 pipeline, 2 input (default after import). */
 flagcxResult_t flagcxLocalPlanSetAlgorithm(flagcxLocalPlan_t plan, int algorithm);
 /* Host arrays of one device pointer per rank; scratchbuffs may be NULL when the

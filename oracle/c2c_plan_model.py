@@ -169,6 +169,17 @@ class Model:
             if op in (SEND, RECV):
                 writes += self._send_recv(cl, fn, root)
                 continue
+            if op == ALLTOALLV:                              # c2c_algo.cc:482-508: peers of the own cluster only
+                sc, sd, rc, rd = self.v_args
+                for r in have:
+                    for i in members:
+                        cnt = sc[r][i]
+                        assert cnt == (rc[i][r] if i in fn else 0), "unmatched AlltoAllv piece %d -> %d" % (r, i)
+                        if cnt:
+                            src = self._buf(r, fn[r].send_type)
+                            dst = self._buf(i, 1 if fn[i].recv_type == 1 else 2)
+                            writes.append((dst, rd[i][r], src[sd[r][i]:sd[r][i] + cnt].copy()))
+                continue
             S = [self._buf(r, fn[r].send_type) for r in comm]
             D = [self._buf(r, 1 if fn[r].recv_type == 1 else 2) for r in comm]
             so, ro = [fn[r].send_off for r in comm], [fn[r].recv_off for r in comm]
@@ -276,8 +287,10 @@ class Model:
     def _width(self, table, s):
         return max((len(getattr(p, table)[s]) if s < len(getattr(p, table)) else 0) for p in self.plans)
 
-    def execute(self, send, recv, scratch, root=-1, algorithm=ALGO_INPUT):
-        """flagcxC2cPlanner::execute, c2c_algo.cc:2121-2298; buffers are modified in place."""
+    def execute(self, send, recv, scratch, root=-1, algorithm=ALGO_INPUT, v_args=None):
+        """flagcxC2cPlanner::execute, c2c_algo.cc:2121-2298; buffers are modified in place.
+        v_args: (sendCounts, sDispls, recvCounts, rDispls) of an AlltoAllv, row r = rank r's arrays."""
+        self.v_args = v_args
         self.send, self.recv = send, recv
         self.scratch = scratch if scratch is not None else [None] * self.n
         self.algorithm = algorithm

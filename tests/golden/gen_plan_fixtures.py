@@ -23,6 +23,13 @@ The fixtures are data: plan documents, no reference code.  Three sets:
                          for 2 clusters of 2 where every rank is an inter-rank
                          (flagcx/core/c2c_algo.cc:1494-1537, 1668-1690, 1824-1866):
                          hetero sends read the user send buffer.
+  alltoallv4_{0..3}.xml  the all-to-all-v that findStrategy lays out for 2 clusters of 2
+                         (flagcx/core/c2c_algo.cc:1554-1556, 1618-1630, and the NoOp inter
+                         and post functions): the pieces for the own cluster travel in the
+                         AlltoAllv homo function, whose counts are arguments of execute()
+                         and not part of the document; the cross-cluster pieces are P2P ops
+                         with their displacements and counts.  ALLTOALLV_UNITS below is the
+                         count / displacement matrix in chunks, shared with the test.
 """
 import os
 import runpy
@@ -142,6 +149,63 @@ def allgather4(outdir):
             to_xml(rank_=rank, path_=outdir)
 
 
+# sendCounts[r][i] in chunks: rank r sends that many chunks to rank i (ragged, one empty piece
+# inside a cluster, one across); displacements pack the pieces in peer order
+ALLTOALLV_UNITS = [[1, 2, 3, 0],
+                   [0, 1, 1, 2],
+                   [2, 0, 1, 3],
+                   [1, 1, 2, 1]]
+
+
+def alltoallv_layout(units=ALLTOALLV_UNITS):
+    n = len(units)
+    send = [list(row) for row in units]
+    recv = [[units[r][i] for r in range(n)] for i in range(n)]
+    sd = [[sum(send[r][:i]) for i in range(n)] for r in range(n)]
+    rd = [[sum(recv[i][:r]) for r in range(n)] for i in range(n)]
+    return send, sd, recv, rd
+
+
+def alltoallv4(outdir):
+    from algorithm import (BuffRef, Collective, FlagcxWorkflow, Param, Primitive, RedOp, Stage, add_opr, init_buffer,
+                           set_pipeline, set_refresh, to_xml)
+    send_c, sd, recv_c, rd = alltoallv_layout()
+    with FlagcxWorkflow("alltoallv4", Collective.AlltoAllv, [], [], 4):
+        send, recv = {}, {}
+        for rank in range(4):
+            send[rank] = init_buffer(rank, 0, 8)
+            recv[rank] = init_buffer(rank, 1, 8)
+        set_pipeline(1, 0, 1, 0, 1)
+        for rank in range(4):
+            set_refresh(rank, -1, 0, 0, 0, 8, RedOp.nop)
+        for rank in range(4):
+            cl = rank // 2
+            # pre: AlltoAllv inside the cluster; offsets and count stay 0 (c2c_algo.cc:1554-1556)
+            add_opr(rank_=rank, stage_=Stage.PreHomoFunc, step_=0,
+                    params_={Param.send_buff: BuffRef(send[rank], 0, 0), Param.recv_buff: BuffRef(recv[rank], 0, 0),
+                             Param.count: 0, Param.homo_type: 0, Param.comm_op: Primitive.AlltoAllv})
+            # hetero: one send and one receive per rank of the other cluster that has something (c2c_algo.cc:1618-1630)
+            for i in range(4):
+                if i // 2 == cl:
+                    continue
+                if send_c[rank][i]:
+                    add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=0,
+                            params_={Param.peer_or_root_rank: i, Param.send_offset: sd[rank][i], Param.recv_offset: -1,
+                                     Param.count: send_c[rank][i]})
+                if recv_c[rank][i]:
+                    add_opr(rank_=rank, stage_=Stage.HeteroFunc, step_=0,
+                            params_={Param.peer_or_root_rank: i, Param.send_offset: -1, Param.recv_offset: rd[rank][i],
+                                     Param.count: recv_c[rank][i]})
+            add_opr(rank_=rank, stage_=Stage.HomoInterFunc, step_=0,
+                    params_={Param.send_type: 0, Param.recv_type: 1, Param.send_offset: 0, Param.recv_offset: 0,
+                             Param.count: 8, Param.homo_type: 1, Param.comm_op: Primitive.Nop})
+            add_opr(rank_=rank, stage_=Stage.PostHomoFunc, step_=0,
+                    params_={Param.send_type: 0, Param.recv_type: 1, Param.send_offset: 0, Param.recv_offset: 0,
+                             Param.count: 8, Param.homo_type: 2, Param.comm_op: Primitive.Nop})
+        for rank in range(4):
+            to_xml(rank_=rank, path_=outdir)
+
+
 def main():
     if not os.path.isdir(TOOLS):
         sys.exit("reference tree not found at %s" % REF)
@@ -150,6 +214,7 @@ def main():
     reference_example(OUT)
     allreduce8(OUT)
     allgather4(OUT)
+    alltoallv4(OUT)
     print("wrote", sorted(os.listdir(OUT)))
 
 

@@ -2,6 +2,7 @@
 (tests/golden/plans, made by tests/golden/gen_plan_fixtures.py) and against the numpy
 restatement of flagcxC2cPlanner::execute (oracle/c2c_plan_model.py); roots in the
 second cluster; Send / Recv homo functions of all three homoTypes."""
+import importlib.util
 import os
 
 import numpy as np
@@ -15,6 +16,10 @@ from tests.util import dev_empty, from_dev, same, to_dev
 
 PLANS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "plans")
 CL8 = [0, 0, 0, 0, 1, 1, 1, 1]
+# the generator of the fixtures holds the all-to-all-v chunk matrix they were written from
+_spec = importlib.util.spec_from_file_location("gen_plan_fixtures", os.path.join(os.path.dirname(PLANS), "gen_plan_fixtures.py"))
+GEN = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(GEN)
 
 
 def fixture(name):
@@ -42,7 +47,8 @@ def test_reference_example_is_refused_for_its_negative_offsets():
     assert "negative" in str(e.value) and "test_4.xml" in str(e.value)
 
 
-@pytest.mark.parametrize("name,clusters,commop,chunks", [("allreduce8", CL8, 6, 8), ("allgather4", [0, 0, 1, 1], 7, 4)])
+@pytest.mark.parametrize("name,clusters,commop,chunks", [("allreduce8", CL8, 6, 8), ("allgather4", [0, 0, 1, 1], 7, 4),
+                                                         ("alltoallv4", [0, 0, 1, 1], 10, 8)])
 def test_dsl_layout_imports_and_exports_byte_for_byte(tmp_path, name, clusters, commop, chunks):
     """The DSL's pretty-printed layout has the indentation of exportXml
     (flagcx/core/c2c_algo.cc:1050-1087) and no <nChunks> line: exporting what was
@@ -79,6 +85,32 @@ def test_model_gives_the_allgather_closed_form():
     m.execute(send, recv, None)
     for r in range(4):
         assert np.array_equal(recv[r], np.concatenate(send)), r
+
+
+def alltoallv_case(scale, dtype, seed):
+    """Counts / displacements in elements for the fixture's chunk matrix, inputs and the
+    closed form: rank i's recv holds, at rDispls[i][r], what rank r keeps at sDispls[r][i]."""
+    send_c, sd, recv_c, rd = GEN.alltoallv_layout()
+    mul = lambda m: [[x * scale for x in row] for row in m]
+    v = tuple(mul(m) for m in (send_c, sd, recv_c, rd))
+    n = 8 * scale
+    rng = np.random.default_rng(seed)
+    hosts = [rng.integers(-2**30, 2**30, n).astype(dtype) for _ in range(4)]
+    want = [np.frombuffer(bytes([0x55]) * (n * np.dtype(dtype).itemsize), dtype=dtype).copy() for _ in range(4)]
+    for r in range(4):
+        for i in range(4):
+            c = v[0][r][i]
+            want[i][v[3][i][r]:v[3][i][r] + c] = hosts[r][v[1][r][i]:v[1][r][i] + c]
+    return n, v, hosts, want
+
+
+def test_model_gives_the_alltoallv_closed_form():
+    n, v, hosts, want = alltoallv_case(7, np.int32, 3)
+    m = M.Model(fixture("alltoallv4"), [0, 0, 1, 1], n, M.ALLTOALLV, 5, default_chunks=8)
+    recv = [np.full(n, 0x55555555, dtype=np.int32) for _ in range(4)]
+    m.execute([h.copy() for h in hosts], recv, None, v_args=v)
+    for r in range(4):
+        assert np.array_equal(recv[r], want[r]), r
 
 
 # ------------------------------------------------------------------ GPU: replay
@@ -167,6 +199,48 @@ def test_allgather4_fixture_sends_from_the_user_buffer():
     for r in range(4):
         assert same(got[r], np.concatenate(hosts)), r
         assert same(got[r], want[r]), r
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("npdt,dt", [(np.int32, O.INT32), (np.float32, O.FP32), (np.int8, O.INT8)])
+def test_alltoallv4_fixture_moves_every_piece(npdt, dt):
+    """2 clusters of 2: the pieces for the own cluster travel in the AlltoAllv homo function
+    with the caller's counts and displacements (c2c_algo.cc:482-508), the others as the
+    plan's P2P ops (c2c_algo.cc:1618-1630); ragged counts, two empty pieces."""
+    import torch
+    scale = 30001
+    n, v, hosts, want = alltoallv_case(scale, npdt, 5)
+    ts = np.dtype(npdt).itemsize
+    plan = local.Plan([0, 0, 1, 1], n, 10, local.RedOp.Sum)
+    plan.set_chunks(8)
+    plan.import_xml(fixture("alltoallv4"))
+    send = [to_dev(h) for h in hosts]
+    recv = [to_dev(np.frombuffer(bytes([0x55]) * (n * ts), dtype=npdt)) for _ in range(4)]
+    # without the arrays the homo function cannot run (c2c_algo.cc:2083-2089)
+    with pytest.raises(local.FlagcxError) as e:
+        plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, dt)
+    assert e.value.code == int(local.Result.InvalidArgument) and "AlltoAllv" in str(e.value)
+    with pytest.raises(local.FlagcxError) as e:
+        plan.set_alltoallv(v[0], None, v[2], v[3])
+    assert e.value.code == int(local.Result.InvalidArgument)
+    plan.set_alltoallv(*v)
+    plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, dt)
+    torch.cuda.synchronize()
+    m = M.Model(fixture("alltoallv4"), [0, 0, 1, 1], n, M.ALLTOALLV, 0, default_chunks=8)
+    mrecv = [np.frombuffer(bytes([0x55]) * (n * ts), dtype=npdt).copy() for _ in range(4)]
+    m.execute([h.copy() for h in hosts], mrecv, None, v_args=v)
+    for r in range(4):
+        got = from_dev(recv[r], npdt)
+        assert same(got, want[r]), r
+        assert same(got, mrecv[r]), r
+        assert same(from_dev(send[r], npdt), hosts[r]), r
+    # a receive count that no send matches is an error, not a hang
+    bad = [[list(row) for row in m_] for m_ in v]
+    bad[2][1][0] += 1
+    plan.set_alltoallv(*bad)
+    with pytest.raises(local.FlagcxError) as e:
+        plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, dt)
+    assert e.value.code == int(local.Result.InvalidUsage)
 
 
 def broadcast_two_clusters(prefix, root):
