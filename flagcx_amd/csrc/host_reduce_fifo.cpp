@@ -29,10 +29,11 @@ using namespace flagcx_amd;
 struct flagcxLocalReduceFifo {
   uint64_t *header = nullptr;       // pinned: kQueueHeaderWords words, then the entry ring
   QueueEntry *hostEntries = nullptr;
-  void *devBlock = nullptr;         // device ring | devProduced | progress words
+  void *devBlock = nullptr;         // device ring | devProduced | progress words | ticket counters
   QueueEntry *devEntries = nullptr;
   uint64_t *devProduced = nullptr;
   uint32_t *progress = nullptr;
+  uint64_t *tickets = nullptr;
   uint32_t capacity = 0;
   unsigned maxGrid = 0;
   unsigned grid = 0;
@@ -80,7 +81,8 @@ inline bool overlaps(uintptr_t x, uintptr_t y, uint64_t xbytes, uint64_t ybytes)
 // finished).  The caller holds the mutex.
 flagcxResult_t launchConsumer(flagcxLocalReduceFifo *q, uint64_t base, const char *who) {
   __atomic_store_n(q->header + kQueueState, (uint64_t)kQueueRunning, __ATOMIC_RELEASE);
-  const size_t clearBytes = 128 + (size_t)q->maxGrid * sizeof(uint64_t);
+  const size_t clearBytes = 128 + (size_t)q->maxGrid * sizeof(uint64_t) +
+                            (size_t)kQueueMaxTicketCounters * kQueueTicketStride * sizeof(uint64_t);
   hipError_t e = hipMemsetAsync(q->devProduced, 0, clearBytes, q->stream);
   if (e != hipSuccess) return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString(e));
   QueueKernelArgs a;
@@ -94,6 +96,8 @@ flagcxResult_t launchConsumer(flagcxLocalReduceFifo *q, uint64_t base, const cha
   a.base = base;
   a.linger = q->linger;
   a.windowBytes = q->windowBytes;
+  a.tickets = q->tickets;
+  a.counters = 1; // the launcher sets it from the grid
   // LDS is reserved only to spread the resident wavefronts over the CUs (at most
   // `waves` + 2 fit on one), in whole 1280-byte allocation granules.  A fifth of
   // every CU's LDS stays free, so that other launches that need LDS (this library's
@@ -222,19 +226,21 @@ flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int ca
   q->dtype = dt;
   q->op = rop;
   q->typeSize = ts;
-  // Measured on MI355X (32 x 4 MiB chunks per input): with the workers' units of
-  // 8 / 4 / 1 KiB per input for up to 2 / up to 4 / more inputs, about 64-80 KiB of
-  // loads in flight per CU are enough (two inputs 5.5 / 5.6 / 6.0 TB/s at 16 / 12 / 8
-  // wavefronts per CU, four 5.7 / 6.0 at 14 / 10, eight 6.0 / 6.0 / 5.8 at 8 / 10 / 14);
-  // never more than half a CU's slots, so that residency does not depend on the last
-  // slot being free.  (A limit on the inputs a worker has in flight, which the
-  // launched kernels use for large reduces, only costs here.)
-  static const int kWaves[9] = {8, 8, 8, 10, 10, 10, 10, 10, 10};
+  // Measured on MI355X (128 x 4 MiB chunks per input, units drawn by ticket): with the
+  // workers' units of 8 / 4 / 1 KiB per input for up to 2 / up to 4 / more inputs, about
+  // 64-100 KiB of loads in flight per CU are enough (two inputs 6.05 / 6.0 / 5.8 / 5.6 TB/s at
+  // 8 / 10 / 12 / 14 wavefronts per CU, three 5.9 / 6.05 / 6.0 / 5.7, four 6.35 / 6.0 / 5.8 / 5.6,
+  // six 4.7 / 5.4 / 5.8 / 6.0, eight 5.5 / 5.9 / 6.1 / 6.1); never more than half a CU's
+  // slots, so that residency does not depend on the last slot being free.  (A limit on
+  // the inputs a worker has in flight, which the launched kernels use for large
+  // reduces, only costs here.)
+  static const int kWaves[9] = {8, 8, 8, 10, 8, 14, 14, 12, 12};
   q->wavesPerCU = kWaves[maxRanks];
   const DeviceInfo &info = deviceInfo();
   q->maxGrid = (unsigned)info.numCU * 16u;
   const size_t hostBytes = kQueueHeaderWords * sizeof(uint64_t) + (size_t)capacity * sizeof(QueueEntry);
-  const size_t devBytes = (size_t)capacity * sizeof(QueueEntry) + 128 + (size_t)q->maxGrid * sizeof(uint64_t);
+  const size_t devBytes = (size_t)capacity * sizeof(QueueEntry) + 128 + (size_t)q->maxGrid * sizeof(uint64_t) +
+                          (size_t)kQueueMaxTicketCounters * kQueueTicketStride * sizeof(uint64_t);
   void *host = nullptr;
   hipError_t e = hipHostMalloc(&host, hostBytes, hipHostMallocMapped);
   if (e == hipSuccess) e = hipMalloc(&q->devBlock, devBytes);
@@ -252,6 +258,7 @@ flagcxResult_t flagcxLocalReduceFifoCreate(flagcxLocalReduceFifo_t *fifo, int ca
   q->devEntries = static_cast<QueueEntry *>(q->devBlock);
   q->devProduced = reinterpret_cast<uint64_t *>(q->devEntries + capacity);
   q->progress = reinterpret_cast<uint32_t *>(q->devProduced + 16);
+  q->tickets = q->devProduced + 16 + q->maxGrid;
   *fifo = q;
   return flagcxSuccess;
 }

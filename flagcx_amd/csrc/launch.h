@@ -78,6 +78,10 @@ enum : uint64_t { kQueueIdle = 0, kQueueRunning = 1, kQueueStopped = 2, kQueueTi
 // side wins when an entry arrives while the consumer is leaving.
 constexpr uint64_t kQueueParkedBit = 1ull << 63;
 
+// Ticket counters of the reduce queue's workers: at most this many, each in a KiB of its own.
+constexpr int kQueueMaxTicketCounters = 64;
+constexpr int kQueueTicketStride = 128; // 64-bit words
+
 struct QueueKernelArgs {
   uint64_t *hostHeader;          // pinned, device-visible
   const QueueEntry *hostEntries; // pinned ring, `capacity` entries
@@ -89,6 +93,8 @@ struct QueueKernelArgs {
   uint64_t base;                 // entries finished before this launch; device counts are relative to it
   int64_t linger;                // idle polls before the consumer parks; 0 = stay until stopped
   uint64_t windowBytes;          // traffic of the entries the workers may have in work together
+  uint64_t *tickets;             // ticket counters, kQueueTicketStride words apart, zero at launch
+  uint32_t counters;             // how many of them this launch uses (every one has workers)
 };
 
 // Launches the consumer for one element type: grid = min(occupancy, wavesPerCU) *

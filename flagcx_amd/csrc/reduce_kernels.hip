@@ -286,7 +286,12 @@ static int launchQueueOp(const QueueKernelArgs &q, int wavesPerCU, int numCU, in
   if (g > maxGrid) g = maxGrid;
   if (g < 2) return (int)hipErrorLaunchOutOfResources;
   *grid = (unsigned)g;
-  reduceQueueKernel<elem_t, OP><<<dim3((unsigned)g), dim3(64), lds, stream>>>(q);
+  // workgroups 8n..8n+7 (one per XCD) share ticket counter n modulo the number of
+  // counters; every counter in use has workers
+  QueueKernelArgs a = q;
+  const uint64_t groups = (g - 1) / 8 + 1;
+  a.counters = (uint32_t)(groups < (uint64_t)kQueueMaxTicketCounters ? groups : (uint64_t)kQueueMaxTicketCounters);
+  reduceQueueKernel<elem_t, OP><<<dim3((unsigned)g), dim3(64), lds, stream>>>(a);
   return (int)hipGetLastError();
 }
 

@@ -10,10 +10,10 @@
 //            device ring, publishes the count the workers poll (device memory, so
 //            only one wavefront reads over PCIe), folds the workers' progress
 //            words into `consumed` in the host header.
-//   worker : for each forwarded entry takes the KiB tiles whose running global
-//            index is congruent to its number modulo W (the numbering runs on
-//            across entries, so entries of a few thousand tiles still spread
-//            evenly), in the same per-tile shape as the launch-per-call kernels.
+//   worker : draws tickets for units of one or a few KiB tiles in a numbering that
+//            runs on across entries (so entries of a few thousand tiles still spread
+//            evenly, and whoever is free takes the next unit), and folds each in the
+//            same per-tile shape as the launch-per-call kernels.
 //
 // Coherence is per access, not per cache: a kernel that never ends gets no
 // launch-boundary invalidate or write-back, and cache-wide maintenance from
@@ -67,6 +67,13 @@ __device__ __forceinline__ void systemStore(uint64_t *p, uint64_t v) {
 __device__ __forceinline__ void waitOwnMemory() {
   __atomic_signal_fence(__ATOMIC_SEQ_CST);
   __builtin_amdgcn_s_waitcnt(0);
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
+// As above, except that the youngest operation may still be outstanding.
+__device__ __forceinline__ void waitAllButYoungest() {
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __builtin_amdgcn_s_waitcnt(0x0001); // vmcnt(1), expcnt(0), lgkmcnt(0)
   __atomic_signal_fence(__ATOMIC_SEQ_CST);
 }
 
@@ -347,82 +354,128 @@ __device__ __forceinline__ void queueEntry(const uint64_t (&src)[8], uint64_t ds
   }
 }
 
+// Units are numbered through, entry after entry, from the first entry of this launch
+// on, and handed out by ticket: counter c of q.counters hands out the units congruent
+// to c, in ascending order, to the workers that share it (a worker's counter follows
+// from its workgroup number; every counter has workers from all XCDs).  Whoever is
+// free takes the next unit, as the hardware dispatcher does for a launched grid, so
+// a slow CU or XCD holds nobody else back (units dealt out by congruence to the worker
+// number ran 10 % slower: every entry waited for its slowest worker).  The next
+// ticket is fetched while the current unit is in flight; tickets drawn beyond the
+// published entries are simply held until those entries arrive.  Counters are 1 KiB
+// apart, in different memory channels.
 template <typename T, int OP>
 __device__ inline void queueWorker(const QueueKernelArgs &q) {
-  const uint32_t nworkers = gridDim.x - 1;
   const uint32_t worker = blockIdx.x - 1;
-  uint64_t done = 0; // entries this worker has finished since this launch (entry index = q.base + done)
+  const uint32_t nc = q.counters;
+  const uint32_t c = (blockIdx.x / 8) % nc;
+  uint64_t *const mine = q.tickets + (size_t)c * kQueueTicketStride;
+  uint64_t done = 0;     // entries this worker has passed since this launch (entry index = q.base + done)
+  uint64_t unitBase = 0; // number of the first unit of entry `done`
+  uint64_t produced = 0; // entries known to be in the device ring
+  uint64_t reported = 0; // what the progress word says
   uint64_t lastBeat = 0;
-  uint32_t rot = 0;  // units handed out so far, modulo nworkers
-  for (;;) {
-    uint64_t produced;
-    int64_t spins = 0;
-    for (;;) {
-      produced = uniform64(agentLoad(q.devProduced));
-      if (produced > done) break; // the abort value ~0 ends the wait too
-      // an idle queue is the leader's to time out; a worker only gives up by
-      // itself when the leader's heartbeat has stopped for maxSpin polls
-      const uint64_t beat = uniform64(agentLoad(q.devProduced + 1));
-      if (beat != lastBeat) {
-        lastBeat = beat;
-        spins = 0;
-      }
-      if (++spins > q.maxSpin) return;
-      __builtin_amdgcn_s_sleep(4);
-    }
-    if (produced == ~0ull) return;
-    bool stop = false;
-    // lane l holds word l & 15 of the entry; the next entry is fetched while this
-    // one's tiles are in flight
-    uint64_t words =
-        agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (q.base + done) % q.capacity) + (threadIdx.x & 15));
-    while (done < produced) {
-      const uint64_t cur = words;
-      if (done + 1 < produced)
-        words = agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (q.base + done + 1) % q.capacity) +
-                          (threadIdx.x & 15));
-      const uint64_t kv = laneWord(cur, 11);
-      const int k = (int)(uint32_t)kv;
-      done++;
-      if (k == 0) {
-        stop = true;
-        break;
-      }
-      const bool vector = ((kv >> 32) & kQueueFlagAligned) != 0;
-      uint64_t src[8];
-#pragma unroll
-      for (int b = 0; b < 8; b++) src[b] = laneWord(cur, b);
-      const uint64_t dst = laneWord(cur, 8);
-      const uint64_t nvec = laneWord(cur, 9);
-      const uint64_t ht = laneWord(cur, 10);
-      const uint32_t head = (uint32_t)ht, tail = (uint32_t)(ht >> 32);
-      const uint64_t unitBytes = 1024ull * (uint32_t)queueUnitTiles(k);
-      const uint64_t nunits = (nvec * 16 + unitBytes - 1) / unitBytes;
-      const uint32_t first = worker >= rot ? worker - rot : worker + nworkers - rot;
-      switch (k) {
-        case 1: queueEntry<T, OP, 1>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-        case 2: queueEntry<T, OP, 2>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-        case 3: queueEntry<T, OP, 3>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-        case 4: queueEntry<T, OP, 4>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-        case 5: queueEntry<T, OP, 5>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-        case 6: queueEntry<T, OP, 6>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-        case 7: queueEntry<T, OP, 7>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-        default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nworkers); break;
-      }
-      rot = (uint32_t)((rot + nunits) % nworkers);
-      // in a long run of entries let the count move every fourth entry, so that the
-      // leader's window and the producer's ring move while the run is still going
-      if ((done & 3) == 0 && done < produced) {
-        waitOwnMemory();
-        if (threadIdx.x == 0)
-          __hip_atomic_store(q.progress + worker, (uint32_t)done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    // this wavefront's results are acknowledged by memory before the count says so
-    waitOwnMemory();
+  // one ticket in hand and the next on its way: the draw is issued behind a unit's
+  // store, so that no load waits for it (memory operations of a wavefront return in
+  // the order issued), and is read a whole unit later
+  uint64_t ticket = 0, pending = 0;
+  if (threadIdx.x == 0) {
+    ticket = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    pending = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  ticket = uniform64(ticket);
+  // lane l holds word l & 15 of entry `done` (haveCur) and of entry `done + 1` (haveNext)
+  uint64_t cur = 0, next = 0;
+  bool haveCur = false, haveNext = false;
+  auto report = [&]() {
+    // this wavefront's results are acknowledged by memory before the count says so;
+    // the one operation that may still be on its way is the youngest, the ticket draw
+    // issued behind the last store
+    waitAllButYoungest();
     if (threadIdx.x == 0)
       __hip_atomic_store(q.progress + worker, (uint32_t)done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (stop) return;
+    reported = done;
+  };
+  for (;;) {
+    const uint64_t unit = ticket * nc + c;
+    // the entry that holds this unit
+    int k;
+    uint64_t nunits;
+    for (;;) {
+      if (done >= produced) {
+        if (reported != done) report();
+        int64_t spins = 0;
+        for (;;) {
+          produced = uniform64(agentLoad(q.devProduced));
+          if (produced > done) break; // the abort value ~0 ends the wait too
+          // an idle queue is the leader's to time out; a worker only gives up by
+          // itself when the leader's heartbeat has stopped for maxSpin polls
+          const uint64_t beat = uniform64(agentLoad(q.devProduced + 1));
+          if (beat != lastBeat) {
+            lastBeat = beat;
+            spins = 0;
+          }
+          if (++spins > q.maxSpin) return;
+          __builtin_amdgcn_s_sleep(4);
+        }
+        if (produced == ~0ull) return;
+      }
+      if (!haveCur) {
+        cur = agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (q.base + done) % q.capacity) +
+                        (threadIdx.x & 15));
+        haveCur = true;
+      }
+      const uint64_t kv = laneWord(cur, 11);
+      k = (int)(uint32_t)kv;
+      if (k == 0) { // the stop entry: everything before it has been handed out
+        done++;
+        waitOwnMemory();
+        report();
+        return;
+      }
+      const uint64_t unitBytes = 1024ull * (uint32_t)queueUnitTiles(k);
+      nunits = (laneWord(cur, 9) * 16 + unitBytes - 1) / unitBytes;
+      if (nunits == 0) nunits = 1; // head and tail elements only: still somebody's unit
+      if (unit < unitBase + nunits) break;
+      unitBase += nunits;
+      done++;
+      cur = next;
+      haveCur = haveNext;
+      haveNext = false;
+    }
+    // in flight while this unit is folded: the next entry
+    if (!haveNext && done + 1 < produced) {
+      next = agentLoad(reinterpret_cast<const uint64_t *>(q.devEntries + (q.base + done + 1) % q.capacity) +
+                       (threadIdx.x & 15));
+      haveNext = true;
+    }
+    const uint64_t kv = laneWord(cur, 11);
+    const bool vector = ((kv >> 32) & kQueueFlagAligned) != 0;
+    uint64_t src[8];
+#pragma unroll
+    for (int b = 0; b < 8; b++) src[b] = laneWord(cur, b);
+    const uint64_t dst = laneWord(cur, 8);
+    const uint64_t nvec = laneWord(cur, 9);
+    const uint64_t ht = laneWord(cur, 10);
+    const uint32_t head = (uint32_t)ht, tail = (uint32_t)(ht >> 32);
+    const uint64_t first = unit - unitBase;
+    switch (k) {
+      case 1: queueEntry<T, OP, 1>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      case 2: queueEntry<T, OP, 2>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      case 3: queueEntry<T, OP, 3>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      case 4: queueEntry<T, OP, 4>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      case 5: queueEntry<T, OP, 5>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      case 6: queueEntry<T, OP, 6>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      case 7: queueEntry<T, OP, 7>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nunits); break;
+    }
+    // in a long run of entries let the count move every few entries, so that the
+    // leader's window and the producer's ring move while the run is still going
+    ticket = uniform64(pending);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    if (threadIdx.x == 0) pending = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    if (done >= reported + 4) report();
   }
 }
 

@@ -159,8 +159,8 @@ def test_ring_fifo_returns_when_the_consumer_has_left(L):
     rc, want = O.reduce_scatter_rank(send_h, 1, rcount, dt, op)
     torch.cuda.synchronize()
     q = L.ReduceFifo(8, nranks, dt, op)
-    q.set_linger(0)
     try:
+        # the spin bound is reached long before the idle limit at which a consumer parks
         L.lib().flagcxLocalSetMaxSpinCount(1)
         q.start()
         try:
