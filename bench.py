@@ -474,15 +474,15 @@ def config_c5(L):
 def table_sweep(L, args):
     import torch
     g = torch.Generator(device="cuda").manual_seed(0)
-    print("%12s %10s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %8s" %
+    print("%12s %10s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %9s %9s | %8s %8s %6s" %
           ("bytes", "sets", "reduce2us", "GB/s", "pack us", "GB/s", "unpack us", "GB/s", "memcpy us", "GB/s",
-           "memset us", "GB/s", "b2b us"))
+           "memset us", "GB/s", "b2b us", "b2b GB/s", "% peak"))
     size = args.min
     while size <= args.max:
         nsets, out, b2b = sweep_point(L, size, args.table == "sweep-rotate", g)
         print("%12d %10d | " % (size, nsets) +
               " | ".join("%9.2f %9.1f" % out[k][:2] for k in ("reduce2", "pack", "unpack", "memcpy", "memset")) +
-              " | %8.2f" % b2b, flush=True)
+              " | %8.2f %8.1f %6.1f" % (b2b, 3 * size / b2b / 1e3, 3 * size / b2b / 1e3 / HBM_PEAK_GBPS * 100), flush=True)
         size *= 2
 
 

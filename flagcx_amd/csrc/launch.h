@@ -36,6 +36,7 @@ struct LaunchShape {
 LaunchShape launchShapeFor(int k, uint64_t tiles);
 void setWavesPerCU(int k, int waves);
 int tunedWavesPerCU(int k); // the explicit setting, or -1
+int tunedLoadsInFlight(int k); // the explicit setting (0 = all at once), or -1
 
 // LDS bytes to reserve per workgroup so that at most `waves` one-wave workgroups
 // fit on a CU.  0 when no cap is wanted.

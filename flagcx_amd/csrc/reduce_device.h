@@ -382,14 +382,22 @@ __global__ void __launch_bounds__(64) reduceWaveUnalignedKernel(ReduceParams<FLA
 // bytes [16 v + d_j, 16 v + d_j + 16) counted from the source's aligned base, i.e.
 // the top of aligned granule v and the bottom of granule v + 1, where d_j = the
 // source's offset inside a 16-byte line minus the destination's.  Lane i loads
-// granule 64 t + i of every source, takes granule 64 t + i + 1 from lane i + 1, and
-// lane 63 takes it from lane 0 of the NEXT tile, which the same wavefront has
-// already asked for: a wavefront walks R consecutive tiles, one tile ahead with its
-// loads, so every granule is fetched once (plus one granule per R tiles), where
-// unaligned 16-byte loads touch a ninth cache line per KiB, and in another XCD's L2
-// than the wavefront that fetches the rest of that line.
+// granule 64 t + i of every source and takes granule 64 t + i + 1 from lane i + 1;
+// lane 63 needs the first granule of the NEXT tile, which one more load with a
+// one-granule descriptor brings (only lane 0 of it is in range).
+// That granule sits in a cache line which the wavefront of the next tile fetches as
+// well.  Workgroup b runs on XCD b mod 8, each XCD with an L2 of its own, so with
+// tile = workgroup number the line would come from memory twice (128 bytes more per
+// KiB and source: 71-78 % of peak where the aligned kernel reaches 83-85 %).  Tiles
+// are therefore dealt out in runs of kShiftRun consecutive tiles per XCD: the
+// wavefronts of a run start within a few hundred nanoseconds of each other on one
+// XCD, and seven of eight look-ahead granules are L2 hits (runs of 4 measured 2-3
+// points lower, runs of 12 and 16 the same or lower; a second full load one granule
+// further on instead of the lane shift doubles the L2 traffic: 61 %).
 // Descriptors are clipped to the granules that hold source bytes, so nothing
 // outside a source's own 16-byte lines is ever read.
+constexpr int kShiftRun = 8;
+
 template <int K>
 struct ShiftParams {
   const void *base[K]; // source address rounded down to 16, at the first body element
@@ -398,7 +406,7 @@ struct ShiftParams {
   const void *src[K];  // original pointers (head and tail elements)
   void *dst;
   uint64_t nvec, head, tail;
-  int32_t tilesPerWave;
+  int32_t inflight; // 2: ask for the next source only when at most one earlier source is outstanding
 };
 
 // bytes [4 Q + b, 4 Q + b + 16) of the 32 bytes (lo, hi).  Q is a template argument
@@ -432,55 +440,50 @@ __global__ void __launch_bounds__(64) reduceWaveShiftKernel(ShiftParams<K> p) {
   constexpr int N = 16 / sizeof(T);
   const uint32_t lane = threadIdx.x;
   const uint64_t ntiles = (p.nvec + 63) / 64;
-  const uint64_t R = (uint64_t)p.tilesPerWave;
   const uint64_t headBytes = p.head * sizeof(T);
-  for (uint64_t t0 = (uint64_t)blockIdx.x * R; t0 < ntiles; t0 += (uint64_t)gridDim.x * R) {
-    const uint64_t tEnd = t0 + R < ntiles ? t0 + R : ntiles;
-    // Granules of a tile: a descriptor from granule 64 t on, clipped to the source's own
-    // granules and to `want` of them: 64 for a tile of this walk, 1 for the tile after
-    // the walk (only its first granule is needed, by lane 63 of the last tile), 0 beyond.
-    auto loadTile = [&](u32x4 (&out)[K], uint64_t t) {
-      const uint64_t want = t < tEnd ? 64 : t == tEnd ? 1 : 0;
+  // runs of kShiftRun consecutive tiles on one XCD; the grid is a whole number of
+  // rounds of 8 runs (a grid smaller than the tiles takes several passes), tiles beyond
+  // the last do nothing
+  constexpr uint64_t kRound = 8ull * kShiftRun;
+  const uint64_t padded = (ntiles + kRound - 1) / kRound * kRound;
+  for (uint64_t b = blockIdx.x; b < padded; b += gridDim.x) {
+    const uint64_t bi = b / 8, bx = b % 8;
+    const uint64_t t = ((bi / kShiftRun) * 8 + bx) * kShiftRun + bi % kShiftRun;
+    if (t >= ntiles) continue;
+    u32x4 cur[K], ahead[K];
 #pragma unroll
-      for (int j = 0; j < K; j++) {
-        const uint64_t g0 = t * 64;
-        const uint64_t left = p.granules[j] > g0 ? p.granules[j] - g0 : 0;
-        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)((const char *)p.base[j] + g0 * 16), 0, (uint32_t)(left < want ? left : want) * 16u, kRsrcFlags);
-        out[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16u, 0, kLoadAux);
-      }
-    };
-    u32x4 cur[K], nxt[K];
-    loadTile(cur, t0);
-    loadTile(nxt, t0 + 1);
-    for (uint64_t t = t0; t < tEnd; t++) {
-      u32x4 in[K];
-#pragma unroll
-      for (int j = 0; j < K; j++) {
-        u32x4 hi;
-#pragma unroll
-        for (int d = 0; d < 4; d++) {
-          const uint32_t fromNext = __builtin_amdgcn_readfirstlane(nxt[j][d]); // lane 0 of the next tile
-          // wave_shl:1 - lane i reads lane i + 1; lane 63 has no source lane and keeps `old`
-          hi[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)fromNext, (int)cur[j][d], 0x130, 0xf, 0xf, false);
-        }
-        in[j] = funnel16(cur[j], hi, p.shift[j] >> 2, p.shift[j] & 3u);
-      }
-      // the tile after next is asked for before this one is folded: its loads are in
-      // flight during the arithmetic (the registers of `cur` are free from here on)
-      loadTile(cur, t + 2);
-      const uint64_t off = t * 1024;
-      const uint64_t left = p.nvec * 16 - off;
-      __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
-          (void *)((char *)p.dst + headBytes + off), 0, left < 1024 ? (uint32_t)left : 1024u, kRsrcFlags);
-      __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, lane * 16u, 0, kStoreAux);
-#pragma unroll
-      for (int j = 0; j < K; j++) {
-        const u32x4 tmp = nxt[j];
-        nxt[j] = cur[j];
-        cur[j] = tmp;
+    for (int j = 0; j < K; j++) {
+      const uint64_t g0 = t * 64;
+      const uint64_t left = p.granules[j] > g0 ? p.granules[j] - g0 : 0;
+      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+          (void *)((const char *)p.base[j] + g0 * 16), 0, (uint32_t)(left < 64 ? left : 64) * 16u, kRsrcFlags);
+      cur[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16u, 0, kLoadAux);
+      __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+          (void *)((const char *)p.base[j] + g0 * 16 + 1024), 0, left > 64 ? 16u : 0u, kRsrcFlags);
+      ahead[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, lane * 16u, 0, kLoadAux);
+      if (p.inflight == 2 && j >= 1 && j < K - 1) {
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | 2); // vmcnt(2): this source's two loads only
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
       }
     }
+    u32x4 in[K];
+#pragma unroll
+    for (int j = 0; j < K; j++) {
+      u32x4 hi;
+#pragma unroll
+      for (int d = 0; d < 4; d++) {
+        const uint32_t fromNext = __builtin_amdgcn_readfirstlane(ahead[j][d]); // granule 0 of the next tile
+        // wave_shl:1 - lane i reads lane i + 1; lane 63 has no source lane and keeps `old`
+        hi[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)fromNext, (int)cur[j][d], 0x130, 0xf, 0xf, false);
+      }
+      in[j] = funnel16(cur[j], hi, p.shift[j] >> 2, p.shift[j] & 3u);
+    }
+    const uint64_t off = t * 1024;
+    const uint64_t left = p.nvec * 16 - off;
+    __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((char *)p.dst + headBytes + off), 0, left < 1024 ? (uint32_t)left : 1024u, kRsrcFlags);
+    __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, lane * 16u, 0, kStoreAux);
   }
   // head and tail elements (fewer than 2*N <= 32): last workgroup, one lane each
   if (blockIdx.x == gridDim.x - 1) {

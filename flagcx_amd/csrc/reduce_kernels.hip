@@ -124,7 +124,7 @@ static int launchAny(const ReduceCall &c, const Split &s) {
 }
 
 // Sources at another offset modulo 16 than the output, up to eight of them: aligned
-// loads put in place with lane shifts, a wavefront walking consecutive tiles.
+// loads put in place with lane shifts.
 template <int OP, int K>
 static int launchShift(const ReduceCall &c, const Split &s) {
   ShiftParams<K> p;
@@ -141,19 +141,22 @@ static int launchShift(const ReduceCall &c, const Split &s) {
   p.head = s.head;
   p.tail = s.tail;
   const uint64_t tiles = (s.nvec + 63) / 64;
-  // Two tiles per wavefront: the look-ahead granule costs one extra 16-byte load per
-  // two KiB of every source, and the wavefront is short-lived enough for the
-  // dispatcher to keep the tiles in work dense (4 and 8 tiles measured 2-6 points of
-  // peak lower for 256 MiB inputs).  Wavefronts per CU measured best at 25 / 21 / 16
-  // for up to 3 / 4 / more inputs (bf16, 64 and 256 MiB per input: 73-78, 75-77 and
-  // 70-74 % of peak, against 68-72 % with unaligned 16-byte loads).
-  constexpr int walk = 2;
-  p.tilesPerWave = walk;
-  uint64_t grid = (tiles + (uint64_t)walk - 1) / (uint64_t)walk;
-  if (grid < 1) grid = 1;
-  if (grid > kMaxGrid) grid = kMaxGrid;
+  // One tile per wavefront, dealt out in runs of kShiftRun tiles per XCD (whole rounds of
+  // 8 runs).  Measured on MI355X, bf16 over rotating buffers, percent of peak at 32 /
+  // 128 / 512 MiB per input: 1 input (a misaligned copy) 66 / 77 / 81, 2: 71 / 80 / 83,
+  // 3: 70-75 / 80-82 / 83-84, 4: 74-76 / 81 / 84, 6: 75 / 80-82 / 81, 8: 74-76 / 79 / 77-78
+  // (tile = workgroup number, two tiles per wavefront: 62-65 / 73-76 / 69-80).
+  // Wavefronts per CU: no cap / 25 / 21 / 14 for up to 2 / 3 / 4 / up to 6 inputs; 7 and 8
+  // keep two sources in flight per wavefront at 16, which holds 77-79 % from 128 MiB to
+  // 1 GiB where all at once falls to 70-73 %.
+  constexpr uint64_t span = 8ull * kShiftRun;
+  uint64_t grid = (tiles + span - 1) / span * span;
+  if (grid < span) grid = span;
+  if (grid > kMaxGrid) grid = kMaxGrid; // a multiple of the round: the kernel takes several passes
+  const int loads = tunedLoadsInFlight(K);
+  p.inflight = loads >= 0 ? (loads == 2 ? 2 : 0) : K >= 7 ? 2 : 0;
   const int tuned = tunedWavesPerCU(K);
-  const int lds = ldsReservation(tuned >= 0 ? tuned : K <= 3 ? 25 : K == 4 ? 21 : 16);
+  const int lds = ldsReservation(tuned >= 0 ? tuned : K <= 2 ? 0 : K == 3 ? 25 : K == 4 ? 21 : K <= 6 ? 14 : 16);
   reduceWaveShiftKernel<elem_t, OP, K><<<dim3((unsigned)grid), dim3(64), lds, c.stream>>>(p);
   return (int)hipGetLastError();
 }
