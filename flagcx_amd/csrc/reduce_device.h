@@ -43,6 +43,9 @@ struct ReduceParams {
   uint64_t tail;   // elements after the body
   int32_t k;       // number of inputs actually used (== K except generic)
   int32_t inflight; // 1..3 (< K): a wavefront keeps the loads of at most that many inputs in flight; 0: of all K
+  // (32-bit fields: narrower kernel arguments are fetched with vector loads at the start of every wavefront)
+  uint32_t lead;   // bytes by which the first tile is shortened, so that every later tile starts on a 128-byte line of dst
+  uint32_t run;    // consecutive tiles that stay on one XCD (1: tile = workgroup number)
 };
 
 // ------------------------------------------------------------------ widen
@@ -188,19 +191,38 @@ constexpr int kRsrcFlags = 0x00020000;
 // out-of-range lanes load zeros and their stores are dropped by the hardware.
 // dst may be one of the inputs: a lane reads its positions before it writes
 // them, and no other lane touches them.
-template <typename T, int OP, int K, int U>
+// TILED: the first tile may be short and tiles may be dealt out in runs per XCD (p.lead,
+// p.run); without it tile = workgroup number from the first body byte on, which is what
+// line-aligned buffers take (the extra scalar work at the start of every short-lived
+// wavefront costs a percent of bandwidth).
+template <typename T, int OP, int K, int U, bool TILED>
 __device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
   constexpr int N = 16 / sizeof(T);
   constexpr uint32_t kTileBytes = 64u * U * 16u;
   const uint64_t bodyBytes = p.nvec * 16;
-  const uint64_t ntiles = (bodyBytes + kTileBytes - 1) / kTileBytes;
+  const uint32_t lead = TILED ? p.lead : 0;
+  const uint64_t ntiles = (bodyBytes + lead + kTileBytes - 1) / kTileBytes;
   const uint64_t headBytes = p.head * sizeof(T);
   const uint32_t voff = threadIdx.x * 16u;
+  // Workgroup b runs on XCD b mod 8, every XCD with an L2 of its own.  Where tiles do
+  // not start on a cache line of every buffer, neighbouring tiles share lines: runs of
+  // p.run consecutive tiles then stay on one XCD, so that a shared line is fetched into,
+  // and written back from, one L2.  The grid is a whole number of rounds of 8 runs.
+  const uint64_t run = TILED ? p.run : 1;
+  const uint64_t round = 8 * run;
+  const uint64_t padded = run > 1 ? (ntiles + round - 1) / round * round : ntiles;
 
-  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const uint64_t off = t * kTileBytes;
+  for (uint64_t b = blockIdx.x; b < padded; b += gridDim.x) {
+    uint64_t t = b;
+    if (TILED && run > 1) {
+      const uint64_t bi = b / 8, bx = b % 8;
+      t = ((bi / run) * 8 + bx) * run + bi % run;
+      if (t >= ntiles) continue;
+    }
+    const uint64_t off = TILED ? (t ? t * kTileBytes - lead : 0) : t * kTileBytes;
     const uint64_t left = bodyBytes - off;
-    const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
+    const uint32_t cap = TILED ? (t ? kTileBytes : kTileBytes - lead) : kTileBytes;
+    const uint32_t span = left < cap ? (uint32_t)left : cap;
     u32x4 in[U][K];
 #pragma unroll
     for (int j = 0; j < K; j++) {
@@ -240,9 +262,9 @@ __device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
   }
 }
 
-template <typename T, int OP, int K, int U>
+template <typename T, int OP, int K, int U, bool TILED>
 __global__ void __launch_bounds__(64) reduceWaveKernel(ReduceParams<K> p) {
-  reduceWaveBody<T, OP, K, U>(p);
+  reduceWaveBody<T, OP, K, U, TILED>(p);
 }
 
 // Several independent reductions of the same type, op and K in one launch:
@@ -255,9 +277,9 @@ struct ReduceBatchParams {
   ReduceParams<K> seg[FLAGCX_BATCH_MAX];
 };
 
-template <typename T, int OP, int K, int U>
+template <typename T, int OP, int K, int U, bool TILED>
 __global__ void __launch_bounds__(64) reduceBatchKernel(ReduceBatchParams<K> bp) {
-  reduceWaveBody<T, OP, K, U>(bp.seg[blockIdx.y]);
+  reduceWaveBody<T, OP, K, U, TILED>(bp.seg[blockIdx.y]);
 }
 
 // Aligned body, any k up to FLAGCX_MAX_RANKS, same streaming shape as above: one
@@ -407,6 +429,7 @@ struct ShiftParams {
   void *dst;
   uint64_t nvec, head, tail;
   int32_t inflight; // 2: ask for the next source only when at most one earlier source is outstanding
+  uint32_t lead;    // bytes by which the first tile is shortened: later tiles start on a 128-byte line of dst
 };
 
 // bytes [4 Q + b, 4 Q + b + 16) of the 32 bytes (lo, hi).  Q is a template argument
@@ -439,7 +462,7 @@ template <typename T, int OP, int K>
 __global__ void __launch_bounds__(64) reduceWaveShiftKernel(ShiftParams<K> p) {
   constexpr int N = 16 / sizeof(T);
   const uint32_t lane = threadIdx.x;
-  const uint64_t ntiles = (p.nvec + 63) / 64;
+  const uint64_t ntiles = (p.nvec * 16 + p.lead + 1023) / 1024;
   const uint64_t headBytes = p.head * sizeof(T);
   // runs of kShiftRun consecutive tiles on one XCD; the grid is a whole number of
   // rounds of 8 runs (a grid smaller than the tiles takes several passes), tiles beyond
@@ -450,10 +473,12 @@ __global__ void __launch_bounds__(64) reduceWaveShiftKernel(ShiftParams<K> p) {
     const uint64_t bi = b / 8, bx = b % 8;
     const uint64_t t = ((bi / kShiftRun) * 8 + bx) * kShiftRun + bi % kShiftRun;
     if (t >= ntiles) continue;
+    // the first tile is short, so that the others start on a line of the destination
+    const uint64_t off = t ? t * 1024 - p.lead : 0;
+    const uint64_t g0 = off / 16;
     u32x4 cur[K], ahead[K];
 #pragma unroll
     for (int j = 0; j < K; j++) {
-      const uint64_t g0 = t * 64;
       const uint64_t left = p.granules[j] > g0 ? p.granules[j] - g0 : 0;
       __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
           (void *)((const char *)p.base[j] + g0 * 16), 0, (uint32_t)(left < 64 ? left : 64) * 16u, kRsrcFlags);
@@ -479,10 +504,10 @@ __global__ void __launch_bounds__(64) reduceWaveShiftKernel(ShiftParams<K> p) {
       }
       in[j] = funnel16(cur[j], hi, p.shift[j] >> 2, p.shift[j] & 3u);
     }
-    const uint64_t off = t * 1024;
     const uint64_t left = p.nvec * 16 - off;
+    const uint32_t cap = t ? 1024u : 1024u - p.lead;
     __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)((char *)p.dst + headBytes + off), 0, left < 1024 ? (uint32_t)left : 1024u, kRsrcFlags);
+        (void *)((char *)p.dst + headBytes + off), 0, left < cap ? (uint32_t)left : cap, kRsrcFlags);
     __builtin_amdgcn_raw_buffer_store_b128(foldVec<T, OP, K>(in, K), rd, lane * 16u, 0, kStoreAux);
   }
   // head and tail elements (fewer than 2*N <= 32): last workgroup, one lane each

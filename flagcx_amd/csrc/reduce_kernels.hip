@@ -68,6 +68,42 @@ static Split splitFor(const ReduceCall &c) {
   return s;
 }
 
+// Where the tiles start.  All pointers agree modulo 16 here, but not necessarily modulo
+// the 128-byte cache line, and a KiB tile that does not start on a line shares its first
+// and last line with its neighbours, which run on other XCDs: such a stream costs an
+// extra line fetch (or a partial line write) per KiB.  The first tile is cut short by
+// `lead` bytes so that all later tiles start on a line of as many of the K + 1 streams as
+// possible (the destination counts double: a straddling store stream costs more than a
+// straddling load stream).  Measured, 256 MiB bf16 per input, percent of peak: every
+// buffer 16 or 64 bytes into a line 68 / 74-77 -> 83-85 (as with line-aligned buffers);
+// sources 80 and destination 16 bytes into a line 66-70 -> 78.
+// Sources that still straddle get runs of kLineRun consecutive tiles per XCD, so that a
+// shared line is fetched into one L2 once (+1 to +3 points; with only the destination
+// straddling the runs cost 2 to 6 points and are not used, as they cost 4 with every
+// stream on a line).
+constexpr uint32_t kLineRun = 8;
+template <int K>
+static void setTiling(ReduceParams<K> &p, const ReduceCall &c, const Split &s) {
+  const uintptr_t headBytes = s.head * sizeof(elem_t);
+  uint32_t off[K + 1];
+  for (int j = 0; j < K; j++) off[j] = (uint32_t)(((uintptr_t)c.src[j] + headBytes) & 127u);
+  off[K] = (uint32_t)(((uintptr_t)c.dst + headBytes) & 127u);
+  uint32_t best = off[K];
+  int bestScore = -1;
+  for (int i = 0; i <= K; i++) {
+    int score = 0;
+    for (int j = 0; j <= K; j++) score += off[j] == off[i] ? (j == K ? 2 : 1) : 0;
+    if (score > bestScore) {
+      bestScore = score;
+      best = off[i];
+    }
+  }
+  p.lead = s.nvec ? best : 0; // tile 1 starts 1024 - best bytes in: on a line of the streams that sit `best` bytes into theirs
+  bool sourceStraddles = false;
+  for (int j = 0; j < K; j++) sourceStraddles = sourceStraddles || off[j] != best;
+  p.run = sourceStraddles ? kLineRun : 1;
+}
+
 template <int OP, int K>
 static int launchFixed(const ReduceCall &c, const Split &s) {
   constexpr int U = unrollFor(K);
@@ -79,16 +115,21 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   p.tail = s.tail;
   p.k = K;
   const uint64_t tileBytes = 64ull * U * 16ull;
-  uint64_t tiles = (s.nvec * 16 + tileBytes - 1) / tileBytes;
+  setTiling(p, c, s);
+  uint64_t tiles = (s.nvec * 16 + p.lead + tileBytes - 1) / tileBytes;
   // a limit on the inputs in flight per wavefront trades latency per wavefront for
   // DRAM efficiency: by default only where the launch runs many rounds of resident
   // wavefronts
   const LaunchShape shape = launchShapeFor(K, tiles);
   p.inflight = shape.loads;
   if (tiles < 1) tiles = 1;
+  if (p.run > 1) tiles = (tiles + 8ull * p.run - 1) / (8ull * p.run) * (8ull * p.run);
   if (tiles > kMaxGrid) tiles = kMaxGrid;
   const int lds = ldsReservation(shape.waves);
-  reduceWaveKernel<elem_t, OP, K, U><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
+  if (p.lead == 0 && p.run == 1)
+    reduceWaveKernel<elem_t, OP, K, U, false><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
+  else
+    reduceWaveKernel<elem_t, OP, K, U, true><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -103,6 +144,8 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   p.tail = s.tail;
   p.k = c.k;
   p.inflight = 0;
+  p.lead = 0;
+  p.run = 1;
   uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
@@ -140,7 +183,9 @@ static int launchShift(const ReduceCall &c, const Split &s) {
   p.nvec = s.nvec;
   p.head = s.head;
   p.tail = s.tail;
-  const uint64_t tiles = (s.nvec + 63) / 64;
+  // the first tile is cut short so that the others start on a 128-byte line of the destination
+  p.lead = s.nvec ? (uint32_t)(((uintptr_t)c.dst + headBytes) & 127u) : 0;
+  const uint64_t tiles = (s.nvec * 16 + p.lead + 1023) / 1024;
   // One tile per wavefront, dealt out in runs of kShiftRun tiles per XCD (whole rounds of
   // 8 runs).  Measured on MI355X, bf16 over rotating buffers, percent of peak at 32 /
   // 128 / 512 MiB per input: 1 input (a misaligned copy) 66 / 77 / 81, 2: 71 / 80 / 83,
@@ -208,7 +253,9 @@ static int launchBatchFixed(const ReduceCall *calls, const Split *splits, int n)
       p.tail = s.tail;
       p.k = K;
       p.inflight = 0;
-      const uint64_t tiles = (s.nvec * 16 + tileBytes - 1) / tileBytes;
+      setTiling(p, c, s);
+      uint64_t tiles = (s.nvec * 16 + p.lead + tileBytes - 1) / tileBytes;
+      if (p.run > 1) tiles = (tiles + 8ull * p.run - 1) / (8ull * p.run) * (8ull * p.run);
       if (tiles > maxTiles) maxTiles = tiles;
       totalTiles += tiles;
     }
@@ -216,8 +263,14 @@ static int launchBatchFixed(const ReduceCall *calls, const Split *splits, int n)
     const LaunchShape shape = launchShapeFor(K, totalTiles);
     for (int i = 0; i < m; i++) bp.seg[i].inflight = shape.loads;
     const int lds = ldsReservation(shape.waves);
-    reduceBatchKernel<elem_t, OP, K, U>
-        <<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, calls[0].stream>>>(bp);
+    bool tiled = false;
+    for (int i = 0; i < m; i++) tiled = tiled || bp.seg[i].lead != 0 || bp.seg[i].run != 1;
+    if (tiled)
+      reduceBatchKernel<elem_t, OP, K, U, true>
+          <<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, calls[0].stream>>>(bp);
+    else
+      reduceBatchKernel<elem_t, OP, K, U, false>
+          <<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, calls[0].stream>>>(bp);
     const int err = (int)hipGetLastError();
     if (err) return err;
   }

@@ -145,6 +145,45 @@ def test_unaligned_and_mixed_offsets(L, dt):
         assert same(got[:doff], guard[:doff]) and same(got[doff + n:], guard[doff + n:]), (offs, doff)
 
 
+@pytest.mark.parametrize("dt,k", [(O.BF16, 8), (O.FP32, 2), (O.INT8, 3), (O.FP64, 1), (O.INT32, 5)],
+                         ids=lambda v: str(v))
+def test_positions_inside_cache_lines(L, dt, k):
+    """Buffers that start anywhere inside a 128-byte line: the first tile is cut short so that
+    later tiles start on a line (of most buffers, or of the destination), tiles may be dealt
+    out in runs per XCD, and grids are padded to whole rounds; every byte of the result and
+    nothing outside it is written, for sizes of less than a tile, a few tiles and many rounds."""
+    import torch
+    ts = O.type_size(dt)
+    per16 = 16 // ts
+    pad = 256 // ts
+    for n in (per16 * 3 + 1, 1024 // ts * 5 + 3, 1024 // ts * 200 + per16 + 1):
+        srcs = make_inputs(dt, k, n + 2 * pad, seed=31 + dt + n % 97)
+        devs = [to_dev(s) for s in srcs]
+        # (source offsets, destination offset) in elements: all at the same place in their lines,
+        # sources on a line and the destination not, the other way round, every source elsewhere
+        # (same offset modulo 16 bytes), and sources that need the lane-shift kernel
+        cases = [([per16] * k, per16), ([4 * per16] * k, 4 * per16), ([0] * k, per16), ([5 * per16] * k, per16),
+                 ([(j % 8) * per16 for j in range(k)], 2 * per16), ([1 + j % 3 for j in range(k)], per16),
+                 ([1 + j % 3 for j in range(k)], 3 * per16 + 1)]
+        for offs, doff in cases:
+            out = dev_empty(n + 2 * pad, ts, fill=0x55 if ts == 1 else 0x5555)
+            guard = from_dev(out, srcs[0].dtype).copy()
+            views = [d[o:o + n] for d, o in zip(devs, offs)]
+            L.reduce(views, out[doff:doff + n], O.SUM, dtype=dt)
+            torch.cuda.synchronize()
+            rc, want = O.reduce([np.ascontiguousarray(s[o:o + n]) for s, o in zip(srcs, offs)], dt, O.SUM)
+            got = from_dev(out, srcs[0].dtype)
+            assert same(got[doff:doff + n], want, nan_class=is_float(dt), dtype=dt), (n, offs, doff)
+            assert same(got[:doff], guard[:doff]) and same(got[doff + n:], guard[doff + n:]), (n, offs, doff)
+        # in place on the first input, inside a line
+        o = 3 * per16
+        want = O.reduce([np.ascontiguousarray(s[o:o + n]) for s in srcs], dt, O.SUM)[1]
+        views = [d[o:o + n] for d in devs]
+        L.reduce(views, views[0], O.SUM, dtype=dt)
+        torch.cuda.synchronize()
+        assert same(from_dev(devs[0], srcs[0].dtype)[o:o + n], want, nan_class=is_float(dt), dtype=dt), n
+
+
 @pytest.mark.parametrize("dt", [O.FP32, O.BF16, O.INT32], ids=lambda d: DT_NAME[d])
 def test_in_place_on_any_input(L, dt):
     import torch
