@@ -35,18 +35,25 @@ struct ListParams {
 };
 
 // LIST: 0 both sides strided, 1 sources from a pointer list, 2 destinations from one
-template <int U, int LIST>
+// TILED: a chunk's first tile is cut short by the destination's position inside its
+// 128-byte cache line, so that all later tiles store whole lines (a tile that starts
+// inside a line shares its first and last line with tiles that run on other XCDs: two
+// partial writes per line, 66-76 % of peak for a 256 MiB copy where whole lines reach
+// 83 %).  Chunks whose destinations all start on a line take the kernel without it.
+template <int U, int LIST, bool TILED>
 __device__ __forceinline__ void copyWaveBody(const CopyParams &p, const ListParams *l) {
   constexpr uint32_t kTileBytes = 64u * U * 16u;
-  const uint64_t ntiles = (p.body + kTileBytes - 1) / kTileBytes;
   const uint32_t voff = threadIdx.x * 16u;
   for (uint64_t c = blockIdx.y; c < p.nchunks; c += gridDim.y) {
     const char *s = (LIST == 1 ? l->src[c] : p.src + c * p.srcStride) + p.head;
     char *d = (LIST == 2 ? l->dst[c] : p.dst + c * p.dstStride) + p.head;
+    const uint32_t lead = TILED ? (uint32_t)((uintptr_t)d & 127u) : 0;
+    const uint64_t ntiles = (p.body + lead + kTileBytes - 1) / kTileBytes;
     for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-      const uint64_t off = t * kTileBytes;
+      const uint64_t off = TILED ? (t ? t * kTileBytes - lead : 0) : t * kTileBytes;
       const uint64_t left = p.body - off;
-      const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
+      const uint32_t cap = TILED ? (t ? kTileBytes : kTileBytes - lead) : kTileBytes;
+      const uint32_t span = left < cap ? (uint32_t)left : cap;
       __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(s + off), 0, span, kRsrcFlags);
       __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void *)(d + off), 0, span, kRsrcFlags);
       u32x4 v[U];
@@ -70,13 +77,13 @@ __device__ __forceinline__ void copyWaveBody(const CopyParams &p, const ListPara
 
 // The strided form carries 72 bytes of arguments; only the list forms pay for the
 // pointer tables.
-template <int U>
+template <int U, bool TILED>
 __global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p) {
-  copyWaveBody<U, 0>(p, nullptr);
+  copyWaveBody<U, 0, TILED>(p, nullptr);
 }
-template <int U, int LIST>
+template <int U, int LIST, bool TILED>
 __global__ void __launch_bounds__(64) copyWaveListKernel(CopyParams p, ListParams l) {
-  copyWaveBody<U, LIST>(p, &l);
+  copyWaveBody<U, LIST, TILED>(p, &l);
 }
 
 // Element path: W-byte units, chunk by chunk.
@@ -105,14 +112,25 @@ static int launchCopyT(const CopyParams &p, const ListParams &l, bool vector, un
   const uint64_t gy = p.nchunks < kMaxGridY ? p.nchunks : kMaxGridY;
   if (vector) {
     constexpr uint64_t tileBytes = 64ull * kCopyUnroll * 16ull;
-    uint64_t gx = (p.body + tileBytes - 1) / tileBytes;
+    // does every chunk's destination body start on a 128-byte line?
+    bool onLines = true;
+    if (LIST == 2) {
+      for (uint64_t j = 0; j < p.nchunks; j++) onLines = onLines && (((uintptr_t)l.dst[j] + p.head) & 127u) == 0;
+    } else {
+      onLines = (((uintptr_t)p.dst + p.head) & 127u) == 0 && (p.nchunks == 1 || (p.dstStride & 127u) == 0);
+    }
+    uint64_t gx = (p.body + (onLines ? 0 : 127) + tileBytes - 1) / tileBytes;
     if (gx < 1) gx = 1;
     if (gx > kMaxGridX) gx = kMaxGridX;
     const int lds = ldsReservation(launchShapeFor(0, 0).waves);
-    if (LIST == 0)
-      copyWaveKernel<kCopyUnroll><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), lds, stream>>>(p);
-    else
-      copyWaveListKernel<kCopyUnroll, LIST><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), lds, stream>>>(p, l);
+    const dim3 grid((unsigned)gx, (unsigned)gy);
+    if (LIST == 0) {
+      if (onLines) copyWaveKernel<kCopyUnroll, false><<<grid, dim3(64), lds, stream>>>(p);
+      else copyWaveKernel<kCopyUnroll, true><<<grid, dim3(64), lds, stream>>>(p);
+    } else {
+      if (onLines) copyWaveListKernel<kCopyUnroll, LIST, false><<<grid, dim3(64), lds, stream>>>(p, l);
+      else copyWaveListKernel<kCopyUnroll, LIST, true><<<grid, dim3(64), lds, stream>>>(p, l);
+    }
     return (int)hipGetLastError();
   }
   uint64_t gx = (p.chunkBytes / width + 255) / 256;
@@ -228,14 +246,20 @@ __global__ void __launch_bounds__(64 * kFillWaves) fillWaveKernel(FillParams p) 
   const int r = blockIdx.y;
   char *base = p.ptr[r] + p.head[r];
   const uint64_t body = p.body[r];
-  const uint64_t ntiles = (body + kTileBytes - 1) / kTileBytes;
+  // the first tile is cut short by the range's position inside its 128-byte cache line,
+  // so that every later tile stores whole lines: tiles that start inside a line share
+  // lines with tiles of other workgroups, and a store stream of partial lines runs at
+  // 48 % of peak where whole lines reach 88-90 % (1 GiB, range 16 bytes into a line)
+  const uint32_t lead = (uint32_t)((uintptr_t)base & 127u);
+  const uint64_t ntiles = (body + lead + kTileBytes - 1) / kTileBytes;
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
   const uint32_t voff = lane * 16u;
   const u32x4 v = {p.pattern, p.pattern, p.pattern, p.pattern};
   for (uint64_t t = (uint64_t)blockIdx.x * kFillWaves + wave; t < ntiles; t += (uint64_t)gridDim.x * kFillWaves) {
-    const uint64_t off = t * kTileBytes;
+    const uint64_t off = t ? t * kTileBytes - lead : 0;
     const uint64_t left = body - off;
-    const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
+    const uint32_t cap = t ? kTileBytes : kTileBytes - lead;
+    const uint32_t span = left < cap ? (uint32_t)left : cap;
     __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void *)(base + off), 0, span, kRsrcFlags);
     __builtin_amdgcn_raw_buffer_store_b128(v, rd, voff, 0, kStoreAux);
   }
@@ -269,7 +293,7 @@ int launchFill(void *p0, uint64_t n0, void *p1, uint64_t n1, int value, hipStrea
   const uint32_t b = (uint32_t)(value & 0xff);
   p.pattern = b | (b << 8) | (b << 16) | (b << 24);
   constexpr uint64_t groupBytes = 1024ull * kFillWaves;
-  uint64_t gx = (maxBody + groupBytes - 1) / groupBytes;
+  uint64_t gx = (maxBody + 127 + groupBytes - 1) / groupBytes; // a range inside a line has a short first tile
   if (gx < 1) gx = 1;
   if (gx > kMaxGridX) gx = kMaxGridX;
   fillWaveKernel<<<dim3((unsigned)gx, (unsigned)nr), dim3(64 * kFillWaves), 0, stream>>>(p);

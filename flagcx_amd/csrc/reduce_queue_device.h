@@ -287,19 +287,29 @@ __device__ inline void queueLeader(const QueueKernelArgs &q) {
 // per KiB (two fp32 inputs, 32 entries of 4 MiB: 4.6 -> 5.9 TB/s).
 constexpr int queueUnitTiles(int k) { return k <= 2 ? 8 : k <= 4 ? 4 : 1; }
 
+// Where an entry's body sits inside a 128-byte line of its destination (a multiple of 16).
+__device__ __forceinline__ uint32_t queueLead(uint64_t dst, uint64_t headBytes) {
+  return (uint32_t)((dst + headBytes) & 127u);
+}
+
 // This worker's units of one entry, K inputs known at compile time.  ALIGNED:
 // every pointer agrees modulo 16 and tiles go through clipped buffer descriptors;
 // otherwise the destination's tiling with unaligned 16-byte loads.
 template <typename T, int OP, int K, int G, bool ALIGNED>
 __device__ __forceinline__ void queueTiles(const uint64_t (&src)[8], uint64_t dst, uint64_t headBytes,
-                                           uint64_t bodyBytes, uint64_t first, uint64_t stride) {
+                                           uint64_t bodyBytes, uint32_t lead, uint64_t first, uint64_t stride) {
   constexpr uint32_t kUnitBytes = 1024u * G;
   const uint32_t voff = threadIdx.x * 16u;
-  const uint64_t nunits = (bodyBytes + kUnitBytes - 1) / kUnitBytes;
+  // the first unit is short by `lead` bytes, so that the others start on a 128-byte line
+  // of the destination (units that start inside a line share lines with units that other
+  // XCDs fold)
+  const uint64_t nunits = (bodyBytes + lead + kUnitBytes - 1) / kUnitBytes;
   for (uint64_t u = first; u < nunits; u += stride) {
-    const uint64_t off = headBytes + u * kUnitBytes;
-    const uint64_t left = bodyBytes - u * kUnitBytes;
-    const uint32_t span = left < kUnitBytes ? (uint32_t)left : kUnitBytes;
+    const uint64_t boff = u ? u * kUnitBytes - lead : 0;
+    const uint64_t off = headBytes + boff;
+    const uint64_t left = bodyBytes - boff;
+    const uint32_t cap = u ? kUnitBytes : kUnitBytes - lead;
+    const uint32_t span = left < cap ? (uint32_t)left : cap;
     u32x4 in[G][K];
     if (ALIGNED) {
 #pragma unroll
@@ -336,12 +346,13 @@ __device__ __forceinline__ void queueEntry(const uint64_t (&src)[8], uint64_t ds
   constexpr int N = 16 / sizeof(T);
   constexpr int G = queueUnitTiles(K);
   const uint64_t headBytes = (uint64_t)head * sizeof(T);
+  const uint32_t lead = queueLead(dst, headBytes);
   if (aligned) {
-    queueTiles<T, OP, K, G, true>(src, dst, headBytes, nvec * 16, first, stride);
+    queueTiles<T, OP, K, G, true>(src, dst, headBytes, nvec * 16, lead, first, stride);
   } else {
     // plain global loads carry no scope bits: drop whatever this CU and L2 hold
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "");
-    queueTiles<T, OP, K, G, false>(src, dst, headBytes, nvec * 16, first, stride);
+    queueTiles<T, OP, K, G, false>(src, dst, headBytes, nvec * 16, lead, first, stride);
   }
   // head and tail elements: the worker that owns unit 0, one lane each
   if (first == 0 && threadIdx.x < head + tail) {
@@ -434,7 +445,9 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
         return;
       }
       const uint64_t unitBytes = 1024ull * (uint32_t)queueUnitTiles(k);
-      nunits = (laneWord(cur, 9) * 16 + unitBytes - 1) / unitBytes;
+      const uint64_t elemBytes = sizeof(T);
+      nunits = (laneWord(cur, 9) * 16 + queueLead(laneWord(cur, 8), (uint32_t)laneWord(cur, 10) * elemBytes) + unitBytes - 1) /
+               unitBytes;
       if (nunits == 0) nunits = 1; // head and tail elements only: still somebody's unit
       if (unit < unitBase + nunits) break;
       unitBase += nunits;

@@ -4,7 +4,7 @@
 //
 //   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
 //             [-W wavesPerCU] [-L lingerPolls] [-s spinLimit] [-q ringCapacity]
-//             [-D windowBytes] [-a separateAllocations] [-g arrivalGapUs]
+//             [-D windowBytes] [-a separateAllocations] [-g arrivalGapUs] [-x bytesIntoTheBuffers]
 //
 // A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
 // staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
@@ -13,6 +13,7 @@
 // With -g the chunks are handed over one every arrivalGapUs microseconds of host
 // time (chunks that arrive one by one, the case the queue is for) instead of all at
 // once; the batch call, which needs every chunk, then starts after the last arrival.
+// With -x every buffer starts that many bytes further on (positions inside 128-byte lines).
 // Also: latency of ONE small entry, enqueue -> Wait, against launch -> stream sync.
 #include "../../include/flagcx_amd.h"
 
@@ -66,6 +67,7 @@ int main(int argc, char **argv) {
   long long linger = -1;
   int capacity = 64, separate = 0;
   double gapUs = 0.0;
+  size_t shift = 0; // -x: every buffer starts this many bytes further on (positions inside cache lines)
   size_t window = 0;
   for (int i = 1; i + 1 < argc; i += 2) {
     const char *f = argv[i], *v = argv[i + 1];
@@ -83,6 +85,7 @@ int main(int argc, char **argv) {
     else if (!strcmp(f, "-D")) window = strtoull(v, 0, 0);
     else if (!strcmp(f, "-a")) separate = atoi(v);
     else if (!strcmp(f, "-g")) gapUs = atof(v);
+    else if (!strcmp(f, "-x")) shift = strtoull(v, 0, 0);
   }
   flagcxLocalReduceFifo_t fifo = nullptr;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
@@ -96,13 +99,15 @@ int main(int argc, char **argv) {
   std::vector<void *> src(k + 1);
   void *pool = nullptr;
   if (separate) {
-    for (int j = 0; j <= k; j++) CK(hipMalloc(&src[j], shardBytes));
+    for (int j = 0; j <= k; j++) CK(hipMalloc(&src[j], shardBytes + 4096));
   } else {
     const size_t poolBytes = (size_t)(k + 1) * (shardBytes + 128 * 1024);
     CK(hipMalloc(&pool, poolBytes));
     FX(flagcxLocalPlaceBuffers(pool, poolBytes, shardBytes, k + 1, src.data()));
   }
   for (int j = 0; j <= k; j++) CK(hipMemset(src[j], 0, shardBytes)); // zeros are valid in every type
+  if (shift % ts || shift > 4096) return 2;
+  for (int j = 0; j <= k; j++) src[j] = (char *)src[j] + shift;
   void *dst = src[k];
   flagcxStream st;
   CK(hipStreamCreateWithFlags(&st.base, hipStreamNonBlocking));
@@ -220,7 +225,7 @@ int main(int argc, char **argv) {
   FX(flagcxLocalReduceFifoDestroy(fifo));
   fifo = nullptr;
   if (separate)
-    for (int j = 0; j <= k; j++) CK(hipFree(src[j]));
+    for (int j = 0; j <= k; j++) CK(hipFree((char *)src[j] - shift));
   else
     CK(hipFree(pool));
   return 0;

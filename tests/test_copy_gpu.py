@@ -29,7 +29,8 @@ def test_memcpy_sizes_and_offsets(L, size):
     import torch
     src_h = rand_bytes(size + 64, size)
     src = to_dev(src_h)
-    for so, do in ((0, 0), (1, 1), (3, 3), (0, 5), (7, 2), (4, 8), (2, 4)):
+    # the last four: 16-byte aligned on both sides but inside a 128-byte line (short first tile)
+    for so, do in ((0, 0), (1, 1), (3, 3), (0, 5), (7, 2), (4, 8), (2, 4), (16, 16), (0, 48), (32, 0), (19, 35)):
         dst = torch.full((size + 64,), 0xAB, dtype=torch.uint8, device="cuda")
         L.memcpy(dst.data_ptr() + do, src.data_ptr() + so, size)
         torch.cuda.synchronize()
@@ -54,7 +55,7 @@ def test_self_copy_reference_pattern(L):
 @pytest.mark.parametrize("size", [1, 31, 4096, 100003])
 def test_memset(L, size):
     import torch
-    for off, val in ((0, 0), (1, 0x5A), (9, 0xFF), (16, 7)):
+    for off, val in ((0, 0), (1, 0x5A), (9, 0xFF), (16, 7), (48, 3), (35, 9)):
         buf = torch.full((size + 64,), 0xCD, dtype=torch.uint8, device="cuda")
         L.memset(buf.data_ptr() + off, val, size)
         torch.cuda.synchronize()
@@ -81,13 +82,13 @@ def test_refresh_matches_oracle(L, tsz, dt):
 
 
 @pytest.mark.parametrize("chunk,stride", [(64, 512), (4096, 32768), (100, 800), (48, 48), (17, 33),
-                                          (1 << 20, 8 << 20), (6, 64)])
+                                          (1 << 20, 8 << 20), (6, 64), (4096 + 16, 8192 + 48), (2048, 4096 + 16)])
 def test_pack_unpack_round_trip(L, chunk, stride):
     import torch
     nch = 8
     span = (nch - 1) * stride + chunk
     h = rand_bytes(span + 32, chunk + stride)
-    for base in (0, 4, 1):
+    for base in (0, 4, 1, 16):  # 16: vector path with every chunk inside a 128-byte line
         src = to_dev(h)
         staged = torch.full((nch * chunk + 32,), 0x77, dtype=torch.uint8, device="cuda")
         L.pack(staged.data_ptr() + base, src.data_ptr() + base, nch, chunk, stride)
