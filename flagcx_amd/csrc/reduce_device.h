@@ -294,13 +294,15 @@ __global__ void __launch_bounds__(64) reduceWaveAnyKernel(ReduceParams<FLAGCX_MA
   constexpr uint32_t kTileBytes = 1024u;
   const int k = p.k;
   const uint64_t bodyBytes = p.nvec * 16;
-  const uint64_t ntiles = (bodyBytes + kTileBytes - 1) / kTileBytes;
+  const uint32_t lead = p.lead; // the first tile is short: the others start on a cache line of most buffers
+  const uint64_t ntiles = (bodyBytes + lead + kTileBytes - 1) / kTileBytes;
   const uint64_t headBytes = p.head * sizeof(T);
   const uint32_t voff = threadIdx.x * 16u;
   for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const uint64_t off = t * kTileBytes;
+    const uint64_t off = t ? t * kTileBytes - lead : 0;
     const uint64_t left = bodyBytes - off;
-    const uint32_t span = left < kTileBytes ? (uint32_t)left : kTileBytes;
+    const uint32_t cap = t ? kTileBytes : kTileBytes - lead;
+    const uint32_t span = left < cap ? (uint32_t)left : cap;
     typename F::acc_t acc[N];
     for (int j0 = 0; j0 < k; j0 += B) {
       u32x4 in[B];

@@ -146,7 +146,18 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   p.inflight = 0;
   p.lead = 0;
   p.run = 1;
-  uint64_t tiles = (s.nvec * 16 + 1023) / 1024;
+  if (s.vector && s.nvec) {
+    // the position inside a 128-byte line that most buffers share (the destination counts double)
+    const uintptr_t headBytes = s.head * sizeof(elem_t);
+    int count[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int j = 0; j < c.k; j++) count[(((uintptr_t)c.src[j] + headBytes) & 127u) >> 4]++;
+    count[(((uintptr_t)c.dst + headBytes) & 127u) >> 4] += 2;
+    int best = 0;
+    for (int i = 1; i < 8; i++)
+      if (count[i] > count[best]) best = i;
+    p.lead = (uint32_t)best * 16u;
+  }
+  uint64_t tiles = (s.nvec * 16 + p.lead + 1023) / 1024;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
   // more than eight inputs are loaded eight at a time; measured on MI355X: 9..10

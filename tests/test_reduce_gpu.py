@@ -145,7 +145,7 @@ def test_unaligned_and_mixed_offsets(L, dt):
         assert same(got[:doff], guard[:doff]) and same(got[doff + n:], guard[doff + n:]), (offs, doff)
 
 
-@pytest.mark.parametrize("dt,k", [(O.BF16, 8), (O.FP32, 2), (O.INT8, 3), (O.FP64, 1), (O.INT32, 5)],
+@pytest.mark.parametrize("dt,k", [(O.BF16, 8), (O.FP32, 2), (O.INT8, 3), (O.FP64, 1), (O.INT32, 5), (O.FP16, 11)],
                          ids=lambda v: str(v))
 def test_positions_inside_cache_lines(L, dt, k):
     """Buffers that start anywhere inside a 128-byte line: the first tile is cut short so that
