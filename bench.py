@@ -59,7 +59,7 @@ MiB = 1 << 20
 # (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a copy of
 # known size; not measured by this program.
 TRAFFIC_SOURCE = "profiles/reduce8_bf16_sum_256MiB_pmc.txt"
-TRAFFIC_BYTES = 2415728688
+TRAFFIC_BYTES = 2415742114
 
 
 def log(*a):
@@ -742,7 +742,7 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES,
                      "traffic_source": TRAFFIC_SOURCE + " (rocprofv3 counter runs of this same command, "
                                                         "not measured by this run)",
-                     "kernel": "reduceWaveKernel<bf16,sum,K=8,U=1>", "avg_launch_ms": round(kern_ms, 5),
+                     "kernel": "reduceWaveKernel<bf16,sum,K=8,U=1,TILED=false>", "avg_launch_ms": round(kern_ms, 5),
                      "algorithmic_bytes_per_launch": ALGO_BYTES},
         "latency_us_4KiB": {"workload": "2-input fp32 sum, 4 KiB per buffer",
                             "c_caller": c_lat,
