@@ -105,9 +105,10 @@ flagcxResult_t flagcxLocalStagedReduceScatterNoAlloc(const void *const *sendbuff
     return sfail(flagcxInvalidArgument, "%s: %zu elements of %zu bytes exceed the static staging area of %zu bytes",
                  who, recvcount, ts, kStagingBytes);
   const size_t size = recvcount * ts;
-  // a peer's region: its slice at recvbuff's offset inside a 16-byte line (so that
-  // the reduce sees every input at the same offset), regions 256-byte aligned
-  const size_t skew = (uintptr_t)recvbuff & 15u;
+  // a peer's region: its slice at recvbuff's position inside a 128-byte cache line (so
+  // that the reduce sees the staged inputs and the output at the same position and
+  // starts its tiles on their lines), regions 256-byte aligned
+  const size_t skew = (uintptr_t)recvbuff & 127u;
   const size_t region = (skew + size + kRegionAlign - 1) / kRegionAlign * kRegionAlign;
   const size_t need = (size_t)(nranks - 1) * region;
   if (need > kStagingBytes)
