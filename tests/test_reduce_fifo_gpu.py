@@ -80,9 +80,10 @@ def test_fifo_misaligned_and_in_place(L, dt, op, k):
     n = 50_000
     isz = np.dtype(O.NP_OF[dt]).itemsize
     pad = 16 // isz
-    ins = make_inputs(dt, k, n + 2 * pad, seed=7, op=op)
+    ins = make_inputs(dt, k, n + 8 * pad, seed=7, op=op)
     devs = [to_dev(a) for a in ins]
     out_a = dev_empty(n + 2 * pad, isz, fill=0)
+    out_d = dev_empty(n + 8 * pad, isz, fill=0)
     out_b = dev_empty(n + 2 * pad, isz, fill=0)
     torch.cuda.synchronize()
     # a: every pointer shifted by one element; b: source j shifted by j % pad elements, dst by 1
@@ -95,6 +96,8 @@ def test_fifo_misaligned_and_in_place(L, dt, op, k):
             q.enqueue_reduce([d.data_ptr() + isz for d in devs], out_a.data_ptr() + isz, n)
             q.enqueue_reduce([d.data_ptr() + offs_b[j] * isz for j, d in enumerate(devs)], out_b.data_ptr() + isz, n)
             q.enqueue_reduce([inplace.data_ptr()] + [d.data_ptr() for d in devs[1:]], inplace.data_ptr(), n)
+            # d: 16-byte aligned, 80 bytes into a cache line (sources) and 48 bytes (destination): short first unit
+            q.enqueue_reduce([d.data_ptr() + 80 for d in devs], out_d.data_ptr() + 48, n)
     finally:
         q.close()
     npdt = ins[0].dtype
@@ -105,9 +108,13 @@ def test_fifo_misaligned_and_in_place(L, dt, op, k):
     want_b = expect([a[offs_b[j]:offs_b[j] + n] for j, a in enumerate(ins)], dt, op)
     assert same(got_b[1:n + 1], want_b, nan_class=nan_ok(dt, op), dtype=dt)
     assert not got_b[0].tobytes().strip(b"\0") and not got_b[n + 1:].tobytes().strip(b"\0")
+    got_d = from_dev(out_d, npdt)
+    so, do = 80 // isz, 48 // isz
+    assert same(got_d[do:do + n], expect([a[so:so + n] for a in ins], dt, op), nan_class=nan_ok(dt, op), dtype=dt)
+    assert not got_d[:do].tobytes().strip(b"\0") and not got_d[do + n:].tobytes().strip(b"\0")
     got_c = from_dev(inplace, npdt)
     assert same(got_c[:n], expect([a[:n] for a in ins], dt, op), nan_class=nan_ok(dt, op), dtype=dt)
-    assert same(got_c[n:], ins[0][n:])
+    assert same(got_c[n:n + 2 * pad], ins[0][n:n + 2 * pad])
 
 
 def test_fifo_triggers_chain(L):
