@@ -24,7 +24,7 @@
 // atomics, and "release" is waiting for the wavefront's own stores (s_waitcnt)
 // before the progress word is written.  Only entries whose sources need
 // unaligned global loads (no cache-policy bits there) fall back to a system-scope
-// acquire fence in front of the entry.
+// acquire fence in front of every unit.
 //
 // Every wait is bounded by maxSpin polls: a host that stops producing, or a
 // worker that never becomes resident, ends in kQueueTimedOut, not in a hang
@@ -292,7 +292,8 @@ __device__ __forceinline__ uint32_t queueLead(uint64_t dst, uint64_t headBytes) 
   return (uint32_t)((dst + headBytes) & 127u);
 }
 
-// This worker's units of one entry, K inputs known at compile time.  ALIGNED:
+// The units first, first + stride, ... of one entry (a ticket is one unit), K inputs known at
+// compile time.  ALIGNED:
 // every pointer agrees modulo 16 and tiles go through clipped buffer descriptors;
 // otherwise the destination's tiling with unaligned 16-byte loads.
 template <typename T, int OP, int K, int G, bool ALIGNED>
