@@ -529,6 +529,51 @@ def table_dtypes(L, args):
         torch.cuda.empty_cache()
 
 
+POSITIONS = [("every buffer on a 128-byte line", lambda j, k: 0, 0),
+             ("every buffer 16 bytes into a line", lambda j, k: 16, 16),
+             ("every buffer 64 bytes into a line", lambda j, k: 64, 64),
+             ("sources 16 bytes in, destination on a line", lambda j, k: 16, 0),
+             ("sources on a line, destination 16 bytes in", lambda j, k: 0, 16),
+             ("sources 80 bytes in, destination 16 bytes in", lambda j, k: 80, 16),
+             ("sources 2..14 bytes in (another offset modulo 16)", lambda j, k: 2 + 2 * (j % 7), 0),
+             ("the same, destination 16 bytes in", lambda j, k: 2 + 2 * (j % 7), 16)]
+
+
+def table_positions(L, args):
+    """bf16 sum of k inputs whose buffers start at several positions inside their 128-byte
+    cache lines (separate allocations, --sets sets used in turn); percent of 8 TB/s.
+    --once: one launch per case and nothing else (for counter runs)."""
+    import torch
+    lib = L.lib()
+    nbytes = args.mib * MiB
+    n = nbytes // 2
+    st = L.current_stream()
+    sref = C.byref(st)
+    for k in args.k:
+        nsets = 1 if args.once else args.sets
+        raws = [[torch.empty(n + 256, dtype=torch.bfloat16, device="cuda") for _ in range(k + 1)] for _ in range(nsets)]
+        for raw in raws:
+            for t in raw[:k]:
+                t.view(torch.int16).random_(0, 16000)
+        if not args.once:
+            print("k=%d bf16 sum, %d MiB per input, %d buffer set(s) in turn; percent of 8 TB/s" % (k, args.mib, nsets),
+                  flush=True)
+        for name, so, do in POSITIONS:
+            sets = [((C.c_void_p * k)(*[raw[j].data_ptr() + so(j, k) for j in range(k)]), raw[k].data_ptr() + do)
+                    for raw in raws]
+
+            def go(i):
+                L.check(lib.flagcxLocalReduce(sets[i][0], k, sets[i][1], n, 9, int(L.RedOp.Sum), sref))
+            if args.once:
+                go(0)
+                torch.cuda.synchronize()
+                continue
+            ms = timed_sets_ms(go, nsets, warmup=2 * nsets, iters=8 * nsets)
+            print("  %-52s %5.1f" % (name, (k + 1) * nbytes / (ms * 1e-3) / 1e9 / 80.0), flush=True)
+        del raws
+        torch.cuda.empty_cache()
+
+
 STRIDES = [128 * MiB, 128 * MiB + 4096, 128 * MiB + 65536, 129 * MiB + 4096, 256 * MiB, 512 * MiB,
            1024 * MiB, 1024 * MiB + 4096, 1024 * MiB + 65536, 1025 * MiB, 1026 * MiB + 8192, 1057 * MiB + 12288]
 CAPS = [8, 10, 12, 14, 16, 18, 21, 25, 0, -1]   # caps that whole LDS granules can express; -1 = the library's choice
@@ -598,13 +643,14 @@ def main():
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also run N flagcxLocalMemcpy launches of 256 MiB (a copy of known size "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--table", choices=["sweep", "sweep-rotate", "configs", "dtypes", "stride"],
+    ap.add_argument("--table", choices=["sweep", "sweep-rotate", "configs", "dtypes", "stride", "positions"],
                     help="print one of the tables instead of the JSON line")
     ap.add_argument("--min", type=int, default=1 << 10, help="sweep tables: smallest size")
     ap.add_argument("--max", type=int, default=1 << 30, help="sweep tables: largest size")
-    ap.add_argument("--k", type=int, nargs="+", default=[8, 4, 2], help="dtypes / stride tables: inputs")
-    ap.add_argument("--mib", type=int, default=256, help="dtypes / stride tables: MiB per input")
-    ap.add_argument("--sets", type=int, default=2, help="dtypes / stride tables: buffer sets used in turn")
+    ap.add_argument("--k", type=int, nargs="+", default=[8, 4, 2], help="dtypes / stride / positions tables: inputs")
+    ap.add_argument("--mib", type=int, default=256, help="dtypes / stride / positions tables: MiB per input")
+    ap.add_argument("--sets", type=int, default=2, help="dtypes / stride / positions tables: buffer sets used in turn")
+    ap.add_argument("--once", action="store_true", help="positions table: one launch per case, no timing")
     ap.add_argument("--loads", type=int, default=-1,
                     help="stride table: inputs in flight per wavefront for the cap columns (-1: the library's choice)")
     args = ap.parse_args()
@@ -623,7 +669,7 @@ def main():
 
     if args.table:
         {"sweep": table_sweep, "sweep-rotate": table_sweep, "configs": table_configs, "dtypes": table_dtypes,
-         "stride": table_stride}[args.table](L, args)
+         "stride": table_stride, "positions": table_positions}[args.table](L, args)
         return
 
     # The 8 input buffers and the output live in one allocation, at the addresses
