@@ -256,7 +256,9 @@ def test_every_number_of_inputs_in_flight_gives_the_same_bytes(L, k, dt, op):
 
 
 def test_buffers_beyond_4GiB(L):
-    """Counts and byte offsets past 2^32: reduce, copy, fill and strided pack."""
+    """Counts and byte offsets past 2^32: reduce, copy, fill and strided pack.  (Every
+    assertion is on a plain bool or int computed beforehand: a failing assertion that
+    holds a 4 GiB tensor makes the test runner format it on the host.)"""
     import torch
     n = (1 << 32) + 4099
     g = torch.Generator(device="cuda").manual_seed(7)
@@ -265,22 +267,69 @@ def test_buffers_beyond_4GiB(L):
     out = torch.empty(n, dtype=torch.uint8, device="cuda")
     L.reduce([a, b], out, L.RedOp.Sum)                       # uint8 sum wraps modulo 256
     torch.cuda.synchronize()
-    assert torch.equal(out, a + b)
+    ok = torch.equal(out, a + b)
+    assert ok
     L.reduce([a, b], out, L.RedOp.Max)
     torch.cuda.synchronize()
-    assert torch.equal(out, torch.maximum(a, b))
+    ok = torch.equal(out, torch.maximum(a, b))
+    assert ok
     out.zero_()
     L.memcpy(out.data_ptr() + 1, a.data_ptr() + 1, n - 1)    # unaligned head on both sides
     torch.cuda.synchronize()
-    assert torch.equal(out[1:], a[1:]) and int(out[0]) == 0
+    ok, first = torch.equal(out[1:], a[1:]), int(out[0])
+    assert ok and first == 0
     L.memset(out.data_ptr() + 3, 0x5A, n - 6)
     torch.cuda.synchronize()
-    assert bool((out[3:n - 3] == 0x5A).all()) and out[:3].tolist() == [0, int(a[1]), int(a[2])]
-    assert out[n - 3:].tolist() == a[n - 3:].tolist()
+    ok = bool((out[3:n - 3] == 0x5A).all())
+    head, tail, want_head, want_tail = out[:3].tolist(), out[n - 3:].tolist(), [0, int(a[1]), int(a[2])], a[n - 3:].tolist()
+    assert ok and head == want_head and tail == want_tail
     del out, b
     # 2 chunks of 2^31 + 16 bytes at stride 2^31 + 2048: offsets of the second chunk exceed 2^31
     chunk, stride = (1 << 31) + 16, (1 << 31) + 2048
     staged = torch.empty(2 * chunk, dtype=torch.uint8, device="cuda")
     L.pack(staged.data_ptr(), a.data_ptr(), 2, chunk, stride)
     torch.cuda.synchronize()
-    assert torch.equal(staged[:chunk], a[:chunk]) and torch.equal(staged[chunk:], a[stride:stride + chunk])
+    ok0, ok1 = torch.equal(staged[:chunk], a[:chunk]), torch.equal(staged[chunk:], a[stride:stride + chunk])
+    assert ok0 and ok1
+
+
+def _first_difference(x, y):
+    """Index of the first differing element, or -1; compared a GiB at a time (the
+    assertions below only ever see small integers, never a tensor)."""
+    import torch
+    step = 1 << 30
+    for i in range(0, x.numel(), step):
+        if not torch.equal(x[i:i + step], y[i:i + step]):
+            return i + int((x[i:i + step] != y[i:i + step]).nonzero()[0])
+    return -1
+
+
+def test_more_tiles_than_the_largest_grid(L):
+    """Buffers of more than 2^24 KiB: the grids are capped there and every kernel takes a
+    second pass (plain and line-tiled reduce, lane-shift reduce, copy, fill)."""
+    import torch
+    n = (1 << 34) + (1 << 20) + 5
+    g = torch.Generator(device="cuda").manual_seed(11)
+    words = torch.empty((n + 256 + 7) // 8, dtype=torch.int64, device="cuda")
+    words.random_(generator=g)
+    a = words.view(torch.uint8)
+    out = torch.empty(n + 256, dtype=torch.uint8, device="cuda")
+    for so, do in ((0, 0), (16, 16), (1, 0), (3, 16)):     # plain, tiled, shifted, shifted + tiled
+        out.zero_()
+        L.reduce([a[so:so + n]], out[do:do + n], L.RedOp.Sum)
+        torch.cuda.synchronize()
+        diff = _first_difference(out[do:do + n], a[so:so + n])
+        before, after = int(out[:do].sum()), int(out[do + n:].sum())
+        assert (diff, before, after) == (-1, 0, 0), (so, do)
+    out.zero_()
+    L.memcpy(out.data_ptr() + 48, a.data_ptr() + 16, n)
+    torch.cuda.synchronize()
+    diff = _first_difference(out[48:48 + n], a[16:16 + n])
+    before, after = int(out[:48].sum()), int(out[48 + n:].sum())
+    assert (diff, before, after) == (-1, 0, 0)
+    out.zero_()
+    L.memset(out.data_ptr() + 16, 0x5A, n)
+    torch.cuda.synchronize()
+    wrong = sum(int((out[i:min(i + (1 << 30), 16 + n)] != 0x5A).sum()) for i in range(16, 16 + n, 1 << 30))
+    before, after = int(out[:16].sum()), int(out[16 + n:].sum())
+    assert (wrong, before, after) == (0, 0, 0)
