@@ -98,6 +98,7 @@ flagcxResult_t launchConsumer(flagcxLocalReduceFifo *q, uint64_t base, const cha
   a.windowBytes = q->windowBytes;
   a.tickets = q->tickets;
   a.counters = 1; // the launcher sets it from the grid
+  a.drawAhead = q->maxRanks > 4 ? 1u : 0u;
   // LDS is reserved only to spread the resident wavefronts over the CUs (at most
   // `waves` + 2 fit on one), in whole 1280-byte allocation granules.  A fifth of
   // every CU's LDS stays free, so that other launches that need LDS (this library's

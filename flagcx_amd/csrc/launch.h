@@ -96,6 +96,7 @@ struct QueueKernelArgs {
   uint64_t windowBytes;          // traffic of the entries the workers may have in work together
   uint64_t *tickets;             // ticket counters, kQueueTicketStride words apart, zero at launch
   uint32_t counters;             // how many of them this launch uses (every one has workers)
+  uint32_t drawAhead;            // the queue takes entries of more than four inputs: picks the kernel instantiation
 };
 
 // Launches the consumer for one element type: grid = min(occupancy, wavesPerCU) *

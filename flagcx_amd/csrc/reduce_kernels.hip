@@ -334,11 +334,11 @@ int FLAGCX_CAT(launchReduceBatch_, FLAGCX_DT)(const ReduceCall *calls, int n) {
 
 // The resident queue consumer.  Its grid must be resident all at once, so the
 // size comes from the occupancy query for this very kernel and LDS reservation.
-template <int OP>
-static int launchQueueOp(const QueueKernelArgs &q, int wavesPerCU, int numCU, int lds, unsigned maxGrid,
+template <int OP, bool AHEAD>
+static int launchQueueOpT(const QueueKernelArgs &q, int wavesPerCU, int numCU, int lds, unsigned maxGrid,
                          hipStream_t stream, unsigned *grid) {
   int fit = 0;
-  hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reduceQueueKernel<elem_t, OP>, 64, (size_t)lds);
+  hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reduceQueueKernel<elem_t, OP, AHEAD>, 64, (size_t)lds);
   if (e != hipSuccess) return (int)e;
   if (wavesPerCU > 0 && fit > wavesPerCU) fit = wavesPerCU;
   // LDS is handed out in 1280-byte granules on gfx950 (160 KiB per CU): count what
@@ -358,8 +358,15 @@ static int launchQueueOp(const QueueKernelArgs &q, int wavesPerCU, int numCU, in
   QueueKernelArgs a = q;
   const uint64_t groups = (g - 1) / 8 + 1;
   a.counters = (uint32_t)(groups < (uint64_t)kQueueMaxTicketCounters ? groups : (uint64_t)kQueueMaxTicketCounters);
-  reduceQueueKernel<elem_t, OP><<<dim3((unsigned)g), dim3(64), lds, stream>>>(a);
+  reduceQueueKernel<elem_t, OP, AHEAD><<<dim3((unsigned)g), dim3(64), lds, stream>>>(a);
   return (int)hipGetLastError();
+}
+
+template <int OP>
+static int launchQueueOp(const QueueKernelArgs &q, int wavesPerCU, int numCU, int lds, unsigned maxGrid,
+                         hipStream_t stream, unsigned *grid) {
+  return q.drawAhead ? launchQueueOpT<OP, true>(q, wavesPerCU, numCU, lds, maxGrid, stream, grid)
+                     : launchQueueOpT<OP, false>(q, wavesPerCU, numCU, lds, maxGrid, stream, grid);
 }
 
 int FLAGCX_CAT(launchReduceQueue_, FLAGCX_DT)(int op, const QueueKernelArgs &q, int wavesPerCU, int numCU, int lds,

@@ -376,7 +376,11 @@ __device__ __forceinline__ void queueEntry(const uint64_t (&src)[8], uint64_t ds
 // ticket is fetched while the current unit is in flight; tickets drawn beyond the
 // published entries are simply held until those entries arrive.  Counters are 1 KiB
 // apart, in different memory channels.
-template <typename T, int OP>
+// AHEAD: the queue takes entries of more than four inputs (units of one KiB per input)
+// and its workers keep the next ticket on its way while they fold a unit; queues of up
+// to four inputs (units of 4 or 8 KiB) draw a ticket when they need it and hold no code
+// for more inputs.
+template <typename T, int OP, bool AHEAD>
 __device__ inline void queueWorker(const QueueKernelArgs &q) {
   const uint32_t worker = blockIdx.x - 1;
   const uint32_t nc = q.counters;
@@ -387,13 +391,17 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
   uint64_t produced = 0; // entries known to be in the device ring
   uint64_t reported = 0; // what the progress word says
   uint64_t lastBeat = 0;
-  // one ticket in hand and the next on its way: the draw is issued behind a unit's
-  // store, so that no load waits for it (memory operations of a wavefront return in
-  // the order issued), and is read a whole unit later
+  // AHEAD: one ticket in hand and the next on its way; the draw is issued behind a unit's
+  // store, so that no load waits for it (memory operations of a wavefront return in the
+  // order issued), and is read a whole unit later.  Otherwise a ticket is drawn when the
+  // previous unit's store has been issued, and waited for: drawing ahead hides the draw's
+  // latency but lets the units in work spread over a window twice as wide, which costs
+  // more than the wait when units are 4 or 8 KiB per input (3 inputs 5.95 -> 6.13 TB/s,
+  // 4 inputs 6.15 -> 6.4) and less when they are one (8 inputs 6.2 -> 6.0).
   uint64_t ticket = 0, pending = 0;
   if (threadIdx.x == 0) {
     ticket = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    pending = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (AHEAD) pending = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   ticket = uniform64(ticket);
   // lane l holds word l & 15 of entry `done` (haveCur) and of entry `done + 1` (haveNext)
@@ -401,9 +409,10 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
   bool haveCur = false, haveNext = false;
   auto report = [&]() {
     // this wavefront's results are acknowledged by memory before the count says so;
-    // the one operation that may still be on its way is the youngest, the ticket draw
-    // issued behind the last store
-    waitAllButYoungest();
+    // with AHEAD the one operation that may still be on its way is the youngest, the
+    // ticket draw issued behind the last store
+    if (AHEAD) waitAllButYoungest();
+    else waitOwnMemory();
     if (threadIdx.x == 0)
       __hip_atomic_store(q.progress + worker, (uint32_t)done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     reported = done;
@@ -478,27 +487,50 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
       case 2: queueEntry<T, OP, 2>(src, dst, head, tail, nvec, vector, first, nunits); break;
       case 3: queueEntry<T, OP, 3>(src, dst, head, tail, nvec, vector, first, nunits); break;
       case 4: queueEntry<T, OP, 4>(src, dst, head, tail, nvec, vector, first, nunits); break;
-      case 5: queueEntry<T, OP, 5>(src, dst, head, tail, nvec, vector, first, nunits); break;
-      case 6: queueEntry<T, OP, 6>(src, dst, head, tail, nvec, vector, first, nunits); break;
-      case 7: queueEntry<T, OP, 7>(src, dst, head, tail, nvec, vector, first, nunits); break;
-      default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nunits); break;
+      default:
+        if constexpr (AHEAD) {
+          switch (k) {
+            case 5: queueEntry<T, OP, 5>(src, dst, head, tail, nvec, vector, first, nunits); break;
+            case 6: queueEntry<T, OP, 6>(src, dst, head, tail, nvec, vector, first, nunits); break;
+            case 7: queueEntry<T, OP, 7>(src, dst, head, tail, nvec, vector, first, nunits); break;
+            default: queueEntry<T, OP, 8>(src, dst, head, tail, nvec, vector, first, nunits); break;
+          }
+        }
+        break; // the host admits no entry with more inputs than the queue was created for
+    }
+    if constexpr (AHEAD) {
+      ticket = uniform64(pending);
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
+      if (threadIdx.x == 0) pending = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    } else {
+      // This counter's next unit lies nc further on: if that is beyond the entry, the worker
+      // has passed it, and if nothing else is published it says so at once (the progress
+      // of a lone small entry does not wait for the ticket draw).
+      if (unit + nc >= unitBase + nunits) {
+        unitBase += nunits;
+        done++;
+        cur = next;
+        haveCur = haveNext;
+        haveNext = false;
+        if (done >= produced) report();
+      }
+      uint64_t drawn = 0;
+      if (threadIdx.x == 0) drawn = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ticket = uniform64(drawn);
     }
     // in a long run of entries let the count move every few entries, so that the
     // leader's window and the producer's ring move while the run is still going
-    ticket = uniform64(pending);
-    __atomic_signal_fence(__ATOMIC_SEQ_CST);
-    if (threadIdx.x == 0) pending = __hip_atomic_fetch_add(mine, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     if (done >= reported + 4) report();
   }
 }
 
-template <typename T, int OP>
+template <typename T, int OP, bool AHEAD>
 __global__ void __launch_bounds__(64) reduceQueueKernel(QueueKernelArgs q) {
   if (blockIdx.x == 0)
     queueLeader(q);
   else
-    queueWorker<T, OP>(q);
+    queueWorker<T, OP, AHEAD>(q);
 }
 
 } // namespace flagcx_amd
