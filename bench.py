@@ -15,7 +15,8 @@ the timed region.  Prints ONE JSON line on stdout:
              with HIP events on the launch stream, against 8 TB/s of HBM3E
   configs    the other benchmark configurations, each with its algorithmic bytes,
              ms per pass, GB/s and fraction of the HBM peak: C1 (2 x fp32 sum, 64 MiB),
-             C3 (fp16 avg reduce-scatter shard: fused, one batch of 32 chunks, chunk
+             C3 (fp16 avg reduce-scatter shard: fused, one batch of 32 chunks, the same
+             batch launched up front and opened chunk by chunk, chunk
              by chunk through the reduce queue, 32 chunk launches), C4 (4 x int32
              max / min), C5 (2-input sum, pack, unpack at 4 KiB, 64 MiB, 1 GiB)
   cpu_baseline  the CPU oracle (a port of the reference's host reduce) timed on
@@ -59,7 +60,7 @@ MiB = 1 << 20
 # (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a copy of
 # known size; not measured by this program.
 TRAFFIC_SOURCE = "profiles/reduce8_bf16_sum_256MiB_pmc.txt"
-TRAFFIC_BYTES = 2415739416
+TRAFFIC_BYTES = 2415742444
 
 
 def log(*a):
@@ -315,6 +316,38 @@ def c3_queue_ms(L, nranks, descs, warmup=5, iters=20):
     return times[len(times) // 2], grid
 
 
+def c3_gated_ms(L, nranks, descs, warmup=5, iters=20):
+    """The shard as ONE batch launched before any chunk is said to be there, its descriptors opened
+    chunk by chunk: host wall clock from the launch call to the end of the stream synchronisation."""
+    import torch
+    lib = L.lib()
+    keep = [(C.c_void_p * nranks)(*d[0]) for d in descs]
+    arr = (L.ReduceDesc * len(descs))(*[L.ReduceDesc(keep[i], d[1], d[2]) for i, d in enumerate(descs)])
+    first = C.c_uint64()
+    side = torch.cuda.Stream()
+    st = L.Stream(side.cuda_stream)
+    times = []
+    torch.cuda.synchronize()
+    lib.flagcxLocalSetMaxSpinCount(1 << 22)
+    gate = L.Gate()
+    try:
+        for it in range(warmup + iters):
+            t0 = time.perf_counter()
+            L.check(lib.flagcxLocalReduceBatchGated(gate._h, arr, len(descs), nranks, int(L.DataType.Float16),
+                                                    int(L.RedOp.Avg), C.byref(st), C.byref(first)))
+            for c in range(len(descs)):
+                lib.flagcxLocalGateOpen(gate._h, first.value + c + 1)
+            side.synchronize()
+            if it >= warmup:
+                times.append((time.perf_counter() - t0) * 1e3)
+        assert gate.query()[2] == 0, "the gated launch gave up waiting"
+    finally:
+        gate.destroy()
+        lib.flagcxLocalSetMaxSpinCount(-1)
+    times.sort()
+    return times[len(times) // 2]
+
+
 def config_c3(L, full=False, separate=False):
     import torch
     nranks, per_rank, shard, send, recv, pool = make_c3(L, separate)
@@ -329,6 +362,9 @@ def config_c3(L, full=False, separate=False):
     ms, grid = c3_queue_ms(L, nranks, descs)
     rows["C3_queue_32x4MiB"] = row(nb, ms, note="chunk by chunk through the resident reduce queue, host wall clock "
                                                 "first enqueue -> Wait; %d resident wavefronts" % grid)
+    ms = c3_gated_ms(L, nranks, descs)
+    rows["C3_gated_batch_32x4MiB"] = row(nb, ms, note="one batch launched up front, a host store per chunk lets its "
+                                                      "wavefronts go; host wall clock launch -> stream sync")
     ms = timed_ms(lambda: L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE))
     rows["C3_per_chunk_launches"] = row(nb, ms, note="32 launches of 4 MiB chunks on one stream, %.2f us per launch"
                                                      % (ms * 1e3 / 32))

@@ -11,7 +11,10 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
 #include <mutex>
+#include <new>
+#include <vector>
 
 namespace flagcx_amd {
 
@@ -200,6 +203,19 @@ ReduceQueueLauncher reduceQueueLauncherFor(int dtype) {
       launchReduceQueue_0, launchReduceQueue_1, launchReduceQueue_2, launchReduceQueue_3,
       launchReduceQueue_4, launchReduceQueue_5, launchReduceQueue_6, launchReduceQueue_7,
       launchReduceQueue_8, launchReduceQueue_9};
+  return (dtype >= 0 && dtype < 10) ? table[dtype] : nullptr;
+}
+
+#define FLAGCX_DECL_GATED(n) int launchReduceGated_##n(const ReduceCall *, int, const GateArgs &);
+FLAGCX_DECL_GATED(0) FLAGCX_DECL_GATED(1) FLAGCX_DECL_GATED(2) FLAGCX_DECL_GATED(3) FLAGCX_DECL_GATED(4)
+FLAGCX_DECL_GATED(5) FLAGCX_DECL_GATED(6) FLAGCX_DECL_GATED(7) FLAGCX_DECL_GATED(8) FLAGCX_DECL_GATED(9)
+#undef FLAGCX_DECL_GATED
+
+ReduceGatedLauncher reduceGatedLauncherFor(int dtype) {
+  static const ReduceGatedLauncher table[10] = {
+      launchReduceGated_0, launchReduceGated_1, launchReduceGated_2, launchReduceGated_3,
+      launchReduceGated_4, launchReduceGated_5, launchReduceGated_6, launchReduceGated_7,
+      launchReduceGated_8, launchReduceGated_9};
   return (dtype >= 0 && dtype < 10) ? table[dtype] : nullptr;
 }
 
@@ -460,6 +476,131 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
     if (r != flagcxSuccess) return r;
   }
   return finish(stream, 0, who);
+}
+
+// ------------------------------------------------------------------ gated batch
+struct flagcxLocalGate {
+  uint64_t *host; // pinned: word 0 = descriptors that may run, word 16 = state
+  uint64_t *dev;  // device copy of word 0
+  std::atomic<uint64_t> launched;
+};
+enum : int { kGateHostCount = 0, kGateHostState = 16 };
+
+flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
+  const char *who = "flagcxLocalGateCreate";
+  if (!gate) return fail(flagcxInvalidArgument, "%s: gate is NULL", who);
+  *gate = nullptr;
+  (void)deviceInfo();
+  flagcxLocalGate *g = new (std::nothrow) flagcxLocalGate;
+  if (!g) return fail(flagcxSystemError, "%s: out of memory", who);
+  g->host = nullptr;
+  g->dev = nullptr;
+  g->launched.store(0);
+  void *h = nullptr, *d = nullptr;
+  hipError_t e = hipHostMalloc(&h, 4096, hipHostMallocMapped);
+  if (e == hipSuccess) e = hipMalloc(&d, 1024);
+  if (e == hipSuccess) e = hipMemset(d, 0, 1024);
+  if (e != hipSuccess) {
+    if (h) (void)hipHostFree(h);
+    if (d) (void)hipFree(d);
+    delete g;
+    return fromHip((int)e, who);
+  }
+  memset(h, 0, 4096);
+  g->host = static_cast<uint64_t *>(h);
+  g->dev = static_cast<uint64_t *>(d);
+  *gate = g;
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalGateDestroy(flagcxLocalGate_t gate) {
+  if (!gate) return flagcxSuccess;
+  // a launch that still waits is abandoned: its workgroups leave without touching data
+  __atomic_store_n(gate->host + kGateHostCount, ~0ull, __ATOMIC_RELEASE);
+  hipError_t e = hipDeviceSynchronize();
+  (void)hipHostFree(gate->host);
+  (void)hipFree(gate->dev);
+  delete gate;
+  return fromHip((int)e, "flagcxLocalGateDestroy");
+}
+
+flagcxResult_t flagcxLocalGateOpen(flagcxLocalGate_t gate, uint64_t upto) {
+  if (!gate) return fail(flagcxInvalidArgument, "flagcxLocalGateOpen: gate is NULL");
+  if (upto == ~0ull) return fail(flagcxInvalidArgument, "flagcxLocalGateOpen: count out of range");
+  if (__atomic_load_n(gate->host + kGateHostState, __ATOMIC_ACQUIRE) != kGateOk)
+    return fail(flagcxInternalError, "flagcxLocalGateOpen: a launch on this gate gave up waiting");
+  // the count only ever rises, whatever order concurrent callers arrive in
+  uint64_t cur = __atomic_load_n(gate->host + kGateHostCount, __ATOMIC_RELAXED);
+  while (cur < upto &&
+         !__atomic_compare_exchange_n(gate->host + kGateHostCount, &cur, upto, false, __ATOMIC_RELEASE, __ATOMIC_RELAXED)) {
+  }
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalGateQuery(flagcxLocalGate_t gate, uint64_t *launched, uint64_t *opened, int *state) {
+  if (!gate) return fail(flagcxInvalidArgument, "flagcxLocalGateQuery: gate is NULL");
+  if (launched) *launched = gate->launched.load();
+  if (opened) *opened = __atomic_load_n(gate->host + kGateHostCount, __ATOMIC_ACQUIRE);
+  if (state) *state = (int)__atomic_load_n(gate->host + kGateHostState, __ATOMIC_ACQUIRE);
+  return flagcxSuccess;
+}
+
+flagcxResult_t flagcxLocalReduceBatchGated(flagcxLocalGate_t gate, const flagcxLocalReduceDesc *descs, int ndescs,
+                                           int nranks, flagcxDataType_t datatype, flagcxRedOp_t op,
+                                           flagcxStream_t stream, uint64_t *first) {
+  const char *who = "flagcxLocalReduceBatchGated";
+  if (!gate) return fail(flagcxInvalidArgument, "%s: gate is NULL", who);
+  if (!stream)
+    return fail(flagcxInvalidArgument, "%s: needs a stream (a blocking call could not return before the gate opens)", who);
+  if (ndescs < 0) return fail(flagcxInvalidArgument, "%s: ndescs %d is negative", who, ndescs);
+  if (ndescs > 0 && !descs) return fail(flagcxInvalidArgument, "%s: descs is NULL", who);
+  if (__atomic_load_n(gate->host + kGateHostState, __ATOMIC_ACQUIRE) != kGateOk)
+    return fail(flagcxInternalError, "%s: a launch on this gate gave up waiting", who);
+  const int dt = bitsOf(datatype), rop = bitsOf(op);
+  const size_t ts = typeSize(dt);
+  hipStream_t hs = hipStreamOf(stream);
+  // everything is checked before the first launch: a launch that has gone out waits for its descriptors
+  std::vector<ReduceCall> calls;
+  std::vector<uint64_t> number;
+  calls.reserve((size_t)ndescs);
+  number.reserve((size_t)ndescs);
+  for (int i = 0; i < ndescs; i++) {
+    const flagcxLocalReduceDesc &d = descs[i];
+    if (!d.sendbuffs) return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs is NULL", who, i);
+    ReduceCall c;
+    bool empty;
+    flagcxResult_t r = prepareReduce(d.sendbuffs, nranks, d.recvbuff, d.count, dt, rop, hs, who, c, &empty);
+    if (r != flagcxSuccess) return r;
+    if (empty) continue;
+    if (nranks > 8) return fail(flagcxInvalidArgument, "%s: takes up to 8 inputs, not %d", who, nranks);
+    for (int j = 0; j < nranks; j++)
+      if ((((uintptr_t)c.src[j] ^ (uintptr_t)c.dst) & 15u) != 0)
+        return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs[%d] and recvbuff differ modulo 16", who, i, j);
+    // descriptors of one launch run concurrently
+    const size_t group = calls.size() / kGateBatchMax * kGateBatchMax;
+    for (size_t e = group; e < calls.size(); e++)
+      if ((uintptr_t)calls[e].dst < (uintptr_t)d.recvbuff + d.count * ts &&
+          (uintptr_t)d.recvbuff < (uintptr_t)calls[e].dst + calls[e].count * ts)
+        return fail(flagcxInvalidArgument, "%s: recvbuff of descs[%d] overlaps an earlier one", who, i);
+    calls.push_back(c);
+    number.push_back((uint64_t)i);
+  }
+  const uint64_t base = gate->launched.fetch_add((uint64_t)ndescs);
+  if (first) *first = base;
+  (void)deviceInfo();
+  for (size_t at = 0; at < calls.size(); at += kGateBatchMax) {
+    const int m = (int)(calls.size() - at < (size_t)kGateBatchMax ? calls.size() - at : (size_t)kGateBatchMax);
+    GateArgs a;
+    a.host = gate->host + kGateHostCount;
+    a.dev = gate->dev;
+    a.hostState = gate->host + kGateHostState;
+    a.maxSpin = asyncMaxSpin();
+    for (int i = 0; i < kGateBatchMax; i++) a.need[i] = base + number[at + (size_t)(i < m ? i : 0)];
+    a.all = a.need[m - 1] + 1;
+    flagcxResult_t r = fromHip(reduceGatedLauncherFor(dt)(calls.data() + at, m, a), who);
+    if (r != flagcxSuccess) return r;
+  }
+  return flagcxSuccess;
 }
 
 flagcxResult_t flagcxLocalReduceTriggers(const flagcxLocalReduceTrigger *triggers, int ntriggers,

@@ -106,6 +106,24 @@ typedef int (*ReduceQueueLauncher)(int op, const QueueKernelArgs &, int wavesPer
 ReduceQueueLauncher reduceQueueLauncherFor(int dtype);
 long long asyncMaxSpin(); // async_kernels.hip
 
+// A batch launched before its inputs have arrived (reduce_gate_device.h): its workgroups
+// wait until the host's count has passed their descriptor's number.
+constexpr int kGateBatchMax = 32; // descriptors per launch, as the plain batch launch
+enum : uint64_t { kGateOk = 0, kGateTimedOut = 1 };
+struct GateArgs {
+  const uint64_t *host; // pinned: descriptors numbered below this count may run
+  uint64_t *dev;        // device copy, only ever raised; ~0 = abandoned
+  uint64_t *hostState;  // pinned: kGate*
+  uint64_t all;         // the launch's leader leaves when the count reaches this
+  int64_t maxSpin;
+  uint64_t need[kGateBatchMax]; // number of each segment's descriptor
+};
+// n <= kGateBatchMax reductions that share k (at most 8), op and stream and whose pointers
+// agree modulo 16 per reduction; need[i] is the number of calls[i].  hipErrorInvalidValue
+// for anything else.
+typedef int (*ReduceGatedLauncher)(const ReduceCall *, int n, const GateArgs &);
+ReduceGatedLauncher reduceGatedLauncherFor(int dtype);
+
 // Byte movers (copy_kernels.hip); all return a hipError_t value.
 struct Copy2D {
   void *dst;

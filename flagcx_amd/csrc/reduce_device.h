@@ -183,6 +183,45 @@ constexpr int kLoadAux = kAuxNt;
 constexpr int kStoreAux = kAuxSc1;
 // Raw buffer descriptor word 3 for gfx9-family: 32-bit data format, no swizzle.
 constexpr int kRsrcFlags = 0x00020000;
+// Accesses that must not be served from a line some cache has held since before the data
+// was written (kernels that start before their inputs are complete): re-fetched and
+// written through at system scope.
+constexpr int kCoherentLoadAux = kAuxSc0 | kAuxSc1 | kAuxNt;
+constexpr int kCoherentStoreAux = kAuxSc0 | kAuxSc1;
+
+// One element read / written at system scope (head and tail elements).
+template <int BYTES> struct UintOf;
+template <> struct UintOf<1> { typedef uint8_t type; };
+template <> struct UintOf<2> { typedef uint16_t type; };
+template <> struct UintOf<4> { typedef uint32_t type; };
+template <> struct UintOf<8> { typedef uint64_t type; };
+
+template <typename T>
+__device__ __forceinline__ T coherentLoad(uint64_t base, uint64_t i) {
+  typedef typename UintOf<sizeof(T)>::type U;
+  const U bits = __hip_atomic_load(reinterpret_cast<const U *>((uintptr_t)base) + i, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_SYSTEM);
+  T out;
+  __builtin_memcpy(&out, &bits, sizeof(T));
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ void coherentStore(uint64_t base, uint64_t i, T v) {
+  typedef typename UintOf<sizeof(T)>::type U;
+  U bits;
+  __builtin_memcpy(&bits, &v, sizeof(T));
+  __hip_atomic_store(reinterpret_cast<U *>((uintptr_t)base) + i, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// As foldScalar, every access at system scope.
+template <typename T, int OP>
+__device__ __forceinline__ void foldScalarCoherent(const void *const *src, int k, void *dst, uint64_t i) {
+  typedef Fold<T, OP> F;
+  typename F::acc_t acc = F::init(coherentLoad<T>((uint64_t)(uintptr_t)src[0], i));
+  for (int j = 1; j < k; j++) acc = F::step(coherentLoad<T>((uint64_t)(uintptr_t)src[j], i), acc);
+  coherentStore<T>((uint64_t)(uintptr_t)dst, i, F::fin(acc, k));
+}
+
 
 // Aligned body with K known at compile time; one wavefront per workgroup.
 // All pointers share the same address modulo 16; p.head elements precede the
@@ -195,8 +234,11 @@ constexpr int kRsrcFlags = 0x00020000;
 // p.run); without it tile = workgroup number from the first body byte on, which is what
 // line-aligned buffers take (the extra scalar work at the start of every short-lived
 // wavefront costs a percent of bandwidth).
-template <typename T, int OP, int K, int U, bool TILED>
+// COHERENT: the inputs were completed while this kernel was already on the GPU; loads are
+// re-fetched at system scope.
+template <typename T, int OP, int K, int U, bool TILED, bool COHERENT = false>
 __device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
+  constexpr int kLoad = COHERENT ? kCoherentLoadAux : kLoadAux;
   constexpr int N = 16 / sizeof(T);
   constexpr uint32_t kTileBytes = 64u * U * 16u;
   const uint64_t bodyBytes = p.nvec * 16;
@@ -230,7 +272,7 @@ __device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
           (void *)((const char *)p.src[j] + headBytes + off), 0, span, kRsrcFlags);
 #pragma unroll
       for (int u = 0; u < U; u++)
-        in[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + u * 1024u, 0, kLoadAux);
+        in[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + u * 1024u, 0, kLoad);
       // K loads issued back to back by every resident wavefront reach DRAM as bursts
       // that thrash the row buffers, worst when the K addresses share a channel
       // group (same bank, K rows).  Waiting until at most inflight-1 earlier inputs
@@ -257,7 +299,8 @@ __device__ __forceinline__ void reduceWaveBody(const ReduceParams<K> &p) {
     const uint64_t edge = p.head + p.tail;
     if (threadIdx.x < edge) {
       uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
-      foldScalar<T, OP>(p.src, K, p.dst, i);
+      if (COHERENT) foldScalarCoherent<T, OP>(p.src, K, p.dst, i);
+      else foldScalar<T, OP>(p.src, K, p.dst, i);
     }
   }
 }

@@ -41,9 +41,6 @@
 
 namespace flagcx_amd {
 
-constexpr int kCoherentLoadAux = kAuxSc0 | kAuxSc1 | kAuxNt;
-constexpr int kCoherentStoreAux = kAuxSc0 | kAuxSc1;
-
 __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
@@ -97,30 +94,6 @@ __device__ __forceinline__ uint64_t laneWord(uint64_t v, int word) {
   const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)v, word);
   const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(v >> 32), word);
   return ((uint64_t)hi << 32) | lo;
-}
-
-// One element read / written at system scope (head and tail elements).
-template <int BYTES> struct UintOf;
-template <> struct UintOf<1> { typedef uint8_t type; };
-template <> struct UintOf<2> { typedef uint16_t type; };
-template <> struct UintOf<4> { typedef uint32_t type; };
-template <> struct UintOf<8> { typedef uint64_t type; };
-
-template <typename T>
-__device__ __forceinline__ T coherentLoad(uint64_t base, uint64_t i) {
-  typedef typename UintOf<sizeof(T)>::type U;
-  const U bits = __hip_atomic_load(reinterpret_cast<const U *>((uintptr_t)base) + i, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_SYSTEM);
-  T out;
-  __builtin_memcpy(&out, &bits, sizeof(T));
-  return out;
-}
-template <typename T>
-__device__ __forceinline__ void coherentStore(uint64_t base, uint64_t i, T v) {
-  typedef typename UintOf<sizeof(T)>::type U;
-  U bits;
-  __builtin_memcpy(&bits, &v, sizeof(T));
-  __hip_atomic_store(reinterpret_cast<U *>((uintptr_t)base) + i, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 __device__ inline void queueLeader(const QueueKernelArgs &q) {

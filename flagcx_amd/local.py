@@ -120,6 +120,8 @@ EXPORTS = [
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
     "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
     "flagcxLocalReduceBatch", "flagcxLocalReduceTriggers",
+    "flagcxLocalGateCreate", "flagcxLocalGateDestroy", "flagcxLocalReduceBatchGated", "flagcxLocalGateOpen",
+    "flagcxLocalGateQuery",
     "flagcxLocalFifoInit", "flagcxLocalFifoDestroy", "flagcxLocalFifoDequeue", "flagcxLocalP2pDemo",
     "flagcxLocalRingCreate", "flagcxLocalRingDestroy", "flagcxLocalRingSendRecv",
     "flagcxLocalRingReduceScatter",
@@ -208,6 +210,11 @@ def lib():
         L.flagcxLocalReduceFifoEnqueue.argtypes = [vp, C.POINTER(ReduceTrigger), u64p]
         L.flagcxLocalReduceFifoEnqueueReduce.argtypes = [vp, pp, i, vp, sz, u64p]
         L.flagcxLocalReduceFifoQuery.argtypes = [vp, u64p, u64p, C.POINTER(i)]
+        L.flagcxLocalGateCreate.argtypes = [pp]
+        L.flagcxLocalGateDestroy.argtypes = [vp]
+        L.flagcxLocalReduceBatchGated.argtypes = [vp, C.POINTER(ReduceDesc), i, i, i, i, sp, u64p]
+        L.flagcxLocalGateOpen.argtypes = [vp, C.c_uint64]
+        L.flagcxLocalGateQuery.argtypes = [vp, u64p, u64p, C.POINTER(i)]
         L.flagcxLocalReduceFifoWait.argtypes = [vp, C.c_uint64]
         L.flagcxLocalReduceFifoGetGrid.argtypes = [vp, C.POINTER(C.c_uint)]
         L.flagcxLocalReduceFifoSetWaves.argtypes = [vp, i]
@@ -473,6 +480,46 @@ class Ring:
             self.close()
         except Exception:
             pass
+
+
+class Gate:
+    """A count that the host raises as the inputs of a gated batch complete (flagcxLocalGate*)."""
+
+    def __init__(self):
+        self._h = C.c_void_p()
+        check(lib().flagcxLocalGateCreate(C.byref(self._h)))
+
+    def reduce_batch(self, descs, op, dtype, nranks, stream="current"):
+        """descs as reduce_batch; launched now, folded as open() passes each descriptor's number.
+        Returns the number of descs[0]."""
+        st = current_stream() if stream == "current" else stream
+        keep = [_ptr_array(list(d[0])) for d in descs]
+        arr = (ReduceDesc * len(descs))(*[ReduceDesc(keep[i], d[1], d[2]) for i, d in enumerate(descs)])
+        first = C.c_uint64()
+        check(lib().flagcxLocalReduceBatchGated(self._h, arr, len(descs), nranks, int(dtype), int(op), _sref(st),
+                                                C.byref(first)))
+        return first.value
+
+    def open(self, upto):
+        check(lib().flagcxLocalGateOpen(self._h, upto))
+
+    def query(self):
+        """(descriptors numbered so far, count, state)."""
+        a, b, st = C.c_uint64(), C.c_uint64(), C.c_int()
+        check(lib().flagcxLocalGateQuery(self._h, C.byref(a), C.byref(b), C.byref(st)))
+        return a.value, b.value, st.value
+
+    def destroy(self):
+        if self._h:
+            h, self._h = self._h, C.c_void_p()
+            check(lib().flagcxLocalGateDestroy(h))
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.destroy()
+        return False
 
 
 class ReduceFifo:

@@ -1,10 +1,11 @@
 // fifo_perf.cpp - C++ timing driver for the host-producer / device-consumer reduce
 // queue (flagcxLocalReduceFifo*), beside the launch-per-chunk and batched forms of
-// the same work:
+// the same work, and the batch launched up front with its descriptors opened one by one:
 //
 //   fifo_perf [-k nranks] [-t dtype] [-o op] [-c chunkbytes] [-m nchunks] [-w warmup] [-n iters]
 //             [-W wavesPerCU] [-L lingerPolls] [-s spinLimit] [-q ringCapacity]
 //             [-D windowBytes] [-a separateAllocations] [-g arrivalGapUs] [-x bytesIntoTheBuffers]
+//             [-T wavesPerCUOfLaunchedKernels] [-I inputsInFlightOfLaunchedKernels]
 //
 // A shard of nchunks x chunkbytes per input (default 32 x 4 MiB: the reference's
 // staging step, FLAGCX_P2P_CHUNKSIZE, flagcx/core/p2p.h:11-15) is reduced chunk by
@@ -69,6 +70,7 @@ int main(int argc, char **argv) {
   double gapUs = 0.0;
   size_t shift = 0; // -x: every buffer starts this many bytes further on (positions inside cache lines)
   size_t window = 0;
+  int launchWaves = -1, launchLoads = -1; // -T, -I: flagcxLocalTune / flagcxLocalTuneLoads for the launched kernels
   for (int i = 1; i + 1 < argc; i += 2) {
     const char *f = argv[i], *v = argv[i + 1];
     if (!strcmp(f, "-k")) k = atoi(v);
@@ -86,12 +88,16 @@ int main(int argc, char **argv) {
     else if (!strcmp(f, "-a")) separate = atoi(v);
     else if (!strcmp(f, "-g")) gapUs = atof(v);
     else if (!strcmp(f, "-x")) shift = strtoull(v, 0, 0);
+    else if (!strcmp(f, "-T")) launchWaves = atoi(v);
+    else if (!strcmp(f, "-I")) launchLoads = atoi(v);
   }
   flagcxLocalReduceFifo_t fifo = nullptr;
   const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dtype);
   if (!ts || k < 1 || k > 8 || nchunks < 1 || chunkBytes % ts) return 2;
   FX(flagcxLocalInit());
   flagcxLocalSetMaxSpinCount(spin); // an idle consumer leaves after this many polls
+  if (launchWaves >= 0) FX(flagcxLocalTune(k, launchWaves));
+  if (launchLoads >= 0) FX(flagcxLocalTuneLoads(k, launchLoads));
   const size_t shardBytes = chunkBytes * (size_t)nchunks;
   const size_t chunkCount = chunkBytes / ts;
   // the k inputs and the output in one allocation, in different HBM channel groups
@@ -158,6 +164,32 @@ int main(int argc, char **argv) {
     if (it >= warmup) t.push_back(nowUs() - t0);
   }
   printf("%-46s %10.1f us  %8.1f GB/s\n", "one batch call (all chunks present), sync", median(t), algo / median(t) / 1e3);
+
+  // (2b) the same batch launched up front, its descriptors opened chunk by chunk.  With -g the
+  // launch precedes the first arrival (that is what it is for); without, it is inside the time.
+  {
+    flagcxLocalGate_t gate = nullptr;
+    FX(flagcxLocalGateCreate(&gate));
+    t.clear();
+    for (int it = 0; it < warmup + iters; it++) {
+      uint64_t first = 0;
+      double t0 = nowUs();
+      FX(flagcxLocalReduceBatchGated(gate, descs.data(), nchunks, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op, &st,
+                                     &first));
+      if (gapUs > 0) t0 = nowUs();
+      for (int c = 0; c < nchunks; c++) {
+        arrive(t0, c);
+        FX(flagcxLocalGateOpen(gate, first + (uint64_t)c + 1));
+      }
+      CK(hipStreamSynchronize(st.base));
+      if (it >= warmup) t.push_back(nowUs() - t0);
+    }
+    int gateState = 0;
+    FX(flagcxLocalGateQuery(gate, nullptr, nullptr, &gateState));
+    printf("%-46s %10.1f us  %8.1f GB/s%s\n", "gated batch launched up front, Open per chunk", median(t),
+           algo / median(t) / 1e3, gateState ? "  (GAVE UP WAITING)" : "");
+    FX(flagcxLocalGateDestroy(gate));
+  }
 
   // (3) the resident consumer: enqueue chunk by chunk, wait for the last ticket
   FX(flagcxLocalReduceFifoCreate(&fifo, capacity, k, (flagcxDataType_t)dtype, (flagcxRedOp_t)op));

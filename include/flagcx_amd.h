@@ -244,6 +244,46 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
                                       int nranks, flagcxDataType_t datatype,
                                       flagcxRedOp_t op, flagcxStream_t stream);
 
+/* The same batch, launched BEFORE its inputs have arrived: the pipeline chunks of a
+ * collective are known when it starts, only their arrival times are not.  Where the
+ * reference's proxy would fold a chunk each time a receive completes (the loop
+ * that such completions drive: flagcx/core/proxy.cc:1074-1182), the caller enqueues
+ * the whole list once and then calls flagcxLocalGateOpen as chunks complete: the
+ * wavefronts of descriptor i wait on the GPU, read nothing, until the gate's count
+ * has passed i's number.  One ordinary launch per 32 descriptors, at the rate of
+ * flagcxLocalReduceBatch, and a chunk's fold starts about 2 us after its Open.
+ *
+ * Descriptors get consecutive numbers per gate, from 0 at creation: this call's are
+ * *first .. *first + ndescs - 1 (first may be NULL).  Open(upto) lets every
+ * descriptor numbered below `upto` run; the count only rises, so chunks must be
+ * opened in order (or as far as a contiguous prefix has arrived), and a count may
+ * be opened before the launch that it belongs to.  Inputs must be complete in
+ * device memory before their Open (an event or stream the caller has synchronised
+ * with); results are read after the stream has been synchronised.
+ * Restrictions (flagcxInvalidArgument otherwise): a non-NULL stream, nranks <= 8,
+ * and within one descriptor every sendbuff agrees with recvbuff modulo 16 bytes.
+ * Waiting wavefronts hold CU slots (up to half of every CU's) and most of the LDS:
+ * a kernel that produces the inputs must not need the LDS they hold.
+ * The wait is bounded: when the count has not moved for
+ * FLAGCX_FUNC_MAX_SPIN_COUNT polls (flagcxLocalSetMaxSpinCount; default 2^27,
+ * minutes) the launch gives up, every wavefront that still waits leaves without
+ * touching data, and the gate's state becomes 1 for good: later launches on it
+ * are refused.  Create and Destroy allocate and synchronise (setup time);
+ * Destroy abandons launches that still wait.  Open and Query touch pinned host
+ * memory only and may be called from any thread. */
+typedef struct flagcxLocalGate *flagcxLocalGate_t;
+#define FLAGCX_LOCAL_GATE_OK 0
+#define FLAGCX_LOCAL_GATE_TIMED_OUT 1
+flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate);
+flagcxResult_t flagcxLocalGateDestroy(flagcxLocalGate_t gate);
+flagcxResult_t flagcxLocalReduceBatchGated(flagcxLocalGate_t gate, const flagcxLocalReduceDesc *descs,
+                                           int ndescs, int nranks, flagcxDataType_t datatype,
+                                           flagcxRedOp_t op, flagcxStream_t stream, uint64_t *first);
+flagcxResult_t flagcxLocalGateOpen(flagcxLocalGate_t gate, uint64_t upto);
+/* Descriptors numbered so far, the count, and the state (any pointer may be NULL). */
+flagcxResult_t flagcxLocalGateQuery(flagcxLocalGate_t gate, uint64_t *launched, uint64_t *opened,
+                                    int *state);
+
 /* Consumer of the reference's reduce descriptor, which is declared but has no
  * producer or consumer there (flagcxReduceTrigger, flagcx/include/flagcx_kernel.h:30-35,
  * 52-73; host-producer API commented out at :96-98).  Same 256-bit layout:
