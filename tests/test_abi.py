@@ -24,6 +24,22 @@ def declared_symbols():
     return sorted(names)
 
 
+def test_headers_are_plain_c(tmp_path):
+    """The boundary is a C ABI: both headers compile as C99 (and as C++11) with nothing but the C library."""
+    import shutil
+    import subprocess
+    src = '#include "flagcx_amd.h"\n#include "flagcx_amd_adaptor.h"\nint main(void) { return (int)flagcxSuccess; }\n'
+    inc = os.path.join(ROOT, "include")
+    for cc, name, std in (("gcc", "t.c", "-std=c99"), ("g++", "t.cpp", "-std=c++11")):
+        if not shutil.which(cc):
+            pytest.skip(cc + " not installed")
+        f = tmp_path / name
+        f.write_text(src)
+        r = subprocess.run([cc, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I", inc, str(f)],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+
+
 def test_library_exports_every_declared_symbol():
     L = local.lib()
     names = declared_symbols()
