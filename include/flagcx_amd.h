@@ -264,6 +264,8 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
  * and within one descriptor every sendbuff agrees with recvbuff modulo 16 bytes.
  * Waiting wavefronts hold CU slots (up to half of every CU's) and most of the LDS:
  * a kernel that produces the inputs must not need the LDS they hold.
+ * Work on another stream may be queued behind a launch that waits (streams share
+ * hardware queues): never make an Open depend on the completion of such work.
  * The wait is bounded: when the count has not moved for
  * FLAGCX_FUNC_MAX_SPIN_COUNT polls (flagcxLocalSetMaxSpinCount; default 2^27,
  * minutes) the launch gives up, every wavefront that still waits leaves without
