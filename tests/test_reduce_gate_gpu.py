@@ -232,3 +232,42 @@ def test_gated_batch_argument_errors(L):
         with torch.cuda.stream(side):
             assert gate.reduce_batch([], op, dt, 2) == 0
         side.synchronize()
+
+
+def test_c3_shard_streamed_through_the_gate(L):
+    """8 ranks x 1 GiB fp16, N(0, sigma = 0.01); rank 3's 128 MiB shard as 32 descriptors of 4 MiB in ring
+    order, launched up front and opened one by one: the same bytes as the one-launch reduce-scatter, and a
+    window of them against the oracle."""
+    import torch
+    MiB = 1 << 20
+    nranks, per_rank = 8, 512 * MiB
+    shard = per_rank // nranks
+    send = []
+    for r in range(nranks):
+        g = torch.Generator(device="cuda").manual_seed(100 + r)
+        buf = torch.empty(per_rank, dtype=torch.float16, device="cuda")
+        for s in range(nranks):
+            buf[s * shard:(s + 1) * shard] = (torch.randn(shard, generator=g, device="cuda") * 0.01).to(torch.float16)
+        send.append(buf)
+    rank = 3
+    fused = torch.empty(shard, dtype=torch.float16, device="cuda")
+    gated = torch.zeros(shard, dtype=torch.float16, device="cuda")
+    L.reduce_scatter(send, rank, fused, L.RedOp.Avg)
+    chunk = L.CHUNKSIZE // 2
+    descs = [([send[(rank + 1 + j) % nranks].data_ptr() + (rank * shard + c * chunk) * 2 for j in range(nranks)],
+              gated.data_ptr() + c * chunk * 2, chunk) for c in range(shard // chunk)]
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with L.Gate() as gate:
+        with torch.cuda.stream(side):
+            first = gate.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks)
+        for c in range(len(descs)):
+            gate.open(first + c + 1)
+        side.synchronize()
+        assert gate.query() == (len(descs), len(descs), OK)
+    equal = bool(torch.equal(fused.view(torch.int16), gated.view(torch.int16)))
+    assert equal
+    w0, w1 = 5 * MiB + 3, 6 * MiB + 3
+    win = [send[(rank + 1 + j) % nranks][rank * shard + w0:rank * shard + w1].cpu().numpy() for j in range(nranks)]
+    rc, want = O.reduce(win, O.FP16, O.AVG)
+    assert rc == 0 and same(gated[w0:w1].cpu().numpy(), want)
