@@ -25,7 +25,7 @@ def L():
     assert torch.cuda.is_available()
     from flagcx_amd import local
     assert local.lib().flagcxLocalInit() == 0
-    local.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+    local.lib().flagcxLocalSetMaxSpinCount(1 << 21)  # seconds: far above any pause of the host between two calls
     yield local
     local.lib().flagcxLocalSetMaxSpinCount(-1)
 
@@ -172,9 +172,9 @@ def test_gated_launch_gives_up_when_nothing_opens(L):
     L.lib().flagcxLocalSetMaxSpinCount(2000)
     try:
         gate = L.Gate()
+        gate.open(1)  # the first descriptor may run (opened before the launch, so no host timing is involved), the others never arrive
         with torch.cuda.stream(side):
             gate.reduce_batch([([d.data_ptr() for d in devs], o.data_ptr(), n) for o in outs], op, dt, k)
-        gate.open(1)  # the first descriptor runs, the others never arrive
         side.synchronize()
         assert gate.query() == (3, 1, TIMED_OUT)
         assert same(from_dev(outs[0], ins[0].dtype), expect(ins, dt, op), nan_class=True, dtype=dt)
@@ -188,7 +188,7 @@ def test_gated_launch_gives_up_when_nothing_opens(L):
         assert e.value.code == L.Result.InternalError
         gate.destroy()
     finally:
-        L.lib().flagcxLocalSetMaxSpinCount(1 << 19)
+        L.lib().flagcxLocalSetMaxSpinCount(1 << 21)
 
 
 def test_gate_destroy_abandons_a_waiting_launch(L):
