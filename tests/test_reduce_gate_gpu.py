@@ -271,3 +271,29 @@ def test_c3_shard_streamed_through_the_gate(L):
     win = [send[(rank + 1 + j) % nranks][rank * shard + w0:rank * shard + w1].cpu().numpy() for j in range(nranks)]
     rc, want = O.reduce(win, O.FP16, O.AVG)
     assert rc == 0 and same(gated[w0:w1].cpu().numpy(), want)
+
+
+def test_gate_opened_from_another_thread(L):
+    """The proxy's shape: one thread launches and synchronises, another one raises the count as chunks complete."""
+    import threading
+    import torch
+    dt, op, k, n, chunks = O.FP32, O.SUM, 4, 1 << 16, 48
+    ins = make_inputs(dt, k, n * chunks, seed=21, op=op)
+    devs = [to_dev(a) for a in ins]
+    out = dev_empty(n * chunks, 4, fill=0x55)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with L.Gate() as gate:
+        def proxy():
+            for c in range(chunks):
+                time.sleep(0.0002)
+                gate.open(c + 1)
+        t = threading.Thread(target=proxy)
+        with torch.cuda.stream(side):
+            gate.reduce_batch([([d.data_ptr() + c * n * 4 for d in devs], out.data_ptr() + c * n * 4, n)
+                               for c in range(chunks)], op, dt, k)
+        t.start()
+        side.synchronize()
+        t.join()
+        assert gate.query() == (chunks, chunks, OK)
+    assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
