@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstring>
 #include <atomic>
+#include <map>
 #include <mutex>
 #include <new>
 #include <vector>
@@ -482,9 +483,39 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
 struct flagcxLocalGate {
   uint64_t *host; // pinned: word 0 = descriptors that may run, word 16 = state
   uint64_t *dev;  // device copy of word 0
+  bool uncached;  // dev comes from the pool of uncached words below
+  int device;
   std::atomic<uint64_t> launched;
 };
 enum : int { kGateHostCount = 0, kGateHostState = 16 };
+
+// Device words in uncached memory, 128 bytes apart, for the gates' counts: wavefronts read
+// them through the scalar path, which sees memory only if no cache keeps the line.  Such
+// memory is never given back to the runtime (freeing uncached memory that kernels have read
+// has been seen to corrupt later allocations on this platform): words of destroyed gates
+// are handed to the next gate on the same device, pages stay until the process ends.
+static std::mutex gGateWordsMutex;
+static std::map<int, std::vector<uint64_t *>> gGateWords;
+
+static uint64_t *takeUncachedWord(int device) {
+  std::lock_guard<std::mutex> lock(gGateWordsMutex);
+  std::vector<uint64_t *> &pool = gGateWords[device];
+  if (pool.empty()) {
+    void *page = nullptr;
+    if (hipExtMallocWithFlags(&page, 4096, hipDeviceMallocUncached) != hipSuccess || !page) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    for (int i = 0; i < 4096 / 128; i++) pool.push_back(static_cast<uint64_t *>(page) + i * 16);
+  }
+  uint64_t *w = pool.back();
+  pool.pop_back();
+  return w;
+}
+static void returnUncachedWord(int device, uint64_t *w) {
+  std::lock_guard<std::mutex> lock(gGateWordsMutex);
+  gGateWords[device].push_back(w);
+}
 
 flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
   const char *who = "flagcxLocalGateCreate";
@@ -496,13 +527,21 @@ flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
   g->host = nullptr;
   g->dev = nullptr;
   g->launched.store(0);
+  g->device = 0;
+  g->uncached = false;
   void *h = nullptr, *d = nullptr;
-  hipError_t e = hipHostMalloc(&h, 4096, hipHostMallocMapped);
-  if (e == hipSuccess) e = hipMalloc(&d, 1024);
-  if (e == hipSuccess) e = hipMemset(d, 0, 1024);
+  hipError_t e = hipGetDevice(&g->device);
+  if (e == hipSuccess) e = hipHostMalloc(&h, 4096, hipHostMallocMapped);
+  if (e == hipSuccess) {
+    d = takeUncachedWord(g->device);
+    g->uncached = d != nullptr;
+    if (!d) e = hipMalloc(&d, 128); // wavefronts then read the count with vector loads
+  }
+  if (e == hipSuccess) e = hipMemset(d, 0, 128);
   if (e != hipSuccess) {
     if (h) (void)hipHostFree(h);
-    if (d) (void)hipFree(d);
+    if (d && g->uncached) returnUncachedWord(g->device, static_cast<uint64_t *>(d));
+    else if (d) (void)hipFree(d);
     delete g;
     return fromHip((int)e, who);
   }
@@ -519,7 +558,8 @@ flagcxResult_t flagcxLocalGateDestroy(flagcxLocalGate_t gate) {
   __atomic_store_n(gate->host + kGateHostCount, ~0ull, __ATOMIC_RELEASE);
   hipError_t e = hipDeviceSynchronize();
   (void)hipHostFree(gate->host);
-  (void)hipFree(gate->dev);
+  if (gate->uncached) returnUncachedWord(gate->device, gate->dev);
+  else (void)hipFree(gate->dev);
   delete gate;
   return fromHip((int)e, "flagcxLocalGateDestroy");
 }
@@ -595,6 +635,7 @@ flagcxResult_t flagcxLocalReduceBatchGated(flagcxLocalGate_t gate, const flagcxL
     a.dev = gate->dev;
     a.hostState = gate->host + kGateHostState;
     a.maxSpin = asyncMaxSpin();
+    a.scalarRead = gate->uncached ? 1 : 0;
     for (int i = 0; i < kGateBatchMax; i++) a.need[i] = base + number[at + (size_t)(i < m ? i : 0)];
     a.all = a.need[m - 1] + 1;
     flagcxResult_t r = fromHip(reduceGatedLauncherFor(dt)(calls.data() + at, m, a), who);

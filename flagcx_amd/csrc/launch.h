@@ -116,6 +116,7 @@ struct GateArgs {
   uint64_t *hostState;  // pinned: kGate*
   uint64_t all;         // the launch's leader leaves when the count reaches this
   int64_t maxSpin;
+  uint64_t scalarRead;  // dev is uncached device memory: the first read of a wavefront goes through the scalar path
   uint64_t need[kGateBatchMax]; // number of each segment's descriptor
 };
 // n <= kGateBatchMax reductions that share k (at most 8), op and stream and whose pointers

@@ -14,10 +14,13 @@
 // Workgroups are dispatched in order, descriptor after descriptor, so those that wait hold
 // wavefront slots only behind the ones that can run, and a grid dispatched tile by tile
 // keeps the rate of the plain batch launch (a resident grid that draws its tiles by
-// ticket stays 5 to 7 % below it).  One read of the device word costs nothing measurable;
-// an acquire fence behind it would cost tens of microseconds per wavefront (cache-wide
-// maintenance), so coherence is per access, as in the reduce queue: data loads carry
-// sc0 sc1 and are issued only after the count has been seen.
+// ticket stays 5 to 7 % below it).  The read of the device word in front of a wavefront's
+// loads is what the gate costs: 5 to 11 % as a vector load (whatever its scope: it queues
+// behind the CU's streaming loads), 3 to 4 % as a scalar load, which is how the first look
+// is taken when the word could be placed in uncached memory.  An acquire fence behind the
+// read would cost tens of microseconds per wavefront (cache-wide maintenance), so coherence
+// is per access, as in the reduce queue: data loads carry sc0 sc1 and are issued only after
+// the count has been seen.
 //
 // Every wait is bounded: the leader gives up after maxSpin polls without a change of the
 // host's count, marks the gate abandoned (device word ~0, state word in pinned memory) and
@@ -59,8 +62,16 @@ __device__ __forceinline__ uint64_t gateLead(const GateArgs &g) {
 __device__ __forceinline__ bool gateWait(const GateArgs &g, uint64_t need) {
   for (int64_t spins = 0;;) {
     uint64_t v = 0;
-    if (threadIdx.x == 0) v = agentLoad(g.dev);
-    v = uniform64(v);
+    if (g.scalarRead && spins == 0) {
+      // One 8-byte scalar load that bypasses the scalar cache.  The word lives in uncached
+      // device memory, so what comes back is what memory holds; the scalar path does not
+      // queue behind the CU's streaming vector loads, which is what a vector read of the
+      // count costs (3 to 8 % of the launch's rate).  Only the first look takes it.
+      asm volatile("s_load_dwordx2 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(g.dev) : "memory");
+    } else {
+      if (threadIdx.x == 0) v = agentLoad(g.dev);
+      v = uniform64(v);
+    }
     if (v == ~0ull) return false;
     if (v > need) return true;
     // the leader's bound comes first; this one only ends a workgroup whose leader is gone

@@ -345,14 +345,18 @@ static int launchGatedFixed(const ReduceCall *calls, const Split *splits, int n,
     totalTiles += tiles;
   }
   if (maxTiles > kMaxGrid) maxTiles = kMaxGrid;
-  // Every wavefront reads the gate's count before its loads, about a microsecond in which
-  // it holds its slot without traffic: more resident wavefronts than the plain batch launch
-  // make up for part of it.  Measured, 128 chunks of 4 MiB per input, TB/s with the plain
-  // batch's shape -> with this one (the plain batch itself): 2 inputs 5.63 -> 6.13 (6.53),
-  // 3: 5.39 -> 6.26 (6.43), 4: 5.63 -> 6.33 (6.69), 6: 5.84 -> 6.22 (6.68), 8: 6.10 -> 6.35 (6.71).
+  // Every wavefront reads the gate's count before its loads and holds its slot without
+  // traffic meanwhile: somewhat more resident wavefronts than the plain batch launch make
+  // up for part of it.  Measured, 128 chunks of 4 MiB per input, TB/s: vector read with the
+  // plain batch's shape -> vector read with its own shape -> scalar read with its own shape
+  // (the plain batch itself): 2 inputs 5.63 -> 6.13 -> 6.19 (6.53), 3: 5.39 -> 6.26 -> 6.33
+  // (6.43), 4: 5.63 -> 6.33 -> 6.45 (6.65), 6: 5.84 -> 6.22 -> 6.44 (6.68), 8: 6.10 -> 6.35
+  // -> 6.47 (6.69); shards of 32 chunks gain more from the scalar read (2 inputs 5.9 -> 6.4).
   LaunchShape shape = launchShapeFor(K, totalTiles);
   if (K <= 3) shape.loads = 0;
-  if (tunedWavesPerCU(K) < 0) shape.waves = K <= 3 ? 0 : K <= 5 ? 21 : 18;
+  if (tunedWavesPerCU(K) < 0)
+    shape.waves = g.scalarRead ? (K == 1 ? 0 : K == 2 ? 25 : K == 3 ? 21 : K <= 5 ? 18 : 16)
+                               : (K <= 3 ? 0 : K <= 5 ? 21 : 18);
   for (int i = 0; i < n; i++) bp.seg[i].inflight = shape.loads;
   for (int i = n; i < FLAGCX_BATCH_MAX; i++) bp.seg[i] = bp.seg[0];
   const int lds = ldsReservation(shape.waves);
