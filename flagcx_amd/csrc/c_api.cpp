@@ -533,7 +533,10 @@ flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
   hipError_t e = hipGetDevice(&g->device);
   if (e == hipSuccess) e = hipHostMalloc(&h, 4096, hipHostMallocMapped);
   if (e == hipSuccess) {
-    d = takeUncachedWord(g->device);
+    // FLAGCX_LOCAL_GATE_CACHED=1: keep the count in ordinary device memory (vector reads), as on a
+    // device that has no uncached memory to give
+    const char *cached = getenv("FLAGCX_LOCAL_GATE_CACHED");
+    d = (cached && cached[0] == '1') ? nullptr : takeUncachedWord(g->device);
     g->uncached = d != nullptr;
     if (!d) e = hipMalloc(&d, 128); // wavefronts then read the count with vector loads
   }

@@ -297,3 +297,27 @@ def test_gate_opened_from_another_thread(L):
         t.join()
         assert gate.query() == (chunks, chunks, OK)
     assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
+
+
+def test_gate_with_its_count_in_ordinary_device_memory(L, monkeypatch):
+    """The fallback for devices without uncached memory: vector reads of the count, same bytes."""
+    import torch
+    monkeypatch.setenv("FLAGCX_LOCAL_GATE_CACHED", "1")
+    dt, op, k = O.BF16, O.SUM, 8
+    counts = [5, 4097, (1 << 18) + 3, 1 << 20]
+    ins = [make_inputs(dt, k, n, seed=700 + i, op=op) for i, n in enumerate(counts)]
+    devs = [[to_dev(a) for a in group] for group in ins]
+    outs = [dev_empty(n, 2, fill=0x55) for n in counts]
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with L.Gate() as gate:
+        with torch.cuda.stream(side):
+            gate.reduce_batch([([d.data_ptr() for d in devs[i]], outs[i].data_ptr(), counts[i])
+                               for i in range(len(counts))], op, dt, k)
+        for upto in range(1, len(counts) + 1):
+            time.sleep(0.001)
+            gate.open(upto)
+        side.synchronize()
+        assert gate.query() == (len(counts), len(counts), OK)
+    for i, n in enumerate(counts):
+        assert same(from_dev(outs[i], ins[i][0].dtype), expect(ins[i], dt, op), nan_class=True, dtype=dt), n
