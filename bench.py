@@ -391,6 +391,8 @@ def config_c3(L, full=False, separate=False):
                                                 hbm_gbps=round(staged / ms / 1e6, 1))
         L.lib().flagcxLocalSetMaxSpinCount(1 << 22)
         fifo = L.ReduceFifo(64, nranks, L.DataType.Float16, L.RedOp.Avg)
+        # a hardware queue of its own for the consumer: the copy stream must never wait behind it
+        fifo.set_own_queue(True)
         torch.cuda.synchronize()
         with fifo:
             for _ in range(5):

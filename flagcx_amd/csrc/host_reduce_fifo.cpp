@@ -424,6 +424,37 @@ flagcxResult_t flagcxLocalReduceFifoSetLinger(flagcxLocalReduceFifo_t q, int64_t
   return flagcxSuccess;
 }
 
+flagcxResult_t flagcxLocalReduceFifoSetOwnQueue(flagcxLocalReduceFifo_t q, int own) {
+  const char *who = "flagcxLocalReduceFifoSetOwnQueue";
+  if (!q) return flagcxInvalidArgument;
+  std::lock_guard<std::mutex> lock(q->mu);
+  if (q->started) return qfail(q, flagcxInvalidUsage, "%s: the queue is started", who);
+  // A stream with a CU mask does not come from the runtime's pool of hardware queues (the
+  // mask is a property of the queue): with every CU in the mask it differs from an ordinary
+  // stream only in that no other stream is ever mapped to its hardware queue, and in that
+  // the runtime creates such streams blocking.
+  hipStream_t fresh = nullptr;
+  hipError_t e;
+  if (own) {
+    uint32_t mask[32];
+    for (int i = 0; i < 32; i++) mask[i] = 0xffffffffu;
+    int words = (deviceInfo().numCU + 31) / 32;
+    if (words < 1) words = 1;
+    if (words > 32) words = 32;
+    e = hipExtStreamCreateWithCUMask(&fresh, (uint32_t)words, mask);
+  } else {
+    e = hipStreamCreateWithFlags(&fresh, hipStreamNonBlocking);
+  }
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return qfail(q, flagcxUnhandledDeviceError, "%s: %s", who, hipGetErrorString(e));
+  }
+  (void)hipStreamSynchronize(q->stream);
+  (void)hipStreamDestroy(q->stream);
+  q->stream = fresh;
+  return flagcxSuccess;
+}
+
 flagcxResult_t flagcxLocalReduceFifoSetWindow(flagcxLocalReduceFifo_t q, size_t bytes) {
   if (!q) return flagcxInvalidArgument;
   std::lock_guard<std::mutex> lock(q->mu);

@@ -131,7 +131,7 @@ EXPORTS = [
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
-    "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoSetLinger", "flagcxLocalReduceFifoSetWindow", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
+    "flagcxLocalReduceFifoSetWaves", "flagcxLocalReduceFifoSetLinger", "flagcxLocalReduceFifoSetOwnQueue", "flagcxLocalReduceFifoSetWindow", "flagcxLocalReduceFifoGetType", "flagcxLocalRingReduceScatterFifo",
     "flagcxLocalReduceFifoGetLastError", "flagcxLocalStagedReduceScatterNoAlloc",
 ]
 
@@ -210,6 +210,7 @@ def lib():
         L.flagcxLocalReduceFifoEnqueue.argtypes = [vp, C.POINTER(ReduceTrigger), u64p]
         L.flagcxLocalReduceFifoEnqueueReduce.argtypes = [vp, pp, i, vp, sz, u64p]
         L.flagcxLocalReduceFifoQuery.argtypes = [vp, u64p, u64p, C.POINTER(i)]
+        L.flagcxLocalReduceFifoSetOwnQueue.argtypes = [vp, i]
         L.flagcxLocalGateCreate.argtypes = [pp]
         L.flagcxLocalGateDestroy.argtypes = [vp]
         L.flagcxLocalReduceBatchGated.argtypes = [vp, C.POINTER(ReduceDesc), i, i, i, i, sp, u64p]
@@ -583,6 +584,10 @@ class ReduceFifo:
 
     def set_window(self, nbytes):
         self._check(lib().flagcxLocalReduceFifoSetWindow(self._h, nbytes))
+
+    def set_own_queue(self, own=True):
+        """A hardware queue of its own for the consumer (its stream then is a blocking one)."""
+        self._check(lib().flagcxLocalReduceFifoSetOwnQueue(self._h, 1 if own else 0))
 
     def set_linger(self, polls):
         self._check(lib().flagcxLocalReduceFifoSetLinger(self._h, polls))

@@ -497,6 +497,15 @@ flagcxResult_t flagcxLocalReduceFifoGetType(flagcxLocalReduceFifo_t fifo, flagcx
 flagcxResult_t flagcxLocalReduceFifoSetWindow(flagcxLocalReduceFifo_t fifo, size_t bytes);
 /* Idle polls before the consumer parks (0: never).  Not between Start and Stop. */
 flagcxResult_t flagcxLocalReduceFifoSetLinger(flagcxLocalReduceFifo_t fifo, int64_t polls);
+/* own != 0: the consumer gets a hardware queue that no other stream is mapped to, so that
+ * no launch on any stream ever waits behind it (the runtime spreads ordinary streams over a
+ * few hardware queues, four per process here, and work on a stream that lands on the
+ * consumer's waits until the consumer parks).  The price: such a stream is a blocking one,
+ * i.e. work on the NULL stream and the consumer wait for each other.  For callers that
+ * keep their work on non-blocking streams of their own, as the reference's proxies do
+ * (flagcx/core/proxy.cc:1094-1097); leave it off where the NULL stream is in use (PyTorch's
+ * default stream is).  Default off.  Not between Start and Stop. */
+flagcxResult_t flagcxLocalReduceFifoSetOwnQueue(flagcxLocalReduceFifo_t fifo, int own);
 /* Workgroups (one wavefront each) of the running consumer: 1 leader + workers. */
 flagcxResult_t flagcxLocalReduceFifoGetGrid(flagcxLocalReduceFifo_t fifo, unsigned *workgroups);
 const char *flagcxLocalReduceFifoGetLastError(flagcxLocalReduceFifo_t fifo);

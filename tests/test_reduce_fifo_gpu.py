@@ -430,3 +430,51 @@ def test_fifo_chunked_shard_matches_single_launch(L):
     sample = slice(0, 4096)
     want = expect([d[sample].view(torch.int16).cpu().numpy().view(np.float16) for d in devs], dt, op)
     assert same(piecewise[sample].view(torch.int16).cpu().numpy().view(np.float16), want, nan_class=True, dtype=dt)
+
+
+def test_consumer_on_a_queue_of_its_own_holds_no_stream_up(L):
+    """With flagcxLocalReduceFifoSetOwnQueue no stream shares the consumer's hardware queue: launches on many
+    other streams finish while a consumer that never parks sits on the GPU.  (Without it some of these
+    streams would wait until the consumer leaves, here at its spin bound, seconds later.)"""
+    import time
+    import torch
+    dt, op, n = O.FP32, O.SUM, 4096
+    ins = make_inputs(dt, 2, n, seed=77, op=op)
+    devs = [to_dev(a) for a in ins]
+    out = dev_empty(n, 4, fill=0)
+    others = [torch.cuda.Stream() for _ in range(12)]
+    work = [torch.zeros(1024, dtype=torch.int32, device="cuda") for _ in others]
+    torch.cuda.synchronize()
+    q = L.ReduceFifo(8, 2, dt, op)
+    try:
+        q.set_linger(0)
+        q.set_own_queue(True)
+        with q:
+            q.wait(q.enqueue_reduce([d.data_ptr() for d in devs], out.data_ptr(), n))
+            t0 = time.perf_counter()
+            for s, w in zip(others, work):
+                with torch.cuda.stream(s):
+                    w.add_(1)
+                s.synchronize()
+            elapsed = time.perf_counter() - t0
+            assert q.query()[2] == RUNNING
+        assert elapsed < 0.25, elapsed
+    finally:
+        q.close()
+    assert all(int(w[0].item()) == 1 for w in work)
+    assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
+    # switching back gives an ordinary stream again, and the queue still works
+    q = L.ReduceFifo(8, 2, dt, op)
+    try:
+        q.set_own_queue(True)
+        q.set_own_queue(False)
+        out.zero_()
+        torch.cuda.synchronize()
+        with q:
+            q.wait(q.enqueue_reduce([d.data_ptr() for d in devs], out.data_ptr(), n))
+            with pytest.raises(L.FlagcxError) as e:
+                q.set_own_queue(True)
+            assert e.value.code == L.Result.InvalidUsage
+    finally:
+        q.close()
+    assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
