@@ -485,6 +485,8 @@ struct flagcxLocalGate {
   uint64_t *dev;  // device copy of word 0
   bool uncached;  // dev comes from the pool of uncached words below
   int device;
+  std::mutex mu;
+  hipStream_t own; // created on request: a stream with a hardware queue of its own; its address is the flagcxStream_t handed out
   std::atomic<uint64_t> launched;
 };
 enum : int { kGateHostCount = 0, kGateHostState = 16 };
@@ -529,6 +531,7 @@ flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
   g->launched.store(0);
   g->device = 0;
   g->uncached = false;
+  g->own = nullptr;
   void *h = nullptr, *d = nullptr;
   hipError_t e = hipGetDevice(&g->device);
   if (e == hipSuccess) e = hipHostMalloc(&h, 4096, hipHostMallocMapped);
@@ -560,11 +563,33 @@ flagcxResult_t flagcxLocalGateDestroy(flagcxLocalGate_t gate) {
   // a launch that still waits is abandoned: its workgroups leave without touching data
   __atomic_store_n(gate->host + kGateHostCount, ~0ull, __ATOMIC_RELEASE);
   hipError_t e = hipDeviceSynchronize();
+  if (gate->own) (void)hipStreamDestroy(gate->own);
   (void)hipHostFree(gate->host);
   if (gate->uncached) returnUncachedWord(gate->device, gate->dev);
   else (void)hipFree(gate->dev);
   delete gate;
   return fromHip((int)e, "flagcxLocalGateDestroy");
+}
+
+flagcxResult_t flagcxLocalGateOwnStream(flagcxLocalGate_t gate, flagcxStream_t *stream) {
+  const char *who = "flagcxLocalGateOwnStream";
+  if (!gate || !stream) return fail(flagcxInvalidArgument, "%s: NULL argument", who);
+  std::lock_guard<std::mutex> lock(gate->mu);
+  if (!gate->own) {
+    // a CU mask (every CU set) takes the stream out of the runtime's pool of hardware queues
+    uint32_t mask[32];
+    for (int i = 0; i < 32; i++) mask[i] = 0xffffffffu;
+    int words = (deviceInfo().numCU + 31) / 32;
+    if (words < 1) words = 1;
+    if (words > 32) words = 32;
+    hipStream_t s = nullptr;
+    const hipError_t e = hipExtStreamCreateWithCUMask(&s, (uint32_t)words, mask);
+    if (e != hipSuccess) return fromHip((int)e, who);
+    gate->own = s;
+  }
+  // the stream wrapper's first member is the hipStream_t (hipStreamOf above)
+  *stream = reinterpret_cast<flagcxStream_t>(&gate->own);
+  return flagcxSuccess;
 }
 
 flagcxResult_t flagcxLocalGateOpen(flagcxLocalGate_t gate, uint64_t upto) {

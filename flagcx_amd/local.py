@@ -121,7 +121,7 @@ EXPORTS = [
     "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
     "flagcxLocalReduceBatch", "flagcxLocalReduceTriggers",
     "flagcxLocalGateCreate", "flagcxLocalGateDestroy", "flagcxLocalReduceBatchGated", "flagcxLocalGateOpen",
-    "flagcxLocalGateQuery",
+    "flagcxLocalGateQuery", "flagcxLocalGateOwnStream",
     "flagcxLocalFifoInit", "flagcxLocalFifoDestroy", "flagcxLocalFifoDequeue", "flagcxLocalP2pDemo",
     "flagcxLocalRingCreate", "flagcxLocalRingDestroy", "flagcxLocalRingSendRecv",
     "flagcxLocalRingReduceScatter",
@@ -216,6 +216,7 @@ def lib():
         L.flagcxLocalReduceBatchGated.argtypes = [vp, C.POINTER(ReduceDesc), i, i, i, i, sp, u64p]
         L.flagcxLocalGateOpen.argtypes = [vp, C.c_uint64]
         L.flagcxLocalGateQuery.argtypes = [vp, u64p, u64p, C.POINTER(i)]
+        L.flagcxLocalGateOwnStream.argtypes = [vp, C.POINTER(sp)]
         L.flagcxLocalReduceFifoWait.argtypes = [vp, C.c_uint64]
         L.flagcxLocalReduceFifoGetGrid.argtypes = [vp, C.POINTER(C.c_uint)]
         L.flagcxLocalReduceFifoSetWaves.argtypes = [vp, i]
@@ -503,6 +504,12 @@ class Gate:
 
     def open(self, upto):
         check(lib().flagcxLocalGateOpen(self._h, upto))
+
+    def own_stream(self):
+        """The gate's stream (a Stream structure): a hardware queue that nothing else shares."""
+        p = C.POINTER(Stream)()
+        check(lib().flagcxLocalGateOwnStream(self._h, C.byref(p)))
+        return p.contents
 
     def query(self):
         """(descriptors numbered so far, count, state)."""

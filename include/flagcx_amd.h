@@ -287,6 +287,14 @@ flagcxResult_t flagcxLocalReduceBatchGated(flagcxLocalGate_t gate, const flagcxL
                                            int ndescs, int nranks, flagcxDataType_t datatype,
                                            flagcxRedOp_t op, flagcxStream_t stream, uint64_t *first);
 flagcxResult_t flagcxLocalGateOpen(flagcxLocalGate_t gate, uint64_t upto);
+/* A stream that belongs to the gate (valid until Destroy) and has a hardware queue that no
+ * other stream is mapped to: a gated launch on it can hold up nothing else.  The runtime
+ * spreads ordinary streams over a few hardware queues (four per process here), so with
+ * more streams alive than that, the stream whose work completes the chunks may sit behind
+ * the very launch that waits for them, which then ends in the spin bound.  Launch gated
+ * batches here unless the caller controls how many streams the process holds.  It is a
+ * blocking stream: NULL-stream work and the launch wait for each other. */
+flagcxResult_t flagcxLocalGateOwnStream(flagcxLocalGate_t gate, flagcxStream_t *stream);
 /* Descriptors numbered so far, the count, and the state (any pointer may be NULL). */
 flagcxResult_t flagcxLocalGateQuery(flagcxLocalGate_t gate, uint64_t *launched, uint64_t *opened,
                                     int *state);

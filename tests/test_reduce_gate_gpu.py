@@ -321,3 +321,37 @@ def test_gate_with_its_count_in_ordinary_device_memory(L, monkeypatch):
         assert gate.query() == (len(counts), len(counts), OK)
     for i, n in enumerate(counts):
         assert same(from_dev(outs[i], ins[i][0].dtype), expect(ins[i], dt, op), nan_class=True, dtype=dt), n
+
+
+def test_gated_launch_on_the_gates_own_stream_holds_nothing_up(L):
+    """The pipeline the gate is for, in a process that holds many streams: each chunk's inputs are
+    produced by copies on one of 12 other streams, then the chunk is opened.  On the gate's own stream
+    the waiting launch shares its hardware queue with none of them, so no copy can end up behind it."""
+    import torch
+    dt, op, k, n, chunks = O.FP32, O.SUM, 3, 1 << 15, 24
+    ins = make_inputs(dt, k, n * chunks, seed=31, op=op)
+    staged = [to_dev(a) for a in ins]                       # where the producers read
+    devs = [dev_empty(n * chunks, 4, fill=0) for _ in range(k)]  # where the reductions read
+    out = dev_empty(n * chunks, 4, fill=0x55)
+    others = [torch.cuda.Stream() for _ in range(12)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    with L.Gate() as gate:
+        st = gate.own_stream()
+        gate.reduce_batch([([d.data_ptr() + c * n * 4 for d in devs], out.data_ptr() + c * n * 4, n)
+                           for c in range(chunks)], op, dt, k, stream=st)
+        for c in range(chunks):
+            s = others[(5 * c) % len(others)]
+            with torch.cuda.stream(s):
+                for j in range(k):
+                    devs[j][c * n:(c + 1) * n].copy_(staged[j][c * n:(c + 1) * n])
+            s.synchronize()
+            gate.open(c + 1)
+        assert L.lib().flagcxLocalGateOwnStream(gate._h, None) == L.Result.InvalidArgument
+        import ctypes as C
+        # the device adaptor's streamSynchronize, as the reference would synchronise a flagcxStream_t
+        sync = L.adaptor_fn(L.device_adaptor()[1], "streamSynchronize", C.c_int, C.c_void_p)
+        assert sync(C.addressof(st)) == 0
+        assert gate.query() == (chunks, chunks, OK)
+    assert time.perf_counter() - t0 < 1.0
+    assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
