@@ -123,3 +123,87 @@ def test_tuning_overrides_belong_to_the_calling_thread():
     assert seen == {"tuner": (25, 1), "other": (-1, -1), "tuner_after": (25, 1)}
     w = C.c_int(-2)
     assert lib.flagcxLocalGetTune(8, C.byref(w)) == 0 and w.value == -1     # and the main thread was never touched
+
+
+@pytest.mark.gpu
+def test_queue_gate_and_plain_launches_side_by_side():
+    """The three ways into the reduce at once, each from its own thread: entries through the resident queue
+    (on a hardware queue of its own), gated batches on the gate's own stream opened chunk by chunk, and plain
+    launches on an ordinary stream.  Whatever the runtime's mapping of streams to hardware queues, neither of
+    the two kernels that wait on the GPU can hold the third thread's stream up for good, and every result is
+    the oracle's."""
+    import time
+    import torch
+    from flagcx_amd import local as L
+    assert L.lib().flagcxLocalInit() == 0
+    L.lib().flagcxLocalSetMaxSpinCount(1 << 21)
+    n, rounds = 1 << 16, 12
+    mk = lambda dt, op, k, seed: make_inputs(dt, k, n * rounds, seed=seed, op=op)
+    qi, gi, pi = mk(O.FP16, O.AVG, 8, 1), mk(O.FP32, O.SUM, 3, 2), mk(O.INT32, O.MAX, 4, 3)
+    qd, gd, pd = ([to_dev(a) for a in x] for x in (qi, gi, pi))
+    qo, go, po = dev_empty(n * rounds, 2, fill=0), dev_empty(n * rounds, 4, fill=0), dev_empty(n * rounds, 4, fill=0)
+    plain = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    errors = []
+    barrier = threading.Barrier(3)
+
+    def through_queue():
+        try:
+            q = L.ReduceFifo(16, 8, O.FP16, O.AVG)
+            try:
+                q.set_own_queue(True)
+                with q:
+                    barrier.wait()
+                    t = 0
+                    for r in range(rounds):
+                        t = q.enqueue_reduce([d.data_ptr() + r * n * 2 for d in qd], qo.data_ptr() + r * n * 2, n)
+                        time.sleep(0.0005)
+                    q.wait(t)
+            finally:
+                q.close()
+        except Exception as e:
+            errors.append(("queue", repr(e)))
+
+    def through_gate():
+        try:
+            with L.Gate() as gate:
+                st = gate.own_stream()
+                barrier.wait()
+                first = gate.reduce_batch([([d.data_ptr() + r * n * 4 for d in gd], go.data_ptr() + r * n * 4, n)
+                                           for r in range(rounds)], O.SUM, O.FP32, 3, stream=st)
+                for r in range(rounds):
+                    time.sleep(0.0005)
+                    gate.open(first + r + 1)
+                import ctypes as C
+                sync = L.adaptor_fn(L.device_adaptor()[1], "streamSynchronize", C.c_int, C.c_void_p)
+                assert sync(C.addressof(st)) == 0
+                assert gate.query()[2] == 0
+        except Exception as e:
+            errors.append(("gate", repr(e)))
+
+    def plain_launches():
+        try:
+            st = L.Stream(plain.cuda_stream)
+            barrier.wait()
+            for r in range(rounds):
+                L.reduce([d[r * n:(r + 1) * n] for d in pd], po[r * n:(r + 1) * n], O.MAX, dtype=O.INT32, stream=st)
+                time.sleep(0.0005)
+            plain.synchronize()
+        except Exception as e:
+            errors.append(("plain", repr(e)))
+
+    threads = [threading.Thread(target=f) for f in (through_queue, through_gate, plain_launches)]
+    try:
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join(60)
+    finally:
+        L.lib().flagcxLocalSetMaxSpinCount(-1)
+    assert not errors, errors
+    assert not any(th.is_alive() for th in threads)
+    torch.cuda.synchronize()
+    for ins, out, dt, op in ((qi, qo, O.FP16, O.AVG), (gi, go, O.FP32, O.SUM), (pi, po, O.INT32, O.MAX)):
+        rc, want = O.reduce(ins, dt, op)
+        assert rc == 0
+        assert same(from_dev(out, ins[0].dtype), want, nan_class=dt != O.INT32, dtype=dt), (dt, op)
