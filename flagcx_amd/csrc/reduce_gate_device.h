@@ -84,6 +84,15 @@ __device__ __forceinline__ bool gateWait(const GateArgs &g, uint64_t need) {
 
 template <typename T, int OP, int K, int U>
 __global__ void __launch_bounds__(64) reduceGatedBatchKernel(ReduceBatchParams<K> bp, GateArgs g) {
+  if (blockIdx.x != 0 || blockIdx.y != 0) {
+    // a workgroup beyond its segment's tiles, with no head or tail elements to fold either,
+    // has nothing to wait for (segments of one launch may differ in size)
+    const ReduceParams<K> &p = bp.seg[blockIdx.y];
+    constexpr uint64_t kTileBytes = 64ull * U * 16ull;
+    uint64_t tiles = (p.nvec * 16 + p.lead + kTileBytes - 1) / kTileBytes;
+    if (p.run > 1) tiles = (tiles + 8ull * p.run - 1) / (8ull * p.run) * (8ull * p.run);
+    if (blockIdx.x >= tiles && blockIdx.x != gridDim.x - 1) return;
+  }
   bool open;
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     // the leader's own tile is folded last, if its descriptor has been opened at all
