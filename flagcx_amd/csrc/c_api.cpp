@@ -484,6 +484,7 @@ struct flagcxLocalGate {
   uint64_t *host; // pinned: word 0 = descriptors that may run, word 16 = state
   uint64_t *dev;  // device copy of word 0
   bool uncached;  // dev comes from the pool of uncached words below
+  uint64_t offset; // what both counts started at: the numbers the caller sees are relative to it
   int device;
   std::mutex mu;
   hipStream_t own; // created on request: a stream with a hardware queue of its own; its address is the flagcxStream_t handed out
@@ -496,25 +497,33 @@ enum : int { kGateHostCount = 0, kGateHostState = 16 };
 // memory is never given back to the runtime (freeing uncached memory that kernels have read
 // has been seen to corrupt later allocations on this platform): words of destroyed gates
 // are handed to the next gate on the same device, pages stay until the process ends.
+// A word that is used again goes on counting where its last gate stopped (`floor`), and a
+// word that was left at the abandon mark is never used again: whatever an earlier read may
+// have left anywhere, a value seen for a word is then never above what its gate has opened.
+struct GateWord {
+  uint64_t *ptr;
+  uint64_t floor;
+};
 static std::mutex gGateWordsMutex;
-static std::map<int, std::vector<uint64_t *>> gGateWords;
+static std::map<int, std::vector<GateWord>> gGateWords;
 
-static uint64_t *takeUncachedWord(int device) {
+static GateWord takeUncachedWord(int device) {
   std::lock_guard<std::mutex> lock(gGateWordsMutex);
-  std::vector<uint64_t *> &pool = gGateWords[device];
+  std::vector<GateWord> &pool = gGateWords[device];
   if (pool.empty()) {
     void *page = nullptr;
-    if (hipExtMallocWithFlags(&page, 4096, hipDeviceMallocUncached) != hipSuccess || !page) {
+    if (hipExtMallocWithFlags(&page, 4096, hipDeviceMallocUncached) != hipSuccess || !page ||
+        hipMemset(page, 0, 4096) != hipSuccess) {
       (void)hipGetLastError();
-      return nullptr;
+      return GateWord{nullptr, 0}; // (a page that could not be cleared is not handed out, nor freed)
     }
-    for (int i = 0; i < 4096 / 128; i++) pool.push_back(static_cast<uint64_t *>(page) + i * 16);
+    for (int i = 0; i < 4096 / 128; i++) pool.push_back(GateWord{static_cast<uint64_t *>(page) + i * 16, 0});
   }
-  uint64_t *w = pool.back();
+  const GateWord w = pool.back();
   pool.pop_back();
   return w;
 }
-static void returnUncachedWord(int device, uint64_t *w) {
+static void returnUncachedWord(int device, GateWord w) {
   std::lock_guard<std::mutex> lock(gGateWordsMutex);
   gGateWords[device].push_back(w);
 }
@@ -531,6 +540,7 @@ flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
   g->launched.store(0);
   g->device = 0;
   g->uncached = false;
+  g->offset = 0;
   g->own = nullptr;
   void *h = nullptr, *d = nullptr;
   hipError_t e = hipGetDevice(&g->device);
@@ -539,20 +549,27 @@ flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
     // FLAGCX_LOCAL_GATE_CACHED=1: keep the count in ordinary device memory (vector reads), as on a
     // device that has no uncached memory to give
     const char *cached = getenv("FLAGCX_LOCAL_GATE_CACHED");
-    d = (cached && cached[0] == '1') ? nullptr : takeUncachedWord(g->device);
+    const GateWord w = (cached && cached[0] == '1') ? GateWord{nullptr, 0} : takeUncachedWord(g->device);
+    d = w.ptr;
     g->uncached = d != nullptr;
-    if (!d) e = hipMalloc(&d, 128); // wavefronts then read the count with vector loads
+    g->offset = w.floor;
+    if (!d) {
+      e = hipMalloc(&d, 128); // wavefronts then read the count with vector loads
+      if (e == hipSuccess) e = hipMemset(d, 0, 128);
+    } else {
+      e = hipMemcpy(d, &g->offset, sizeof(uint64_t), hipMemcpyHostToDevice);
+    }
   }
-  if (e == hipSuccess) e = hipMemset(d, 0, 128);
   if (e != hipSuccess) {
     if (h) (void)hipHostFree(h);
-    if (d && g->uncached) returnUncachedWord(g->device, static_cast<uint64_t *>(d));
+    if (d && g->uncached) returnUncachedWord(g->device, GateWord{static_cast<uint64_t *>(d), g->offset});
     else if (d) (void)hipFree(d);
     delete g;
     return fromHip((int)e, who);
   }
   memset(h, 0, 4096);
   g->host = static_cast<uint64_t *>(h);
+  g->host[kGateHostCount] = g->offset;
   g->dev = static_cast<uint64_t *>(d);
   *gate = g;
   return flagcxSuccess;
@@ -561,12 +578,22 @@ flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {
 flagcxResult_t flagcxLocalGateDestroy(flagcxLocalGate_t gate) {
   if (!gate) return flagcxSuccess;
   // a launch that still waits is abandoned: its workgroups leave without touching data
-  __atomic_store_n(gate->host + kGateHostCount, ~0ull, __ATOMIC_RELEASE);
+  const uint64_t opened = __atomic_exchange_n(gate->host + kGateHostCount, ~0ull, __ATOMIC_ACQ_REL);
   hipError_t e = hipDeviceSynchronize();
   if (gate->own) (void)hipStreamDestroy(gate->own);
+  if (gate->uncached) {
+    // the word goes back with the highest count it can have held, unless a leader has left
+    // the abandon mark in it (or it cannot be read): then it is not used again
+    uint64_t last = ~0ull;
+    if (hipMemcpy(&last, gate->dev, sizeof(last), hipMemcpyDeviceToHost) != hipSuccess) (void)hipGetLastError();
+    uint64_t floor = gate->offset + gate->launched.load();
+    if (opened != ~0ull && opened > floor) floor = opened;
+    if (last != ~0ull && opened != ~0ull)
+      returnUncachedWord(gate->device, GateWord{gate->dev, last > floor ? last : floor});
+  } else {
+    (void)hipFree(gate->dev);
+  }
   (void)hipHostFree(gate->host);
-  if (gate->uncached) returnUncachedWord(gate->device, gate->dev);
-  else (void)hipFree(gate->dev);
   delete gate;
   return fromHip((int)e, "flagcxLocalGateDestroy");
 }
@@ -597,10 +624,12 @@ flagcxResult_t flagcxLocalGateOpen(flagcxLocalGate_t gate, uint64_t upto) {
   if (upto == ~0ull) return fail(flagcxInvalidArgument, "flagcxLocalGateOpen: count out of range");
   if (__atomic_load_n(gate->host + kGateHostState, __ATOMIC_ACQUIRE) != kGateOk)
     return fail(flagcxInternalError, "flagcxLocalGateOpen: a launch on this gate gave up waiting");
+  if (upto > ~0ull - 1 - gate->offset) return fail(flagcxInvalidArgument, "flagcxLocalGateOpen: count out of range");
+  const uint64_t target = gate->offset + upto;
   // the count only ever rises, whatever order concurrent callers arrive in
   uint64_t cur = __atomic_load_n(gate->host + kGateHostCount, __ATOMIC_RELAXED);
-  while (cur < upto &&
-         !__atomic_compare_exchange_n(gate->host + kGateHostCount, &cur, upto, false, __ATOMIC_RELEASE, __ATOMIC_RELAXED)) {
+  while (cur < target &&
+         !__atomic_compare_exchange_n(gate->host + kGateHostCount, &cur, target, false, __ATOMIC_RELEASE, __ATOMIC_RELAXED)) {
   }
   return flagcxSuccess;
 }
@@ -608,7 +637,7 @@ flagcxResult_t flagcxLocalGateOpen(flagcxLocalGate_t gate, uint64_t upto) {
 flagcxResult_t flagcxLocalGateQuery(flagcxLocalGate_t gate, uint64_t *launched, uint64_t *opened, int *state) {
   if (!gate) return fail(flagcxInvalidArgument, "flagcxLocalGateQuery: gate is NULL");
   if (launched) *launched = gate->launched.load();
-  if (opened) *opened = __atomic_load_n(gate->host + kGateHostCount, __ATOMIC_ACQUIRE);
+  if (opened) *opened = __atomic_load_n(gate->host + kGateHostCount, __ATOMIC_ACQUIRE) - gate->offset;
   if (state) *state = (int)__atomic_load_n(gate->host + kGateHostState, __ATOMIC_ACQUIRE);
   return flagcxSuccess;
 }
@@ -664,7 +693,7 @@ flagcxResult_t flagcxLocalReduceBatchGated(flagcxLocalGate_t gate, const flagcxL
     a.hostState = gate->host + kGateHostState;
     a.maxSpin = asyncMaxSpin();
     a.scalarRead = gate->uncached ? 1 : 0;
-    for (int i = 0; i < kGateBatchMax; i++) a.need[i] = base + number[at + (size_t)(i < m ? i : 0)];
+    for (int i = 0; i < kGateBatchMax; i++) a.need[i] = gate->offset + base + number[at + (size_t)(i < m ? i : 0)];
     a.all = a.need[m - 1] + 1;
     flagcxResult_t r = fromHip(reduceGatedLauncherFor(dt)(calls.data() + at, m, a), who);
     if (r != flagcxSuccess) return r;

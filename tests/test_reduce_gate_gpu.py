@@ -355,3 +355,26 @@ def test_gated_launch_on_the_gates_own_stream_holds_nothing_up(L):
         assert gate.query() == (chunks, chunks, OK)
     assert time.perf_counter() - t0 < 1.0
     assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
+
+
+def test_numbers_start_at_zero_for_every_gate(L):
+    """A gate's device word comes from a pool and goes on counting where its last gate stopped; the numbers a
+    caller sees do not: each gate numbers its descriptors from 0 and reports its own count."""
+    import torch
+    dt, op, k, n = O.INT32, O.SUM, 2, 4099
+    ins = make_inputs(dt, k, n, seed=41, op=op)
+    devs = [to_dev(a) for a in ins]
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for round_ in range(3):
+        out = dev_empty(n, 4, fill=0x55)
+        torch.cuda.synchronize()
+        with L.Gate() as gate:
+            assert gate.query() == (0, 0, OK)
+            with torch.cuda.stream(side):
+                first = gate.reduce_batch([([d.data_ptr() for d in devs], out.data_ptr(), n)] * 1, op, dt, k)
+            assert first == 0
+            gate.open(1 + round_)          # beyond what was launched: allowed
+            side.synchronize()
+            assert gate.query() == (1, 1 + round_, OK)
+        assert same(from_dev(out, np.int32), expect(ins, dt, op), dtype=dt)
