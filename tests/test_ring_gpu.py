@@ -106,6 +106,8 @@ def test_ring_reduce_scatter_through_the_reduce_queue(L, dt, op, nranks, rcount,
     L.lib().flagcxLocalSetMaxSpinCount(1 << 19)
     q = L.ReduceFifo(8, nranks, dt, op)
     try:
+        # the copy stream must not sit behind the consumer, however many streams this process has made before
+        q.set_own_queue(True)
         with q:
             for rep in range(2):
                 for rank in staged:
@@ -160,6 +162,7 @@ def test_ring_fifo_returns_when_the_consumer_has_left(L):
     torch.cuda.synchronize()
     q = L.ReduceFifo(8, nranks, dt, op)
     try:
+        q.set_own_queue(True)  # the copy stream never waits behind the consumer
         # the spin bound is reached long before the idle limit at which a consumer parks
         L.lib().flagcxLocalSetMaxSpinCount(1)
         q.start()
