@@ -298,16 +298,18 @@ static flagcxResult_t prepareReduce(const void *const *srcs, int k, void *dst, u
   c.k = k;
   c.op = op;
   c.stream = stream;
+  c.anyOrder = 0;
   *empty = false;
   return flagcxSuccess;
 }
 
 static flagcxResult_t reduceOrdered(const void *const *srcs, int k, void *dst, uint64_t count,
-                                    int dtype, int op, hipStream_t stream, const char *who) {
+                                    int dtype, int op, hipStream_t stream, const char *who, bool anyOrder = false) {
   ReduceCall c;
   bool empty;
   flagcxResult_t r = prepareReduce(srcs, k, dst, count, dtype, op, stream, who, c, &empty);
   if (r != flagcxSuccess || empty) return r;
+  c.anyOrder = anyOrder ? 1 : 0;
   (void)deviceInfo();
   return fromHip(reduceLauncherFor(dtype)(c), who);
 }
@@ -778,7 +780,10 @@ static flagcxResult_t reduceScatterImpl(const void *const *sendbuffs, int nranks
       const int r = (rank + 1 + j) % nranks;
       ordered[j] = (const char *)sendbuffs[r] + ((size_t)rank * recvcount + done) * ts;
     }
-    flagcxResult_t res = reduceOrdered(ordered, nranks, (char *)recvbuff + done * ts, n, dt, rop, hs, who);
+    // the chunks of one call are independent of each other: from the second on, a launch may start
+    // while its predecessor drains (the first waits for whatever the stream held before, the launch
+    // after the call for all of them)
+    flagcxResult_t res = reduceOrdered(ordered, nranks, (char *)recvbuff + done * ts, n, dt, rop, hs, who, done > 0);
     if (res != flagcxSuccess) return res;
     done += n;
   } while (done < recvcount);

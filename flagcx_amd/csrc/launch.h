@@ -17,6 +17,7 @@ struct ReduceCall {
   int k;
   int op;         // flagcxRedOp_t value
   hipStream_t stream;
+  int anyOrder;   // this launch need not wait for the launch before it on the stream to finish (chunks of one call)
 };
 
 // Cached per-process facts about the device the library runs on.

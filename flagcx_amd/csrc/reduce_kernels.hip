@@ -2,6 +2,7 @@
 // and provides its launcher.  Compiled once per type with -DFLAGCX_DT=<enum value>
 // so the ten types build in parallel.
 #include "launch.h"
+#include <hip/hip_ext.h>
 #include "reduce_device.h"
 #include "reduce_queue_device.h"
 #include "reduce_gate_device.h"
@@ -127,10 +128,18 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   if (p.run > 1) tiles = (tiles + 8ull * p.run - 1) / (8ull * p.run) * (8ull * p.run);
   if (tiles > kMaxGrid) tiles = kMaxGrid;
   const int lds = ldsReservation(shape.waves);
-  if (p.lead == 0 && p.run == 1)
+  if (c.anyOrder) {
+    if (p.lead == 0 && p.run == 1)
+      hipExtLaunchKernelGGL((reduceWaveKernel<elem_t, OP, K, U, false>), dim3((unsigned)tiles), dim3(64), lds, c.stream,
+                            nullptr, nullptr, hipExtAnyOrderLaunch, p);
+    else
+      hipExtLaunchKernelGGL((reduceWaveKernel<elem_t, OP, K, U, true>), dim3((unsigned)tiles), dim3(64), lds, c.stream,
+                            nullptr, nullptr, hipExtAnyOrderLaunch, p);
+  } else if (p.lead == 0 && p.run == 1) {
     reduceWaveKernel<elem_t, OP, K, U, false><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
-  else
+  } else {
     reduceWaveKernel<elem_t, OP, K, U, true><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
+  }
   return (int)hipGetLastError();
 }
 

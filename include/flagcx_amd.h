@@ -209,7 +209,10 @@ flagcxResult_t flagcxLocalReduceScatter(const void *const *sendbuffs, int nranks
 /* The same result produced chunk by chunk, the way the staging ring hands data
  * over (4 MiB steps, flagcx/core/p2p.cc:81-94): one launch per `chunkbytes` of
  * output.  chunkbytes == 0 selects FLAGCX_LOCAL_CHUNKSIZE; it must be a multiple of
- * the element size. */
+ * the element size.  The chunks of one call do not depend on one another: from the
+ * second on, a launch may start while its predecessor drains (the first still waits
+ * for what the stream held before the call, and what follows the call for all of
+ * them). */
 flagcxResult_t flagcxLocalReduceScatterChunked(const void *const *sendbuffs,
                                                int nranks, int rank,
                                                void *recvbuff, size_t recvcount,
