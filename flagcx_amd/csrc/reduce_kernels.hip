@@ -212,7 +212,8 @@ static int launchShift(const ReduceCall &c, const Split &s) {
   // 128 / 512 MiB per input: 1 input (a misaligned copy) 66 / 77 / 81, 2: 71 / 80 / 83,
   // 3: 70-75 / 80-82 / 83-84, 4: 74-76 / 81 / 84, 6: 75 / 80-82 / 81, 8: 74-76 / 79 / 77-78
   // (tile = workgroup number, two tiles per wavefront: 62-65 / 73-76 / 69-80).
-  // Wavefronts per CU: no cap / 25 / 21 / 14 for up to 2 / 3 / 4 / up to 6 inputs; 7 and 8
+  // Wavefronts per CU: no cap / 25 / 21 / 18 / 14 for up to 2 / 3 / 4 / 5 / 6 inputs (5 inputs at 18 instead of 14:
+  // 72 / 80 / 79 -> 75 / 80 / 83); 7 and 8
   // keep two sources in flight per wavefront at 16, which holds 77-79 % from 128 MiB to
   // 1 GiB where all at once falls to 70-73 %.
   constexpr uint64_t span = 8ull * kShiftRun;
@@ -222,7 +223,7 @@ static int launchShift(const ReduceCall &c, const Split &s) {
   const int loads = tunedLoadsInFlight(K);
   p.inflight = loads >= 0 ? (loads == 2 ? 2 : 0) : K >= 7 ? 2 : 0;
   const int tuned = tunedWavesPerCU(K);
-  const int lds = ldsReservation(tuned >= 0 ? tuned : K <= 2 ? 0 : K == 3 ? 25 : K == 4 ? 21 : K <= 6 ? 14 : 16);
+  const int lds = ldsReservation(tuned >= 0 ? tuned : K <= 2 ? 0 : K == 3 ? 25 : K == 4 ? 21 : K == 5 ? 18 : K == 6 ? 14 : 16);
   reduceWaveShiftKernel<elem_t, OP, K><<<dim3((unsigned)grid), dim3(64), lds, c.stream>>>(p);
   return (int)hipGetLastError();
 }
