@@ -90,21 +90,26 @@ const DeviceInfo &deviceInfo() {
 //  - below that, launches are a few rounds of wavefronts long and want many of
 //    them resident whatever the layout (4 inputs of 16 MiB: 5.2 TB/s at 11 per CU,
 //    5.7-5.8 at 25; 8 inputs of 8 MiB: 5.2 at 8, 5.6-5.7 at 16-25).
+//  - in between (32 .. 88 MiB per input) the best shape changes with the size; the rows come from
+//    sweeps over both layouts (percent of peak, old -> new row): 3 inputs of 32 / 64 / 80 MiB 74 /
+//    80-82 / 82 -> 78 / 84-86 / 87; 4 of 32 / 64 MiB 76 / 81 -> 78-79 / 82.5-83; 5 of 32 / 64 / 80 MiB 77 / 81 / 82-83 ->
+//    79 / 81-83 / 84; 6 of 64 / 80 MiB 83 / 84 -> 84.5 / 84.7; 7 of 64 / 80 MiB 81 / 82 -> 83-84 /
+//    84.5; 8 of 48 / 64 / 80 MiB 81 / 82.4-83.5 / 83 -> 83 / 83.5-84 / 84-85.
 // Rows: from `minTiles` KiB per input on.  First match wins.
 struct ShapeTier {
   uint64_t minTiles;
   int loads, waves;
 };
-static const ShapeTier kShape[9][3] = {
-    /* 0: copies */ {{0, 0, 0}, {0, 0, 0}, {0, 0, 0}},
-    /* 1 */ {{0, 0, 0}, {0, 0, 0}, {0, 0, 0}},
-    /* 2 */ {{98304, 1, 25}, {0, 0, 25}, {0, 0, 25}},
-    /* 3 */ {{131072, 1, 21}, {32768, 1, 25}, {0, 0, 25}},
-    /* 4 */ {{131072, 2, 14}, {32768, 1, 25}, {0, 0, 25}},
-    /* 5 */ {{65536, 2, 16}, {16384, 2, 25}, {0, 0, 21}},
-    /* 6 */ {{65536, 2, 14}, {16384, 2, 25}, {0, 0, 21}},
-    /* 7 */ {{65536, 2, 14}, {16384, 2, 25}, {0, 0, 18}},
-    /* 8 */ {{65536, 2, 14}, {16384, 2, 25}, {0, 0, 18}},
+static const ShapeTier kShape[9][4] = {
+    /* 0: copies */ {{0, 0, 0}, {0, 0, 0}, {0, 0, 0}, {0, 0, 0}},
+    /* 1 */ {{0, 0, 0}, {0, 0, 0}, {0, 0, 0}, {0, 0, 0}},
+    /* 2 */ {{98304, 1, 25}, {0, 0, 25}, {0, 0, 25}, {0, 0, 25}},
+    /* 3 */ {{90112, 1, 25}, {0, 0, 25}, {0, 0, 25}, {0, 0, 25}},
+    /* 4 */ {{131072, 2, 14}, {90112, 1, 25}, {40960, 2, 25}, {0, 0, 25}},
+    /* 5 */ {{106496, 2, 16}, {73728, 1, 25}, {16384, 0, 18}, {0, 0, 21}},
+    /* 6 */ {{90112, 2, 14}, {57344, 2, 16}, {16384, 2, 25}, {0, 0, 21}},
+    /* 7 */ {{90112, 2, 14}, {40960, 1, 25}, {16384, 2, 25}, {0, 0, 18}},
+    /* 8 */ {{90112, 2, 14}, {40960, 1, 25}, {16384, 2, 25}, {0, 0, 18}},
 };
 // explicit settings of the calling thread (flagcxLocalTune, flagcxLocalTuneLoads);
 // -1 = choose as above.  Per thread: a caller that fixes the launch shape for its
@@ -118,8 +123,8 @@ static thread_local TuneOverrides tlsTune;
 LaunchShape launchShapeFor(int k, uint64_t tiles) {
   if (k < 0) k = 0;
   if (k > 8) k = 8;
-  const ShapeTier *t = &kShape[k][2];
-  for (int i = 0; i < 3; i++)
+  const ShapeTier *t = &kShape[k][3];
+  for (int i = 0; i < 4; i++)
     if (tiles >= kShape[k][i].minTiles) {
       t = &kShape[k][i];
       break;
@@ -129,7 +134,7 @@ LaunchShape launchShapeFor(int k, uint64_t tiles) {
   if (k >= 2 && loads >= 0) {
     s.loads = loads < k ? loads : 0;
     // the product of wavefronts and inputs in flight is what has to cover the latency
-    if (s.loads != t->loads) s.waves = s.loads == 0 ? kShape[k][2].waves : s.loads == 1 ? 25 : s.loads == 2 ? 14 : 11;
+    if (s.loads != t->loads) s.waves = s.loads == 0 ? kShape[k][3].waves : s.loads == 1 ? 25 : s.loads == 2 ? 14 : 11;
   }
   if (waves >= 0) s.waves = waves;
   return s;
