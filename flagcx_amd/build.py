@@ -21,7 +21,10 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-fno-fast-math", "-Wall", "-fvisibility=hidden",
          # keep the compiler from forming packed fp32 VALU ops
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # and from fusing the last fp32 operation of a fold into the conversion to fp16 (v_fma_mix*):
+         # that rounds the exact result once, the fold is defined as fp32 results rounded to fp16
+         "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts"]
 
 
 def _run(cmd):

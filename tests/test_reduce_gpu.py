@@ -391,3 +391,81 @@ def test_special_values_on_the_generic_and_element_paths(L, dt):
         torch.cuda.synchronize()
         rc, want = O.reduce([np.ascontiguousarray(pads[0][1:1 + m * m]), rows[1], rows[2]], dt, op)
         assert same(from_dev(out, npdt), want, nan_class=arith_nan_ok(dt, op), dtype=dt), (DT_NAME[dt], OP_NAME[op], "elem")
+
+
+def _tie_columns(k, op, want_columns=64):
+    """Columns of k fp16 values whose fp32 fold lands on a tie between two fp16 values while the exact result
+    does not: rounding the fold's fp32 result (what the fold is defined to do) and rounding the exact result once
+    (what an operation fused into the conversion does) give different fp16 values there."""
+    rng = np.random.default_rng(1000 + 10 * k + op)
+    found = []
+    for _ in range(8):   # (such columns are about 6 in 100 000 for products; sums of a few halves are exact in fp32,
+                         # and a quotient by 3, 5, 6 or 7 never ends in the bits of a tie)
+        if sum(c.shape[1] for c in found) >= want_columns:
+            break
+        f = rng.standard_normal((k, 1 << 20))
+        cand = (1.0 + 0.1 * f if op == O.PROD else f).astype(np.float16)
+        acc32 = cand[0].astype(np.float32)
+        exact = cand[0].astype(np.float64)
+        for j in range(1, k):
+            if op == O.PROD:
+                acc32 = cand[j].astype(np.float32) * acc32
+                exact = cand[j].astype(np.float64) * exact
+            else:
+                acc32 = cand[j].astype(np.float32) + acc32
+                exact = cand[j].astype(np.float64) + exact
+        if op == O.AVG:
+            acc32 = acc32 / np.float32(k)
+            exact = exact / np.float64(k)
+        twice, once = acc32.astype(np.float16), exact.astype(np.float16)
+        found.append(cand[:, twice.view(np.uint16) != once.view(np.uint16)])
+    cols = np.concatenate(found, axis=1)[:, :want_columns]
+    assert cols.shape[1] >= 8, "no rounding ties found for this fold"
+    return cols
+
+
+@pytest.mark.parametrize("op,k", [(O.PROD, 3), (O.PROD, 4), (O.PROD, 5), (O.PROD, 6), (O.PROD, 7), (O.PROD, 8)],
+                         ids=lambda v: str(v))
+def test_fp16_fold_rounds_in_fp32_before_it_rounds_to_fp16(L, op, k):
+    """The fold of halves is a chain of fp32 operations, each rounded to fp32, and ONE final conversion.  A
+    compiler that fuses the last operation into the conversion rounds the exact result once instead, which
+    differs wherever the fp32 result is a tie between two fp16 values (6 elements in 100 000 of random data; it
+    happened for products, in the few head and tail elements only, whose loop over the inputs unrolls).  Every
+    element here is such a case, through one call, a batch, a gated batch and the queue, head and tail included."""
+    import torch
+    cols = _tie_columns(k, op)
+    n = 4096 + 13
+    ins = [np.ascontiguousarray(np.resize(cols[j], n + 16)) for j in range(k)]
+    devs = [to_dev(a) for a in ins]
+    rc, want = O.reduce([np.ascontiguousarray(a[1:n + 1]) for a in ins], O.FP16, op)
+    assert rc == 0
+    outs = [dev_empty(n + 16, 2, fill=0) for _ in range(4)]
+    srcs = [d.data_ptr() + 2 for d in devs]          # one element in: 7 head elements, a tail
+    dst = [o.data_ptr() + 2 for o in outs]
+    L.check(L.lib().flagcxLocalReduce(L._ptr_array(srcs), k, dst[0], n, int(O.FP16), int(op),
+                                      L._sref(L.current_stream())))
+    L.reduce_batch([(srcs, dst[1], n // 2), ([p + (n // 2) * 2 for p in srcs], dst[1] + (n // 2) * 2, n - n // 2)],
+                   op, O.FP16, k)
+    torch.cuda.synchronize()
+    L.lib().flagcxLocalSetMaxSpinCount(1 << 21)
+    side = torch.cuda.Stream()
+    try:
+        with L.Gate() as gate:
+            with torch.cuda.stream(side):
+                gate.reduce_batch([(srcs, dst[2], n)], op, O.FP16, k)
+            gate.open(1)
+            side.synchronize()
+            assert gate.query()[2] == 0
+        q = L.ReduceFifo(4, k, O.FP16, op)
+        try:
+            with q:
+                q.wait(q.enqueue_reduce(srcs, dst[3], n))
+        finally:
+            q.close()
+    finally:
+        L.lib().flagcxLocalSetMaxSpinCount(-1)
+    torch.cuda.synchronize()
+    for name, out in zip(("one call", "batch", "gated batch", "queue"), outs):
+        got = from_dev(out, np.float16)[1:n + 1]
+        differing = np.nonzero(got.view(np.uint16) != want.view(np.uint16))[0]
+        assert differing.size == 0, (name, op, k, differing.size, differing[:8])
