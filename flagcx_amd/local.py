@@ -7,6 +7,7 @@ RuntimeError), never a silent fallback.
 import ctypes as C
 import enum
 import os
+import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(HERE, "lib", "libflagcx_amd.so")
@@ -147,6 +148,15 @@ def lib():
         if not os.path.exists(_LIB_PATH):
             raise RuntimeError("%s is missing: build it with `python -m flagcx_amd.build` "
                                "(there is no fallback implementation)" % _LIB_PATH)
+        # PyTorch ships its own copy of the HIP runtime.  Whichever copy a process loads first serves both,
+        # and PyTorch does not find its GPUs through another one: where torch is in the process, let it
+        # load and initialise its runtime before this library brings in the system's (torch may be imported
+        # later by the same process: tests, bench.py and every user of this binding hold their buffers in it).
+        try:
+            import torch
+            torch.cuda.is_available()
+        except Exception:
+            pass
         L = C.CDLL(_LIB_PATH)
         vp, sz, i, pp = C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)
         sp = C.POINTER(Stream)
