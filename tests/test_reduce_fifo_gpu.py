@@ -478,3 +478,45 @@ def test_consumer_on_a_queue_of_its_own_holds_no_stream_up(L):
     finally:
         q.close()
     assert same(from_dev(out, np.float32), expect(ins, dt, op), nan_class=True, dtype=dt)
+
+
+def test_random_chains_of_dependent_entries_replay_in_order(L):
+    """Seeded random runs of entries over a small pool of buffers: sources repeat, the destination may be one of
+    the sources, later entries read and overwrite what earlier ones wrote, over sub-ranges.  The queue must give
+    what running the entries one after another gives (replayed on the CPU through the oracle)."""
+    import random
+    import torch
+    rnd = random.Random(4242)
+    for case in range(160):
+        dt, op = rnd.choice([(O.INT32, O.SUM), (O.FP32, O.SUM), (O.INT32, O.MAX), (O.FP32, O.PROD), (O.INT64, O.MIN)])
+        npdt = np.dtype(O.NP_OF[dt])
+        isz = npdt.itemsize
+        nbuf, n = rnd.randint(3, 7), rnd.choice([64, 1000, 4096, rnd.randint(1, 100_000)])
+        rng = np.random.default_rng(rnd.randint(0, 1 << 30))
+        if npdt.kind == "f":
+            host = [(1.0 + 0.01 * rng.standard_normal(n)).astype(npdt) for _ in range(nbuf)]
+        else:
+            host = [rng.integers(-1000, 1000, n).astype(npdt) for _ in range(nbuf)]
+        dev = [to_dev(h) for h in host]
+        torch.cuda.synchronize()
+        maxk = rnd.randint(2, 8)
+        q = L.ReduceFifo(rnd.choice([4, 8, 64]), maxk, dt, op)
+        plan = []
+        try:
+            with q:
+                ticket = 0
+                for _ in range(rnd.randint(1, 40)):
+                    srcs = [rnd.randrange(nbuf) for _ in range(rnd.randint(1, maxk))]
+                    d = rnd.randrange(nbuf)
+                    lo = rnd.randrange(0, n)
+                    cnt = rnd.randint(1, n - lo)
+                    plan.append((srcs, d, lo, cnt))
+                    ticket = q.enqueue_reduce([dev[s].data_ptr() + lo * isz for s in srcs], dev[d].data_ptr() + lo * isz, cnt)
+                q.wait(ticket)
+        finally:
+            q.close()
+        torch.cuda.synchronize()
+        for srcs, d, lo, cnt in plan:
+            host[d][lo:lo + cnt] = expect([host[s][lo:lo + cnt] for s in srcs], dt, op)
+        for i in range(nbuf):
+            assert same(from_dev(dev[i], npdt), host[i], nan_class=True, dtype=dt), (case, dt, op, i, plan[:4])
