@@ -359,12 +359,18 @@ def config_c3(L, full=False, separate=False):
     descs = c3_chunk_descs(L, nranks, shard, send, recv, rank)
     ms = timed_ms(lambda: L.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks))
     rows["C3_batch_32x4MiB"] = row(nb, ms, note="32 chunk descriptors, one batch call (needs every chunk present)")
-    ms, grid = c3_queue_ms(L, nranks, descs)
-    rows["C3_queue_32x4MiB"] = row(nb, ms, note="chunk by chunk through the resident reduce queue, host wall clock "
-                                                "first enqueue -> Wait; %d resident wavefronts" % grid)
-    ms = c3_gated_ms(L, nranks, descs)
-    rows["C3_gated_batch_32x4MiB"] = row(nb, ms, note="one batch launched up front, a host store per chunk lets its "
-                                                      "wavefronts go; host wall clock launch -> stream sync")
+    try:
+        ms, grid = c3_queue_ms(L, nranks, descs)
+        rows["C3_queue_32x4MiB"] = row(nb, ms, note="chunk by chunk through the resident reduce queue, host wall clock "
+                                                    "first enqueue -> Wait; %d resident wavefronts" % grid)
+    except Exception as e:   # a row of its own: the others are measured all the same
+        rows["C3_queue_32x4MiB"] = {"error": repr(e)}
+    try:
+        ms = c3_gated_ms(L, nranks, descs)
+        rows["C3_gated_batch_32x4MiB"] = row(nb, ms, note="one batch launched up front, a host store per chunk lets its "
+                                                          "wavefronts go; host wall clock launch -> stream sync")
+    except Exception as e:
+        rows["C3_gated_batch_32x4MiB"] = {"error": repr(e)}
     ms = timed_ms(lambda: L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE))
     rows["C3_per_chunk_launches"] = row(nb, ms, note="32 launches of 4 MiB chunks on one stream, %.2f us per launch"
                                                      % (ms * 1e3 / 32))
@@ -857,22 +863,32 @@ def main():
                          "C5 rows: median of 20 single launches, each between its own event pair; "
                          "frac = GB/s / 8000; buffers placed by flagcxLocalPlaceBuffers unless "
                          "--allocator-layout"}
-        c1_rows, (ca, cb, cout) = config_c1(L, args.allocator_layout)
-        cfg.update(c1_rows)
-        if not args.no_cpu:
-            c1_cpu, ha, hb = cpu_c1_reference_path()
-            result["cpu_baseline"]["c1_fp32_reference_path"] = c1_cpu
-            # the GPU's C1 output against the same sum on the host (fp32 add is exact either way)
-            L.reduce([ca, cb], cout, L.RedOp.Sum)
-            torch.cuda.synchronize()
-            ga, gb = ca.cpu().numpy(), cb.cpu().numpy()
-            cfg["C1_same_buffers"]["bit_exact_vs_host_sum"] = bool(np.array_equal(cout.cpu().numpy(), ga + gb))
-            del ha, hb
-        del ca, cb, cout
-        torch.cuda.empty_cache()
-        cfg.update(config_c3(L, full=False, separate=args.allocator_layout))
-        cfg.update(config_c4(L, args.allocator_layout))
-        cfg.update(config_c5(L))
+        # the rows below are additions to the line: whatever goes wrong in one of them is reported in its
+        # place, and the headline figures above are printed all the same
+        try:
+            c1_rows, (ca, cb, cout) = config_c1(L, args.allocator_layout)
+            cfg.update(c1_rows)
+            if not args.no_cpu:
+                c1_cpu, ha, hb = cpu_c1_reference_path()
+                result["cpu_baseline"]["c1_fp32_reference_path"] = c1_cpu
+                # the GPU's C1 output against the same sum on the host (fp32 add is exact either way)
+                L.reduce([ca, cb], cout, L.RedOp.Sum)
+                torch.cuda.synchronize()
+                ga, gb = ca.cpu().numpy(), cb.cpu().numpy()
+                cfg["C1_same_buffers"]["bit_exact_vs_host_sum"] = bool(np.array_equal(cout.cpu().numpy(), ga + gb))
+                del ha, hb
+            del ca, cb, cout
+            torch.cuda.empty_cache()
+        except Exception as e:
+            cfg["C1_error"] = repr(e)
+            log("bench.py: configuration C1 failed: %r" % (e,))
+        for name, fn in (("C3", lambda: config_c3(L, full=False, separate=args.allocator_layout)),
+                         ("C4", lambda: config_c4(L, args.allocator_layout)), ("C5", lambda: config_c5(L))):
+            try:
+                cfg.update(fn())
+            except Exception as e:
+                cfg[name + "_error"] = repr(e)
+                log("bench.py: configuration %s failed: %r" % (name, e))
         result["configs"] = cfg
 
     print(json.dumps(result))
