@@ -256,6 +256,8 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
  * has passed i's number.  One ordinary launch per 32 descriptors, 3 to 4 % under
  * the rate of flagcxLocalReduceBatch, and a chunk's fold starts about 2 us after
  * its Open.
+ * (An extension: the reference has no such entry point; its counterpart there is
+ * that loop plus one collective call per completed chunk.)
  *
  * Descriptors get consecutive numbers per gate, from 0 at creation: this call's are
  * *first .. *first + ndescs - 1 (first may be NULL).  Open(upto) lets every
