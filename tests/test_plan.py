@@ -134,3 +134,45 @@ def test_plan_execute_one_cluster_block_moves(tmp_path, commop):
         else:
             want = np.concatenate([sum(h[r * chunk:(r + 1) * chunk] for h in hosts), untouched[chunk:]])
         assert same(got, want), (commop, r)
+
+
+@pytest.mark.gpu
+def test_plan_execute_one_cluster_random_shapes(tmp_path):
+    """The same block movers for seeded random rank counts (1..8), roots and chunk sizes."""
+    import random
+    import torch
+    rnd = random.Random(77)
+    for case in range(120):
+        commop = rnd.choice([PX.ALLGATHER, PX.GATHER, PX.ALLTOALL, PX.SCATTER, PX.BROADCAST, PX.REDUCE, PX.REDUCESCATTER])
+        nranks = rnd.randint(1, 8)
+        root = rnd.randrange(nranks)
+        chunk = rnd.choice([1, 3, 16, 1000, rnd.randint(1, 40_000)])
+        prefix = str(tmp_path / ("plan%d" % case))
+        PX.one_cluster_collective(prefix, commop, nranks, root)
+        n = nranks * chunk
+        plan = local.Plan([0] * nranks, n, commop, local.RedOp.Sum)
+        plan.import_xml(prefix)
+        rng = np.random.default_rng(case)
+        hosts = [rng.integers(-2**27, 2**27, n, dtype=np.int32) for _ in range(nranks)]
+        send = [to_dev(h) for h in hosts]
+        recv = [dev_empty(n, 4, fill=0x55) for _ in range(nranks)]
+        plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, O.INT32, root=root)
+        torch.cuda.synchronize()
+        untouched = np.full(n, 0x55, dtype=np.int32)
+        for r in range(nranks):
+            got = from_dev(recv[r], np.int32)
+            if commop == PX.ALLGATHER:
+                want = np.concatenate([hosts[j][:chunk] for j in range(nranks)])
+            elif commop == PX.GATHER:
+                want = np.concatenate([hosts[j][:chunk] for j in range(nranks)]) if r == root else untouched
+            elif commop == PX.ALLTOALL:
+                want = np.concatenate([hosts[j][r * chunk:(r + 1) * chunk] for j in range(nranks)])
+            elif commop == PX.SCATTER:
+                want = np.concatenate([hosts[root][r * chunk:(r + 1) * chunk], untouched[chunk:]])
+            elif commop == PX.BROADCAST:
+                want = np.concatenate([hosts[root][:chunk], untouched[chunk:]])
+            elif commop == PX.REDUCE:
+                want = np.concatenate([sum(h[:chunk] for h in hosts), untouched[chunk:]]) if r == root else untouched
+            else:
+                want = np.concatenate([sum(h[r * chunk:(r + 1) * chunk] for h in hosts), untouched[chunk:]])
+            assert same(got, want.astype(np.int32)), (case, commop, nranks, root, chunk, r)
