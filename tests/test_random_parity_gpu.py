@@ -96,3 +96,67 @@ def test_random_cases_match_the_oracle(L, mode):
         one_case(L, rnd, mode, side, large=False)
     for i in range(12 if mode != "queue" else 6):
         one_case(L, rnd, mode, side, large=True)
+
+
+SPECIAL = {
+    O.FP16: (np.uint16, [0x0000, 0x8000, 0x7c00, 0xfc00, 0x7e00, 0xfe01, 0x7c01, 0x0001, 0x8001, 0x03ff, 0x0400, 0x7bff,
+                         0xfbff, 0x3c00, 0xbc00, 0x3555, 0x4248]),
+    O.BF16: (np.uint16, [0x0000, 0x8000, 0x7f80, 0xff80, 0x7fc0, 0xffc1, 0x7f81, 0x0001, 0x8001, 0x007f, 0x0080, 0x7f7f,
+                         0xff7f, 0x3f80, 0xbf80, 0x3eab, 0x4049]),
+    O.FP32: (np.uint32, [0x00000000, 0x80000000, 0x7f800000, 0xff800000, 0x7fc00000, 0xffc00001, 0x7f800001, 0x00000001,
+                         0x80000001, 0x007fffff, 0x00800000, 0x7f7fffff, 0xff7fffff, 0x3f800000, 0xbf800000, 0x3eaaaaab,
+                         0x40490fdb]),
+    O.FP64: (np.uint64, [0x0, 0x8000000000000000, 0x7ff0000000000000, 0xfff0000000000000, 0x7ff8000000000000,
+                         0xfff8000000000001, 0x7ff0000000000001, 0x1, 0x8000000000000001, 0x000fffffffffffff,
+                         0x0010000000000000, 0x7fefffffffffffff, 0xffefffffffffffff, 0x3ff0000000000000,
+                         0xbff0000000000000, 0x3fd5555555555555, 0x400921fb54442d18]),
+}
+
+
+@pytest.mark.parametrize("mode", ["reduce", "batch", "gated", "queue"])
+def test_random_special_values_match_the_oracle(L, mode):
+    """Inputs drawn from NaNs with payloads, infinities, signed zeros, denormals and the extremes of each
+    floating-point type: min and max return the chosen input bit for bit (the last NaN or zero wins as in the
+    reference's templates), sums and products give the oracle's bits or a NaN where it gives a NaN."""
+    import torch
+    rnd = random.Random({"reduce": 31, "batch": 32, "gated": 33, "queue": 34}[mode])
+    side = torch.cuda.Stream()
+    for case in range(150 if mode != "queue" else 60):
+        dt, op = rnd.choice(list(SPECIAL)), rnd.choice(OPS)
+        ut, pool = SPECIAL[dt]
+        npdt = np.dtype(O.NP_OF[dt])
+        isz = npdt.itemsize
+        k = rnd.randint(1, 8)
+        n = rnd.choice([1, 9, 100, 1031, rnd.randint(1, 20_000)])
+        rng = np.random.default_rng(rnd.randint(0, 1 << 30))
+        ins = [np.array(pool, dtype=ut)[rng.integers(0, len(pool), n + 32)].view(npdt) for _ in range(k)]
+        off = rnd.randrange(0, 16)
+        devs = [to_dev(a) for a in ins]
+        out = dev_empty(n + 32, isz, fill=0)
+        srcs = [d.data_ptr() + off * isz for d in devs]
+        dst = out.data_ptr() + off * isz
+        torch.cuda.synchronize()
+        if mode == "reduce":
+            L.check(L.lib().flagcxLocalReduce(L._ptr_array(srcs), k, dst, n, int(dt), int(op), L._sref(L.current_stream())))
+        elif mode == "batch":
+            h = n // 2
+            L.reduce_batch([(srcs, dst, h), ([p + h * isz for p in srcs], dst + h * isz, n - h)] if h else [(srcs, dst, n)],
+                           op, dt, k)
+        elif mode == "gated":
+            with L.Gate() as gate:
+                with torch.cuda.stream(side):
+                    gate.reduce_batch([(srcs, dst, n)], op, dt, k)
+                gate.open(1)
+                side.synchronize()
+                assert gate.query()[2] == 0
+        else:
+            q = L.ReduceFifo(4, 8, dt, op)
+            try:
+                with q:
+                    q.wait(q.enqueue_reduce(srcs, dst, n))
+            finally:
+                q.close()
+        torch.cuda.synchronize()
+        rc, want = O.reduce([np.ascontiguousarray(a[off:off + n]) for a in ins], dt, op)
+        got = from_dev(out, npdt)[off:off + n]
+        assert rc == 0 and same(got, want, nan_class=op in (O.SUM, O.PROD, O.AVG), dtype=dt), (mode, case, dt, op, k, n, off)
