@@ -145,12 +145,77 @@ union Vec16 {
   T e[16 / sizeof(T)];
 };
 
+// 8-bit elements are folded four at a time in a 32-bit word: the bytes at even and
+// at odd positions are accumulated apart, as the two 16-bit halves of one word each
+// (packed 16-bit instructions; gfx950 has no packed 8-bit ones).  Sums and products
+// wrap modulo 256, so whatever gathers above the low byte of a half is dropped when
+// the halves are put together again; minima and maxima compare the byte in the HIGH
+// position of its half, the other byte cleared, which keeps a signed byte's sign
+// where a signed 16-bit compare looks for it.  The results are those of the
+// element-by-element fold; written this way the data stays packed, where the
+// compiler, left to itself, unpacks eight inputs into one register per byte.
+#ifndef FLAGCX_PACKED_8BIT
+#define FLAGCX_PACKED_8BIT 1
+#endif
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+
+template <typename T, int OP>
+struct Fold8 {
+  static_assert(sizeof(T) == 1, "8-bit element types only");
+  static constexpr bool kSel = (OP == kMax || OP == kMin);
+  static constexpr bool kSigned = ((T)-1 < (T)0);
+  struct acc_t { uint32_t ev, od; };
+  static __device__ __forceinline__ uint32_t shr8(uint32_t w) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w) >> (u16x2)(8));
+  }
+  static __device__ __forceinline__ uint32_t shl8(uint32_t w) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2, w) << (u16x2)(8));
+  }
+  static __device__ __forceinline__ uint32_t evenOf(uint32_t w) { return kSel ? (kSigned ? shl8(w) : (w & 0x00ff00ffu)) : w; }
+  static __device__ __forceinline__ uint32_t oddOf(uint32_t w) { return kSel ? (w & 0xff00ff00u) : shr8(w); }
+  static __device__ __forceinline__ uint32_t join(uint32_t a, uint32_t b) {
+    if (kSel) {
+      if (kSigned) {
+        const i16x2 x = __builtin_bit_cast(i16x2, a), y = __builtin_bit_cast(i16x2, b);
+        return __builtin_bit_cast(uint32_t, OP == kMax ? __builtin_elementwise_max(x, y) : __builtin_elementwise_min(x, y));
+      }
+      const u16x2 x = __builtin_bit_cast(u16x2, a), y = __builtin_bit_cast(u16x2, b);
+      return __builtin_bit_cast(uint32_t, OP == kMax ? __builtin_elementwise_max(x, y) : __builtin_elementwise_min(x, y));
+    }
+    const u16x2 x = __builtin_bit_cast(u16x2, a), y = __builtin_bit_cast(u16x2, b);
+    return __builtin_bit_cast(uint32_t, OP == kProd ? (u16x2)(x * y) : (u16x2)(x + y));
+  }
+  static __device__ __forceinline__ acc_t init(uint32_t w) { return {evenOf(w), oddOf(w)}; }
+  static __device__ __forceinline__ acc_t step(uint32_t w, acc_t b) { return {join(evenOf(w), b.ev), join(oddOf(w), b.od)}; }
+  // the four folded bytes (a sum not yet divided for the average)
+  static __device__ __forceinline__ uint32_t bytes(acc_t a) {
+    if (kSel) return (kSigned ? shr8(a.ev) : a.ev) | a.od;
+    return (a.ev & 0x00ff00ffu) | shl8(a.od);
+  }
+};
+
 // Fold one 16-byte vector position across K registers.
 template <typename T, int OP, int K>
 __device__ __forceinline__ u32x4 foldVec(const u32x4 (&in)[K], int k) {
   typedef Fold<T, OP> F;
   constexpr int N = 16 / sizeof(T);
   Vec16<T> r;
+  if constexpr (sizeof(T) == 1 && FLAGCX_PACKED_8BIT) {
+    typedef Fold8<T, OP> F8;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+      typename F8::acc_t a = F8::init(in[0][d]);
+#pragma unroll
+      for (int j = 1; j < K; j++) a = F8::step(in[j][d], a);
+      r.v[d] = F8::bytes(a);
+    }
+    if (OP == kAvg) {
+#pragma unroll
+      for (int e = 0; e < N; e++) r.e[e] = F::fin((typename F::acc_t)r.e[e], k);
+    }
+    return r.v;
+  }
 #pragma unroll
   for (int e = 0; e < N; e++) {
     Vec16<T> x;
@@ -325,17 +390,87 @@ __global__ void __launch_bounds__(64) reduceBatchKernel(ReduceBatchParams<K> bp)
   reduceWaveBody<T, OP, K, U, TILED>(bp.seg[blockIdx.y]);
 }
 
-// Aligned body, any k up to FLAGCX_MAX_RANKS, same streaming shape as above: one
-// wavefront per workgroup, one KiB of every input per tile.  Inputs are consumed in
-// order in batches of eight loads; the accumulators stay in registers between
-// batches, so the fold and its single final rounding are unchanged.
+// More than eight inputs are consumed in order in batches of eight loads; the
+// accumulators stay in registers between batches, so the fold and its single final
+// rounding are unchanged.  A batch of C inputs is folded as one chain of C steps in
+// straight-line code: C is a template argument (the first batch and those in the
+// middle are full, the last one goes through a switch on what is left).  With the
+// batch length a run-time bound instead, measured on MI355X at 9..16 inputs of
+// 128 MiB: 32-bit integer sum / min / max 65-69 % of the HBM peak and 8-bit min / max
+// 56-62 %, where the other types ran at 84-88 % and all do now.
+// What travels from one batch to the next: the accumulators of one 16-byte position.
+// Where an accumulator has the size of an element (every type but the two 16-bit
+// floating-point ones) they travel packed in four registers, as the inputs do.
+template <typename T, int OP, bool PACKED = sizeof(typename Fold<T, OP>::acc_t) == sizeof(T)>
+struct Carry;
 template <typename T, int OP>
-__global__ void __launch_bounds__(64) reduceWaveAnyKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
+struct Carry<T, OP, true> {
+  typedef typename Fold<T, OP>::acc_t acc_t;
+  Vec16<T> v;
+  __device__ __forceinline__ acc_t get(int e) const { return (acc_t)v.e[e]; }
+  __device__ __forceinline__ void set(int e, acc_t a) { v.e[e] = (T)a; }
+};
+template <typename T, int OP>
+struct Carry<T, OP, false> {
+  typedef typename Fold<T, OP>::acc_t acc_t;
+  acc_t a[16 / sizeof(T)];
+  __device__ __forceinline__ acc_t get(int e) const { return a[e]; }
+  __device__ __forceinline__ void set(int e, acc_t x) { a[e] = x; }
+};
+
+template <typename T, int OP, int C, bool FIRST>
+__device__ __forceinline__ void foldBatch(const u32x4 (&in)[8], Carry<T, OP> &acc) {
+  typedef Fold<T, OP> F;
+  if constexpr (sizeof(T) == 1) {
+    typedef Fold8<T, OP> F8;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+      typename F8::acc_t a = FIRST ? F8::init(in[0][d]) : F8::step(in[0][d], F8::init(acc.v.v[d]));
+#pragma unroll
+      for (int b = 1; b < C; b++) a = F8::step(in[b][d], a);
+      acc.v.v[d] = F8::bytes(a);
+    }
+  } else {
+    constexpr int N = 16 / sizeof(T);
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+      Vec16<T> x;
+      x.v = in[0];
+      typename F::acc_t a = FIRST ? F::init(x.e[e]) : F::step(x.e[e], acc.get(e));
+#pragma unroll
+      for (int b = 1; b < C; b++) {
+        x.v = in[b];
+        a = F::step(x.e[e], a);
+      }
+      acc.set(e, a);
+    }
+  }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ void foldRest(const u32x4 (&in)[8], Carry<T, OP> &acc, int rest) {
+  switch (rest) { // wave-uniform
+    case 1: foldBatch<T, OP, 1, false>(in, acc); break;
+    case 2: foldBatch<T, OP, 2, false>(in, acc); break;
+    case 3: foldBatch<T, OP, 3, false>(in, acc); break;
+    case 4: foldBatch<T, OP, 4, false>(in, acc); break;
+    case 5: foldBatch<T, OP, 5, false>(in, acc); break;
+    case 6: foldBatch<T, OP, 6, false>(in, acc); break;
+    case 7: foldBatch<T, OP, 7, false>(in, acc); break;
+    default: break;
+  }
+}
+
+// Aligned body, k from 8 up to FLAGCX_MAX_RANKS, same streaming shape as above: one
+// wavefront per workgroup, one KiB of every input per tile.
+// (At most 168 registers: twelve wavefronts per CU, the most its launcher asks for.)
+template <typename T, int OP>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3))) reduceWaveAnyKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
   typedef Fold<T, OP> F;
   constexpr int N = 16 / sizeof(T);
   constexpr int B = 8;
   constexpr uint32_t kTileBytes = 1024u;
-  const int k = p.k;
+  const int k = p.k; // >= B: the launcher sends fewer inputs to the kernels above
   const uint64_t bodyBytes = p.nvec * 16;
   const uint32_t lead = p.lead; // the first tile is short: the others start on a cache line of most buffers
   const uint64_t ntiles = (bodyBytes + lead + kTileBytes - 1) / kTileBytes;
@@ -346,33 +481,33 @@ __global__ void __launch_bounds__(64) reduceWaveAnyKernel(ReduceParams<FLAGCX_MA
     const uint64_t left = bodyBytes - off;
     const uint32_t cap = t ? kTileBytes : kTileBytes - lead;
     const uint32_t span = left < cap ? (uint32_t)left : cap;
-    typename F::acc_t acc[N];
-    for (int j0 = 0; j0 < k; j0 += B) {
-      u32x4 in[B];
+    Carry<T, OP> acc;
+    u32x4 in[B];
+    int j0 = 0;
+    for (; j0 + B <= k; j0 += B) {
 #pragma unroll
-      for (int b = 0; b < B; b++)
-        if (j0 + b < k) {
+      for (int b = 0; b < B; b++) {
+        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)((const char *)p.src[j0 + b] + headBytes + off), 0, span, kRsrcFlags);
+        in[b] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kLoadAux);
+      }
+      if (j0 == 0) foldBatch<T, OP, B, true>(in, acc);
+      else foldBatch<T, OP, B, false>(in, acc);
+    }
+    const int rest = k - j0;
+    if (rest > 0) {
+#pragma unroll
+      for (int b = 0; b < B - 1; b++)
+        if (b < rest) {
           __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
               (void *)((const char *)p.src[j0 + b] + headBytes + off), 0, span, kRsrcFlags);
           in[b] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kLoadAux);
         }
-#pragma unroll
-      for (int b = 0; b < B; b++)
-        if (j0 + b < k) {
-          Vec16<T> x;
-          x.v = in[b];
-          if (j0 + b == 0) {
-#pragma unroll
-            for (int e = 0; e < N; e++) acc[e] = F::init(x.e[e]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < N; e++) acc[e] = F::step(x.e[e], acc[e]);
-          }
-        }
+      foldRest<T, OP>(in, acc, rest);
     }
     Vec16<T> r;
 #pragma unroll
-    for (int e = 0; e < N; e++) r.e[e] = F::fin(acc[e], k);
+    for (int e = 0; e < N; e++) r.e[e] = F::fin(acc.get(e), k);
     __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
         (void *)((char *)p.dst + headBytes + off), 0, span, kRsrcFlags);
     __builtin_amdgcn_raw_buffer_store_b128(r.v, rd, voff, 0, kStoreAux);
@@ -386,7 +521,8 @@ __global__ void __launch_bounds__(64) reduceWaveAnyKernel(ReduceParams<FLAGCX_MA
   }
 }
 
-// Sources that do not share the destination's address modulo 16.  The tiling is
+// More than eight sources that do not share the destination's address modulo 16,
+// 8-byte elements (the others take reduceWaveShiftAnyKernel).  The tiling is
 // the destination's (aligned 16-byte stores after p.head elements); each source
 // is read with 16-byte loads at whatever byte offset it happens to have, which
 // the hardware's unaligned access mode serves from at most one extra cache line
@@ -399,37 +535,35 @@ __global__ void __launch_bounds__(64) reduceWaveUnalignedKernel(ReduceParams<FLA
   typedef Fold<T, OP> F;
   constexpr int N = 16 / sizeof(T);
   constexpr int B = 8;
-  const int k = p.k;
+  const int k = p.k; // >= B
   const uint64_t ntiles = (p.nvec + 63) / 64;
   const uint64_t headBytes = p.head * sizeof(T);
   for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
     const uint64_t i = t * 64 + threadIdx.x;
     if (i < p.nvec) {
-      typename F::acc_t acc[N];
-      for (int j0 = 0; j0 < k; j0 += B) {
-        u32x4 in[B];
+      Carry<T, OP> acc;
+      u32x4 in[B];
+      int j0 = 0;
+      for (; j0 + B <= k; j0 += B) {
 #pragma unroll
         for (int b = 0; b < B; b++)
-          if (j0 + b < k)
+          in[b] = __builtin_nontemporal_load(
+              (const u32x4_unaligned *)((const char *)p.src[j0 + b] + headBytes + i * 16));
+        if (j0 == 0) foldBatch<T, OP, B, true>(in, acc);
+        else foldBatch<T, OP, B, false>(in, acc);
+      }
+      const int rest = k - j0;
+      if (rest > 0) {
+#pragma unroll
+        for (int b = 0; b < B - 1; b++)
+          if (b < rest)
             in[b] = __builtin_nontemporal_load(
                 (const u32x4_unaligned *)((const char *)p.src[j0 + b] + headBytes + i * 16));
-#pragma unroll
-        for (int b = 0; b < B; b++)
-          if (j0 + b < k) {
-            Vec16<T> x;
-            x.v = in[b];
-            if (j0 + b == 0) {
-#pragma unroll
-              for (int e = 0; e < N; e++) acc[e] = F::init(x.e[e]);
-            } else {
-#pragma unroll
-              for (int e = 0; e < N; e++) acc[e] = F::step(x.e[e], acc[e]);
-            }
-          }
+        foldRest<T, OP>(in, acc, rest);
       }
       Vec16<T> r;
 #pragma unroll
-      for (int e = 0; e < N; e++) r.e[e] = F::fin(acc[e], k);
+      for (int e = 0; e < N; e++) r.e[e] = F::fin(acc.get(e), k);
       *(u32x4 *)((char *)p.dst + headBytes + i * 16) = r.v;
     }
   }
@@ -561,6 +695,80 @@ __global__ void __launch_bounds__(64) reduceWaveShiftKernel(ShiftParams<K> p) {
     if (threadIdx.x < edge) {
       uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
       foldScalar<T, OP>(p.src, K, p.dst, i);
+    }
+  }
+}
+
+// The same for more than eight sources: batches as in reduceWaveAnyKernel, every
+// source loaded aligned and put in place with lane shifts as above.  Batches of four
+// sources, not eight: two loads per source, and with eight the kernel needs 117-148
+// registers, which leaves room for 12 wavefronts per CU (measured 36-71 % of peak at
+// 9..16 sources of 128 MiB), where this one wants 25 or more (70-77 %).
+template <typename T, int OP>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) reduceWaveShiftAnyKernel(ShiftParams<FLAGCX_MAX_RANKS> p, int k) {
+  typedef Fold<T, OP> F;
+  constexpr int N = 16 / sizeof(T);
+  constexpr int B = 4; // sources per batch: two loads each, and registers enough left for sixteen wavefronts per CU
+  const uint32_t lane = threadIdx.x;
+  const uint64_t ntiles = (p.nvec * 16 + p.lead + 1023) / 1024;
+  const uint64_t headBytes = p.head * sizeof(T);
+  constexpr uint64_t kRound = 8ull * kShiftRun;
+  const uint64_t padded = (ntiles + kRound - 1) / kRound * kRound;
+  for (uint64_t b = blockIdx.x; b < padded; b += gridDim.x) {
+    const uint64_t bi = b / 8, bx = b % 8;
+    const uint64_t t = ((bi / kShiftRun) * 8 + bx) * kShiftRun + bi % kShiftRun;
+    if (t >= ntiles) continue;
+    const uint64_t off = t ? t * 1024 - p.lead : 0;
+    const uint64_t g0 = off / 16;
+    Carry<T, OP> acc;
+    for (int j0 = 0; j0 < k; j0 += B) { // k >= B: the first batch is full
+      const int c = k - j0 < B ? k - j0 : B;
+      u32x4 cur[B], ahead[B];
+#pragma unroll
+      for (int i = 0; i < B; i++)
+        if (i < c) {
+          const int j = j0 + i;
+          const uint64_t left = p.granules[j] > g0 ? p.granules[j] - g0 : 0;
+          __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+              (void *)((const char *)p.base[j] + g0 * 16), 0, (uint32_t)(left < 64 ? left : 64) * 16u, kRsrcFlags);
+          cur[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16u, 0, kLoadAux);
+          __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+              (void *)((const char *)p.base[j] + g0 * 16 + 1024), 0, left > 64 ? 16u : 0u, kRsrcFlags);
+          ahead[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, lane * 16u, 0, kLoadAux);
+        }
+      u32x4 in[8];
+#pragma unroll
+      for (int i = 0; i < B; i++)
+        if (i < c) {
+          u32x4 hi;
+#pragma unroll
+          for (int d = 0; d < 4; d++) {
+            const uint32_t fromNext = __builtin_amdgcn_readfirstlane(ahead[i][d]);
+            hi[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)fromNext, (int)cur[i][d], 0x130, 0xf, 0xf, false);
+          }
+          const uint32_t sh = p.shift[j0 + i];
+          in[i] = funnel16(cur[i], hi, sh >> 2, sh & 3u);
+        }
+      if (j0 == 0) foldBatch<T, OP, B, true>(in, acc);
+      else if (c == B) foldBatch<T, OP, B, false>(in, acc);
+      else if (c == 3) foldBatch<T, OP, 3, false>(in, acc);
+      else if (c == 2) foldBatch<T, OP, 2, false>(in, acc);
+      else foldBatch<T, OP, 1, false>(in, acc);
+    }
+    Vec16<T> r;
+#pragma unroll
+    for (int e = 0; e < N; e++) r.e[e] = F::fin(acc.get(e), k);
+    const uint64_t left = p.nvec * 16 - off;
+    const uint32_t cap = t ? 1024u : 1024u - p.lead;
+    __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((char *)p.dst + headBytes + off), 0, left < cap ? (uint32_t)left : cap, kRsrcFlags);
+    __builtin_amdgcn_raw_buffer_store_b128(r.v, rd, lane * 16u, 0, kStoreAux);
+  }
+  if (blockIdx.x == gridDim.x - 1) {
+    const uint64_t edge = p.head + p.tail;
+    if (threadIdx.x < edge) {
+      uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
+      foldScalar<T, OP>(p.src, k, p.dst, i);
     }
   }
 }

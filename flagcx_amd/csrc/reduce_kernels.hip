@@ -145,6 +145,7 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
 
 template <int OP>
 static int launchAny(const ReduceCall &c, const Split &s) {
+  if (c.k <= 8 || c.k > FLAGCX_MAX_RANKS) return (int)hipErrorInvalidValue; // the kernels fold a full first batch of eight
   ReduceParams<FLAGCX_MAX_RANKS> p;
   for (int j = 0; j < c.k; j++) p.src[j] = c.src[j];
   for (int j = c.k; j < FLAGCX_MAX_RANKS; j++) p.src[j] = nullptr;
@@ -175,15 +176,45 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   // 10, more want 8 (85-86 %).  An explicit flagcxLocalTune(8, n) overrides.
   // (A limit on the inputs in flight, as the kernels for up to eight inputs have
   // it, gains nothing here: within one percent for 9..32 inputs.)
-  // More than eight sources at another offset modulo 16 than the output are read
-  // with unaligned 16-byte loads (up to eight take the lane-shift kernel above).
-  int waves = tunedWavesPerCU(8);
-  if (waves < 0) waves = c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
-  const int lds = ldsReservation(waves);
-  if (s.vector)
-    reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
-  else
-    reduceWaveUnalignedKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), lds, c.stream>>>(p);
+  const int tuned = tunedWavesPerCU(8);
+  const int waves = tuned >= 0 ? tuned : c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
+  if (s.vector) {
+    reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), ldsReservation(waves), c.stream>>>(p);
+    return (int)hipGetLastError();
+  }
+  // More than eight sources at another offset modulo 16 than the output (up to eight
+  // take reduceWaveShiftKernel).  Measured at 128 MiB per source, 9 / 16 / 32 sources,
+  // percent of peak: 8-byte elements (the offset can only be 8) read with unaligned
+  // 16-byte loads 72 / 71 / 70, with aligned loads and lane shifts 74 / 68 / 66;
+  // 4-byte elements 72 / 71 / 70 against 75 / 72 / 72; 2- and 1-byte elements, whose
+  // offsets need not be a multiple of four, 61 / 58 / 55 against 72-77 / 72-75 / 70-72.
+  // The lane-shift kernel takes four sources at a time and wants every wavefront its
+  // registers allow (no cap: 12 per CU gave 53-59 %, 16 62-71 %, 25 and more 70-75 %).
+  if constexpr (sizeof(elem_t) == 8) {
+    reduceWaveUnalignedKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), ldsReservation(waves), c.stream>>>(p);
+  } else {
+    ShiftParams<FLAGCX_MAX_RANKS> q;
+    const uint64_t headBytes = s.head * sizeof(elem_t);
+    for (int j = 0; j < FLAGCX_MAX_RANKS; j++) {
+      const uintptr_t first = j < c.k ? (uintptr_t)c.src[j] + headBytes : 0;
+      q.base[j] = (const void *)(first & ~(uintptr_t)15);
+      q.shift[j] = (uint32_t)(first & 15u);
+      q.granules[j] = j < c.k ? s.nvec + (q.shift[j] ? 1 : 0) : 0;
+      q.src[j] = j < c.k ? c.src[j] : nullptr;
+    }
+    q.dst = c.dst;
+    q.nvec = s.nvec;
+    q.head = s.head;
+    q.tail = s.tail;
+    q.inflight = 0;
+    q.lead = s.nvec ? (uint32_t)(((uintptr_t)c.dst + headBytes) & 127u) : 0;
+    const uint64_t shiftTiles = (s.nvec * 16 + q.lead + 1023) / 1024;
+    constexpr uint64_t span = 8ull * kShiftRun;
+    uint64_t grid = (shiftTiles + span - 1) / span * span;
+    if (grid < span) grid = span;
+    if (grid > kMaxGrid) grid = kMaxGrid;
+    reduceWaveShiftAnyKernel<elem_t, OP><<<dim3((unsigned)grid), dim3(64), ldsReservation(tuned >= 0 ? tuned : 0), c.stream>>>(q, c.k);
+  }
   return (int)hipGetLastError();
 }
 

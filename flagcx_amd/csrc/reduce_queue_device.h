@@ -498,8 +498,10 @@ __device__ inline void queueWorker(const QueueKernelArgs &q) {
   }
 }
 
+// At most 128 registers, so that sixteen consumers per CU (the most a queue may ask
+// for) are resident whatever the element type and operation.
 template <typename T, int OP, bool AHEAD>
-__global__ void __launch_bounds__(64) reduceQueueKernel(QueueKernelArgs q) {
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) reduceQueueKernel(QueueKernelArgs q) {
   if (blockIdx.x == 0)
     queueLeader(q);
   else

@@ -469,3 +469,68 @@ def test_fp16_fold_rounds_in_fp32_before_it_rounds_to_fp16(L, op, k):
         got = from_dev(out, np.float16)[1:n + 1]
         differing = np.nonzero(got.view(np.uint16) != want.view(np.uint16))[0]
         assert differing.size == 0, (name, op, k, differing.size, differing[:8])
+
+
+# ------------------------------------------- more than eight inputs, batch by batch
+
+@pytest.mark.parametrize("dt", ALL_DTYPES, ids=lambda d: DT_NAME[d])
+@pytest.mark.parametrize("op", ALL_OPS, ids=lambda o: OP_NAME[o])
+def test_more_than_eight_inputs_every_batch_remainder(L, dt, op):
+    """More than eight inputs are folded in batches (eight at a time where every source
+    shares the output's address modulo 16, four at a time through lane shifts otherwise,
+    unaligned loads for 8-byte elements): every length of the last batch, with the
+    inputs aligned, all at one other offset, and each at an offset of its own."""
+    import torch
+    ts = O.type_size(dt)
+    per16 = 16 // ts
+    n = 2 * 1024 // ts * 3 + 37            # a few tiles and a ragged end
+    for k in list(range(9, 18)) + [20, 23, 33, 64]:
+        srcs = make_inputs(dt, k, n + 64, seed=5000 + 100 * dt + 10 * op + k, op=op)
+        devs = [to_dev(s) for s in srcs]
+        for name, offs, doff in (("aligned", [0] * k, 0),
+                                 ("one offset", [1] * k, 0),
+                                 ("mixed", [(3 * j + 1) % (2 * per16) for j in range(k)], per16 // 2 if per16 > 1 else 1)):
+            out = dev_empty(n + 64, ts, fill=0x55 if ts == 1 else 0x5555)
+            guard = from_dev(out, srcs[0].dtype).copy()
+            L.reduce([d[o:o + n] for d, o in zip(devs, offs)], out[doff:doff + n], op, dtype=dt)
+            torch.cuda.synchronize()
+            rc, want = O.reduce([np.ascontiguousarray(s[o:o + n]) for s, o in zip(srcs, offs)], dt, op)
+            assert rc == 0
+            got = from_dev(out, srcs[0].dtype)
+            assert same(got[doff:doff + n], want, nan_class=arith_nan_ok(dt, op), dtype=dt), (k, name)
+            assert same(got[:doff], guard[:doff]) and same(got[doff + n:], guard[doff + n:]), (k, name)
+
+
+@pytest.mark.parametrize("dt", [O.INT8, O.UINT8], ids=lambda d: DT_NAME[d])
+@pytest.mark.parametrize("k", [2, 3, 8, 9, 12])
+def test_8bit_folds_on_every_pair_of_byte_values(L, dt, k):
+    """8-bit elements are folded four to a 32-bit word with 16-bit packed arithmetic.
+    Every pair of byte values, in each of the four positions of a word, against plain
+    integer arithmetic done here (not the oracle): sum and product modulo 256, minimum
+    and maximum with the type's sign, the average as the wrapped sum divided by k with C
+    truncation.  Inputs beyond the first two repeat the second value."""
+    npdt = np.dtype(O.NP_OF[dt])
+    a = np.repeat(np.arange(256), 256)
+    b = np.tile(np.arange(256), 256)
+    a = np.concatenate([a, a[:3]])          # 65539 elements: every pair lands in every byte position somewhere
+    b = np.concatenate([b, b[:3]])
+    a = np.concatenate([np.roll(a, s) for s in range(4)])
+    b = np.concatenate([np.roll(b, s) for s in range(4)])
+    srcs = [a.astype(np.uint8).view(npdt)] + [b.astype(np.uint8).view(npdt)] * (k - 1)
+    av, bv = srcs[0].astype(np.int64), srcs[1].astype(np.int64)
+
+    def wrap(x):
+        return (x & 0xFF).astype(np.uint8).view(npdt)
+
+    total = av + (k - 1) * bv
+    wrapped_sum = wrap(total).astype(np.int64)
+    kk = np.int64(np.array(k).astype(npdt))
+    quotient = np.abs(wrapped_sum) // abs(kk) * np.sign(wrapped_sum) * np.sign(kk)   # C division truncates
+    prod = av.copy()
+    for _ in range(k - 1):
+        prod = (prod * bv) & 0xFF
+    want = {O.SUM: wrap(total), O.PROD: wrap(prod), O.MAX: np.maximum(av, bv).astype(npdt),
+            O.MIN: np.minimum(av, bv).astype(npdt), O.AVG: quotient.astype(npdt)}
+    for op in ALL_OPS:
+        got = gpu_reduce(L, srcs, dt, op)
+        assert same(got, want[op]), (DT_NAME[dt], OP_NAME[op], k)
