@@ -195,6 +195,9 @@ struct Fold8 {
   }
 };
 
+// a 16-byte vector at any byte address (the hardware's unaligned access mode serves it)
+typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
+
 // Fold one 16-byte vector position across K registers.
 template <typename T, int OP, int K>
 __device__ __forceinline__ u32x4 foldVec(const u32x4 (&in)[K], int k) {
@@ -511,61 +514,6 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3))) re
     __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
         (void *)((char *)p.dst + headBytes + off), 0, span, kRsrcFlags);
     __builtin_amdgcn_raw_buffer_store_b128(r.v, rd, voff, 0, kStoreAux);
-  }
-  if (blockIdx.x == gridDim.x - 1) {
-    const uint64_t edge = p.head + p.tail;
-    if (threadIdx.x < edge) {
-      uint64_t i = threadIdx.x < p.head ? threadIdx.x : p.head + p.nvec * N + (threadIdx.x - p.head);
-      foldScalar<T, OP>(p.src, k, p.dst, i);
-    }
-  }
-}
-
-// More than eight sources that do not share the destination's address modulo 16,
-// 8-byte elements (the others take reduceWaveShiftAnyKernel).  The tiling is
-// the destination's (aligned 16-byte stores after p.head elements); each source
-// is read with 16-byte loads at whatever byte offset it happens to have, which
-// the hardware's unaligned access mode serves from at most one extra cache line
-// per wavefront request.  Plain global loads: a clipped buffer descriptor would
-// need an aligned base.
-typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
-
-template <typename T, int OP>
-__global__ void __launch_bounds__(64) reduceWaveUnalignedKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
-  typedef Fold<T, OP> F;
-  constexpr int N = 16 / sizeof(T);
-  constexpr int B = 8;
-  const int k = p.k; // >= B
-  const uint64_t ntiles = (p.nvec + 63) / 64;
-  const uint64_t headBytes = p.head * sizeof(T);
-  for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const uint64_t i = t * 64 + threadIdx.x;
-    if (i < p.nvec) {
-      Carry<T, OP> acc;
-      u32x4 in[B];
-      int j0 = 0;
-      for (; j0 + B <= k; j0 += B) {
-#pragma unroll
-        for (int b = 0; b < B; b++)
-          in[b] = __builtin_nontemporal_load(
-              (const u32x4_unaligned *)((const char *)p.src[j0 + b] + headBytes + i * 16));
-        if (j0 == 0) foldBatch<T, OP, B, true>(in, acc);
-        else foldBatch<T, OP, B, false>(in, acc);
-      }
-      const int rest = k - j0;
-      if (rest > 0) {
-#pragma unroll
-        for (int b = 0; b < B - 1; b++)
-          if (b < rest)
-            in[b] = __builtin_nontemporal_load(
-                (const u32x4_unaligned *)((const char *)p.src[j0 + b] + headBytes + i * 16));
-        foldRest<T, OP>(in, acc, rest);
-      }
-      Vec16<T> r;
-#pragma unroll
-      for (int e = 0; e < N; e++) r.e[e] = F::fin(acc.get(e), k);
-      *(u32x4 *)((char *)p.dst + headBytes + i * 16) = r.v;
-    }
   }
   if (blockIdx.x == gridDim.x - 1) {
     const uint64_t edge = p.head + p.tail;

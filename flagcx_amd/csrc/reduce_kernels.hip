@@ -183,16 +183,14 @@ static int launchAny(const ReduceCall &c, const Split &s) {
     return (int)hipGetLastError();
   }
   // More than eight sources at another offset modulo 16 than the output (up to eight
-  // take reduceWaveShiftKernel).  Measured at 128 MiB per source, 9 / 16 / 32 sources,
-  // percent of peak: 8-byte elements (the offset can only be 8) read with unaligned
-  // 16-byte loads 72 / 71 / 70, with aligned loads and lane shifts 74 / 68 / 66;
-  // 4-byte elements 72 / 71 / 70 against 75 / 72 / 72; 2- and 1-byte elements, whose
-  // offsets need not be a multiple of four, 61 / 58 / 55 against 72-77 / 72-75 / 70-72.
-  // The lane-shift kernel takes four sources at a time and wants every wavefront its
-  // registers allow (no cap: 12 per CU gave 53-59 %, 16 62-71 %, 25 and more 70-75 %).
-  if constexpr (sizeof(elem_t) == 8) {
-    reduceWaveUnalignedKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), ldsReservation(waves), c.stream>>>(p);
-  } else {
+  // take reduceWaveShiftKernel): aligned loads and lane shifts, four sources at a time.
+  // The kernel wants every wavefront its registers allow (no cap: 12 per CU gave
+  // 53-59 % of peak, 16 62-71 %, 25 and more 70-77 %, at 9..32 sources of 128 MiB).
+  // Unaligned 16-byte loads instead, measured beside it: 55-61 % on 1- and 2-byte
+  // elements at offsets that are no multiple of four, 70-73 % on 4- and 8-byte
+  // elements at 128 MiB, 66-70 % at 500 MiB and 56-59 % there when the output is one of
+  // the sources, where the lane shifts hold 71-79 %.
+  {
     ShiftParams<FLAGCX_MAX_RANKS> q;
     const uint64_t headBytes = s.head * sizeof(elem_t);
     for (int j = 0; j < FLAGCX_MAX_RANKS; j++) {

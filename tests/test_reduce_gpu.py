@@ -477,9 +477,8 @@ def test_fp16_fold_rounds_in_fp32_before_it_rounds_to_fp16(L, op, k):
 @pytest.mark.parametrize("op", ALL_OPS, ids=lambda o: OP_NAME[o])
 def test_more_than_eight_inputs_every_batch_remainder(L, dt, op):
     """More than eight inputs are folded in batches (eight at a time where every source
-    shares the output's address modulo 16, four at a time through lane shifts otherwise,
-    unaligned loads for 8-byte elements): every length of the last batch, with the
-    inputs aligned, all at one other offset, and each at an offset of its own."""
+    shares the output's address modulo 16, four at a time through lane shifts otherwise):
+    every length of the last batch, with the inputs aligned, all at one other offset, and each at an offset of its own."""
     import torch
     ts = O.type_size(dt)
     per16 = 16 // ts
