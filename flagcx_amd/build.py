@@ -34,6 +34,19 @@ def _run(cmd):
     return r
 
 
+def _no_spills(src, defs, remarks):
+    """The kernels are sized to run out of registers alone: a kernel that the compiler gave a scratch
+    segment (spilled registers, a stack) streams at a fraction of its rate, so the build stops there."""
+    name = None
+    for line in remarks.splitlines():
+        if "remark: Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line:
+            n = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
+            if n:
+                raise RuntimeError("%s %s: kernel %s uses %d bytes of scratch per lane" % (src, " ".join(defs), name, n))
+
+
 def build(verbose=False, jobs=None):
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
@@ -57,7 +70,8 @@ def build(verbose=False, jobs=None):
             pre = defs
         else:
             post = defs
-        _run([HIPCC] + FLAGS + post + ["-c"] + pre + [src, "-o", obj])
+        r = _run([HIPCC] + FLAGS + post + ["-Rpass-analysis=kernel-resource-usage", "-c"] + pre + [src, "-o", obj])
+        _no_spills(src, post, r.stderr)
         return obj
 
     jobs = jobs or min(8, os.cpu_count() or 4)
