@@ -8,7 +8,8 @@
 // descriptors are clipped to the tile, so ragged chunk ends need no branches.
 // A contiguous copy whose two sides differ modulo 16 goes to the one-input reduce
 // kernel for misaligned sources (aligned loads, lane shifts); strided forms whose chunk
-// sizes or strides are not multiples of 16 go through an element path at the
+// sizes or strides are not multiples of 16 split every chunk that way on its own
+// (copyWaveRaggedKernel), chunks under a KiB go through an element path at the
 // widest width every address shares.
 // HBM bound: 2 bytes of traffic per payload byte (1 for fills); no LDS, no MFMA.
 #include "launch.h"
@@ -19,6 +20,8 @@ namespace flagcx_amd {
 constexpr int kCopyUnroll = 1;
 constexpr uint64_t kMaxGridX = 1u << 24;
 constexpr uint64_t kMaxGridY = 65535;
+// chunks shorter than this stay on the element path (a chunk's 16-byte body would be a few vectors)
+constexpr uint64_t kRaggedMinBytes = 1024;
 
 struct CopyParams {
   const char *src;
@@ -86,6 +89,66 @@ __global__ void __launch_bounds__(64) copyWaveListKernel(CopyParams p, ListParam
   copyWaveBody<U, LIST, TILED>(p, &l);
 }
 
+// Several chunks whose sizes, strides or bases are not multiples of 16: every chunk is
+// split on its own into the bytes up to the destination's next 16-byte line, a body of
+// 16-byte vectors stored aligned (first tile cut short at a cache line, as above), and
+// the bytes after it.  A source body at another offset modulo 16 than its destination is
+// read with aligned loads, one granule further than the tile, and put in place with lane
+// shifts, as reduceWaveShiftKernel does for its sources.
+template <int LIST>
+__device__ __forceinline__ void copyWaveRaggedBody(const CopyParams &p, const ListParams *l) {
+  const uint32_t lane = threadIdx.x;
+  for (uint64_t c = blockIdx.y; c < p.nchunks; c += gridDim.y) {
+    const char *s = LIST == 1 ? l->src[c] : p.src + c * p.srcStride;
+    char *d = LIST == 2 ? l->dst[c] : p.dst + c * p.dstStride;
+    uint64_t head = (16u - ((uintptr_t)d & 15u)) & 15u;
+    if (head > p.chunkBytes) head = p.chunkBytes;
+    const uint64_t body = (p.chunkBytes - head) & ~15ull;
+    const uint64_t tail = p.chunkBytes - head - body;
+    const char *sb = s + head;
+    char *db = d + head;
+    const uint32_t lead = (uint32_t)((uintptr_t)db & 127u);
+    const uint32_t shift = (uint32_t)((uintptr_t)sb & 15u);
+    const char *base = sb - shift;                               // aligned granules that hold the body
+    const uint64_t granules = body ? body / 16 + (shift ? 1 : 0) : 0;
+    const uint64_t ntiles = (body + lead + 1023) / 1024;
+    for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+      const uint64_t off = t ? t * 1024 - lead : 0;
+      const uint64_t left = body - off;
+      const uint32_t cap = t ? 1024u : 1024u - lead;
+      const uint32_t span = left < cap ? (uint32_t)left : cap;
+      const uint64_t g0 = off / 16;
+      const uint64_t leftG = granules > g0 ? granules - g0 : 0;
+      __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+          (void *)(base + g0 * 16), 0, (uint32_t)(leftG < 64 ? leftG : 64) * 16u, kRsrcFlags);
+      u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16u, 0, kLoadAux);
+      if (shift) { // the same for every lane of the chunk
+        __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(base + g0 * 16 + 1024), 0, leftG > 64 ? 16u : 0u, kRsrcFlags);
+        const u32x4 ahead = __builtin_amdgcn_raw_buffer_load_b128(ra, lane * 16u, 0, kLoadAux);
+        u32x4 hi;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+          const uint32_t fromNext = __builtin_amdgcn_readfirstlane(ahead[w]); // granule 0 of the next tile
+          hi[w] = (uint32_t)__builtin_amdgcn_update_dpp((int)fromNext, (int)v[w], 0x130, 0xf, 0xf, false);
+        }
+        v = funnel16(v, hi, shift >> 2, shift & 3u);
+      }
+      __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc((void *)(db + off), 0, span, kRsrcFlags);
+      __builtin_amdgcn_raw_buffer_store_b128(v, rd, lane * 16u, 0, kStoreAux);
+    }
+    // the chunk's bytes before and after its body: fewer than 32, one lane each
+    if (blockIdx.x == gridDim.x - 1 && lane < head + tail) {
+      const uint64_t i = lane < head ? lane : head + body + (lane - head);
+      d[i] = s[i];
+    }
+  }
+}
+template <int LIST>
+__global__ void __launch_bounds__(64) copyWaveRaggedKernel(CopyParams p, ListParams l) {
+  copyWaveRaggedBody<LIST>(p, &l);
+}
+
 // Element path: W-byte units, chunk by chunk.
 template <typename W, int LIST>
 __device__ __forceinline__ void copyElemBody(const CopyParams &p, const ListParams *l) {
@@ -131,6 +194,12 @@ static int launchCopyT(const CopyParams &p, const ListParams &l, bool vector, un
       if (onLines) copyWaveListKernel<kCopyUnroll, LIST, false><<<grid, dim3(64), lds, stream>>>(p, l);
       else copyWaveListKernel<kCopyUnroll, LIST, true><<<grid, dim3(64), lds, stream>>>(p, l);
     }
+    return (int)hipGetLastError();
+  }
+  if (p.nchunks > 1 && p.chunkBytes >= kRaggedMinBytes) {
+    uint64_t gx = (p.chunkBytes + 127 + 1023) / 1024 + 1; // tiles of the longest possible body, cut at a line
+    if (gx > kMaxGridX) gx = kMaxGridX;
+    copyWaveRaggedKernel<LIST><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), ldsReservation(launchShapeFor(0, 0).waves), stream>>>(p, l);
     return (int)hipGetLastError();
   }
   uint64_t gx = (p.chunkBytes / width + 255) / 256;

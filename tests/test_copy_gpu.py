@@ -106,6 +106,63 @@ def test_pack_unpack_round_trip(L, chunk, stride):
         assert same(from_dev(back, np.uint8), wantb), (chunk, stride, base)
 
 
+@pytest.mark.parametrize("nch,cb,gap,so,do", [
+    (37, 4099, 3, 5, 9),        # nothing is a multiple of 16: every chunk has head and tail bytes of its own, sources shifted
+    (64, 1024, 1, 0, 1),        # the shortest chunks that take the vector body
+    (64, 70001, 0, 3, 3),       # contiguous chunks, both sides at the same odd offset
+    (200, 2049, 77, 1, 2),
+    (3, 1 << 20, 16, 8, 0),     # 16-byte strides, the two sides 8 bytes apart
+    (9, 1023, 5, 7, 11),        # under a KiB: the element path
+])
+def test_pack_unpack_ragged_chunks(L, nch, cb, gap, so, do):
+    """Strided chunks whose size, stride and bases are no multiples of 16: packed, and unpacked
+    again at another stride, byte-exact against numpy slices, guard bytes untouched."""
+    import torch
+    stride = cb + gap
+    sparse_h = rand_bytes(so + nch * stride + 64, nch * 131 + cb)
+    want = np.concatenate([sparse_h[so + i * stride:so + i * stride + cb] for i in range(nch)])
+    sparse = to_dev(sparse_h)
+    packed = torch.full((do + nch * cb + 64,), 0xAB, dtype=torch.uint8, device="cuda")
+    L.pack(packed.data_ptr() + do, sparse.data_ptr() + so, nch, cb, stride)
+    torch.cuda.synchronize()
+    got = from_dev(packed, np.uint8)
+    assert same(got[do:do + nch * cb], want)
+    assert (got[:do] == 0xAB).all() and (got[do + nch * cb:] == 0xAB).all()
+    stride2 = cb + 2 * gap + 1
+    out = torch.full((so + nch * stride2 + 64,), 0xCD, dtype=torch.uint8, device="cuda")
+    L.unpack(out.data_ptr() + so, packed.data_ptr() + do, nch, cb, stride2)
+    torch.cuda.synchronize()
+    got = from_dev(out, np.uint8)
+    expect = np.full(got.shape, 0xCD, np.uint8)
+    for i in range(nch):
+        expect[so + i * stride2:so + i * stride2 + cb] = want[i * cb:(i + 1) * cb]
+    assert same(got, expect)
+
+
+def test_pack_list_and_unpack_list_of_64_ragged_entries(L):
+    """The most entries a list takes, each at a position of its own inside a cache line."""
+    import torch
+    n, cb = 64, 5003
+    rng = np.random.default_rng(64)
+    offs = [int(x) for x in rng.integers(0, 128, n)]
+    hosts = [rand_bytes(cb + 256, 900 + i) for i in range(n)]
+    want = np.concatenate([hosts[i][offs[i]:offs[i] + cb] for i in range(n)])
+    srcs = [to_dev(h) for h in hosts]
+    packed = torch.full((n * cb + 64,), 0xAB, dtype=torch.uint8, device="cuda")
+    L.pack_list(packed.data_ptr() + 3, [s.data_ptr() + o for s, o in zip(srcs, offs)], cb)
+    torch.cuda.synchronize()
+    got = from_dev(packed, np.uint8)
+    assert same(got[3:3 + n * cb], want) and (got[:3] == 0xAB).all() and (got[3 + n * cb:] == 0xAB).all()
+    dsts = [torch.full((cb + 256,), 0xCD, dtype=torch.uint8, device="cuda") for _ in range(n)]
+    offs2 = [int(x) for x in rng.integers(0, 128, n)]
+    L.unpack_list([d.data_ptr() + o for d, o in zip(dsts, offs2)], packed.data_ptr() + 3, cb)
+    torch.cuda.synchronize()
+    for i, d in enumerate(dsts):
+        g = from_dev(d, np.uint8)
+        assert same(g[offs2[i]:offs2[i] + cb], want[i * cb:(i + 1) * cb]), i
+        assert (g[:offs2[i]] == 0xCD).all() and (g[offs2[i] + cb:] == 0xCD).all(), i
+
+
 @pytest.mark.parametrize("nbytes", [16, 1000, 4096, 65536 + 16, 333])
 def test_pack_list_and_unpack_list(L, nbytes):
     import torch
