@@ -421,8 +421,9 @@ struct Carry<T, OP, false> {
   __device__ __forceinline__ void set(int e, acc_t x) { a[e] = x; }
 };
 
-template <typename T, int OP, int C, bool FIRST>
-__device__ __forceinline__ void foldBatch(const u32x4 (&in)[8], Carry<T, OP> &acc) {
+template <typename T, int OP, int C, bool FIRST, int NI>
+__device__ __forceinline__ void foldBatch(const u32x4 (&in)[NI], Carry<T, OP> &acc) {
+  static_assert(C >= 1 && C <= NI, "a batch folds the first C of the NI vectors");
   typedef Fold<T, OP> F;
   if constexpr (sizeof(T) == 1) {
     typedef Fold8<T, OP> F8;
@@ -450,25 +451,32 @@ __device__ __forceinline__ void foldBatch(const u32x4 (&in)[8], Carry<T, OP> &ac
   }
 }
 
-template <typename T, int OP>
-__device__ __forceinline__ void foldRest(const u32x4 (&in)[8], Carry<T, OP> &acc, int rest) {
-  switch (rest) { // wave-uniform
-    case 1: foldBatch<T, OP, 1, false>(in, acc); break;
-    case 2: foldBatch<T, OP, 2, false>(in, acc); break;
-    case 3: foldBatch<T, OP, 3, false>(in, acc); break;
-    case 4: foldBatch<T, OP, 4, false>(in, acc); break;
-    case 5: foldBatch<T, OP, 5, false>(in, acc); break;
-    case 6: foldBatch<T, OP, 6, false>(in, acc); break;
-    case 7: foldBatch<T, OP, 7, false>(in, acc); break;
-    default: break;
+// One batch of the aligned kernel for more than eight inputs: C loads, then their fold.
+// INFLIGHT as in reduceWaveBody: the next input is asked for when at most that many
+// earlier ones are outstanding (0: all at once).
+template <typename T, int OP, int C, bool FIRST>
+__device__ __forceinline__ void anyBatch(const ReduceParams<FLAGCX_MAX_RANKS> &p, int j0, uint64_t byteOff, uint32_t span,
+                                         uint32_t voff, Carry<T, OP> &acc) {
+  u32x4 in[C];
+#pragma unroll
+  for (int b = 0; b < C; b++) {
+    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const char *)p.src[j0 + b] + byteOff), 0, span, kRsrcFlags);
+    in[b] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kLoadAux);
+    if (b + 1 < C && p.inflight) {
+      if (p.inflight == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | 1);
+      else if (p.inflight == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | 0);
+      else __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
+    }
   }
+  foldBatch<T, OP, C, FIRST>(in, acc);
 }
 
 // Aligned body, k from 8 up to FLAGCX_MAX_RANKS, same streaming shape as above: one
 // wavefront per workgroup, one KiB of every input per tile.
-// (At most 168 registers: twelve wavefronts per CU, the most its launcher asks for.)
+// (At most 128 registers: sixteen wavefronts per CU, the most its launcher asks for.)
 template <typename T, int OP>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3))) reduceWaveAnyKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) reduceWaveAnyKernel(ReduceParams<FLAGCX_MAX_RANKS> p) {
   typedef Fold<T, OP> F;
   constexpr int N = 16 / sizeof(T);
   constexpr int B = 8;
@@ -485,28 +493,19 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3))) re
     const uint32_t cap = t ? kTileBytes : kTileBytes - lead;
     const uint32_t span = left < cap ? (uint32_t)left : cap;
     Carry<T, OP> acc;
-    u32x4 in[B];
-    int j0 = 0;
-    for (; j0 + B <= k; j0 += B) {
-#pragma unroll
-      for (int b = 0; b < B; b++) {
-        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)((const char *)p.src[j0 + b] + headBytes + off), 0, span, kRsrcFlags);
-        in[b] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kLoadAux);
-      }
-      if (j0 == 0) foldBatch<T, OP, B, true>(in, acc);
-      else foldBatch<T, OP, B, false>(in, acc);
-    }
-    const int rest = k - j0;
-    if (rest > 0) {
-#pragma unroll
-      for (int b = 0; b < B - 1; b++)
-        if (b < rest) {
-          __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-              (void *)((const char *)p.src[j0 + b] + headBytes + off), 0, span, kRsrcFlags);
-          in[b] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, kLoadAux);
-        }
-      foldRest<T, OP>(in, acc, rest);
+    const uint64_t at = headBytes + off;
+    anyBatch<T, OP, B, true>(p, 0, at, span, voff, acc);
+    int j0 = B;
+    for (; j0 + B <= k; j0 += B) anyBatch<T, OP, B, false>(p, j0, at, span, voff, acc);
+    switch (k - j0) { // what is left, the same for every wavefront
+      case 1: anyBatch<T, OP, 1, false>(p, j0, at, span, voff, acc); break;
+      case 2: anyBatch<T, OP, 2, false>(p, j0, at, span, voff, acc); break;
+      case 3: anyBatch<T, OP, 3, false>(p, j0, at, span, voff, acc); break;
+      case 4: anyBatch<T, OP, 4, false>(p, j0, at, span, voff, acc); break;
+      case 5: anyBatch<T, OP, 5, false>(p, j0, at, span, voff, acc); break;
+      case 6: anyBatch<T, OP, 6, false>(p, j0, at, span, voff, acc); break;
+      case 7: anyBatch<T, OP, 7, false>(p, j0, at, span, voff, acc); break;
+      default: break;
     }
     Vec16<T> r;
 #pragma unroll
@@ -684,7 +683,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) re
               (void *)((const char *)p.base[j] + g0 * 16 + 1024), 0, left > 64 ? 16u : 0u, kRsrcFlags);
           ahead[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, lane * 16u, 0, kLoadAux);
         }
-      u32x4 in[8];
+      u32x4 in[B];
 #pragma unroll
       for (int i = 0; i < B; i++)
         if (i < c) {

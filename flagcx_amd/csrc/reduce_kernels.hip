@@ -154,7 +154,7 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   p.head = s.head;
   p.tail = s.tail;
   p.k = c.k;
-  p.inflight = 0;
+  p.inflight = tunedLoadsInFlight(8) >= 0 ? tunedLoadsInFlight(8) : 2;
   p.lead = 0;
   p.run = 1;
   if (s.vector && s.nvec) {
@@ -171,13 +171,16 @@ static int launchAny(const ReduceCall &c, const Split &s) {
   uint64_t tiles = (s.nvec * 16 + p.lead + 1023) / 1024;
   if (tiles < 1) tiles = 1;
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  // more than eight inputs are loaded eight at a time; measured on MI355X: 9..10
-  // inputs want 12 wavefronts per CU (88 % of peak against 79 % at 8), 11..13 want
-  // 10, more want 8 (85-86 %).  An explicit flagcxLocalTune(8, n) overrides.
-  // (A limit on the inputs in flight, as the kernels for up to eight inputs have
-  // it, gains nothing here: within one percent for 9..32 inputs.)
+  // More than eight inputs are loaded eight at a time, each batch paced like the kernels
+  // for up to eight: the next input is asked for when at most one earlier one is
+  // outstanding, 16 wavefronts per CU up to 160 MiB per input and 14 above.  Measured on
+  // MI355X, fp32 and bf16, 9 / 12 / 16 / 32 inputs, percent of peak: 128 MiB per input
+  // 85 / 85 / 84 / 83, 256 MiB 85 / 83 / 81 / 80, 512 MiB 82 / 80 / 82 / 80; all eight
+  // loads at once with 12 / 10 / 8 wavefronts (the best caps for that) gave 86 / 84 / 84 /
+  // 82, 80 / 79 / 77 / 76 and 80 / 79 / 75 / 77.  flagcxLocalTune(8, n) and
+  // flagcxLocalTuneLoads(8, n) override.
   const int tuned = tunedWavesPerCU(8);
-  const int waves = tuned >= 0 ? tuned : c.k <= 10 ? 12 : c.k <= 13 ? 10 : 8;
+  const int waves = tuned >= 0 ? tuned : tiles > 160 * 1024 ? 14 : 16;
   if (s.vector) {
     reduceWaveAnyKernel<elem_t, OP><<<dim3((unsigned)tiles), dim3(64), ldsReservation(waves), c.stream>>>(p);
     return (int)hipGetLastError();

@@ -153,6 +153,9 @@ flagcxResult_t flagcxLocalPlaceBuffers(void *pool, size_t poolbytes, size_t byte
  * one or two from 16-96 MiB per input on (from 16 MiB with five and more inputs,
  * 32 MiB with three or four, 96 MiB with two), where 14-25 wavefronts per CU each
  * waiting for its previous input keep DRAM busier than bursts of all inputs.
+ * Reduces of more than eight inputs (loaded eight at a time) take the settings of
+ * nranks == 8; their defaults are two inputs in flight with 16 wavefronts per CU up
+ * to 160 MiB per input and 14 above.
  * The settings belong to the calling thread: they shape the launches that thread
  * makes afterwards and nobody else's.  flagcxLocalInit checks once that the device
  * hands out LDS the way the caps assume (else no cap is applied). */
