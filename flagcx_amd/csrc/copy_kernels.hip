@@ -9,7 +9,7 @@
 // A contiguous copy whose two sides differ modulo 16 goes to the one-input reduce
 // kernel for misaligned sources (aligned loads, lane shifts); strided forms whose chunk
 // sizes or strides are not multiples of 16 split every chunk that way on its own
-// (copyWaveRaggedKernel), chunks under a KiB go through an element path at the
+// (copyWaveRaggedKernel), chunks under 320 bytes go through an element path at the
 // widest width every address shares.
 // HBM bound: 2 bytes of traffic per payload byte (1 for fills); no LDS, no MFMA.
 #include "launch.h"
@@ -20,8 +20,9 @@ namespace flagcx_amd {
 constexpr int kCopyUnroll = 1;
 constexpr uint64_t kMaxGridX = 1u << 24;
 constexpr uint64_t kMaxGridY = 65535;
-// chunks shorter than this stay on the element path (a chunk's 16-byte body would be a few vectors)
-constexpr uint64_t kRaggedMinBytes = 1024;
+// chunks shorter than this stay on the element path (200 000 misaligned chunks of 200 / 500 / 1000 bytes:
+// element path 20 / 26 / 17 % of peak, a workgroup per chunk that splits it 16 / 38 / 55 %)
+constexpr uint64_t kRaggedMinBytes = 320;
 
 struct CopyParams {
   const char *src;
@@ -30,6 +31,7 @@ struct CopyParams {
   uint64_t head; // bytes before the 16-byte body (single-chunk case only)
   uint64_t body; // bytes in the body of each chunk
   uint64_t tail; // bytes after the body (single-chunk case only)
+  uint32_t flat; // copyWaveRaggedKernel: one workgroup per chunk, blockIdx.x walks the chunks
 };
 
 struct ListParams {
@@ -98,7 +100,11 @@ __global__ void __launch_bounds__(64) copyWaveListKernel(CopyParams p, ListParam
 template <int LIST>
 __device__ __forceinline__ void copyWaveRaggedBody(const CopyParams &p, const ListParams *l) {
   const uint32_t lane = threadIdx.x;
-  for (uint64_t c = blockIdx.y; c < p.nchunks; c += gridDim.y) {
+  // chunks by blockIdx.y and a chunk's tiles by blockIdx.x, or (p.flat, short chunks) chunks by
+  // blockIdx.x, which may be longer than the 65535 a grid allows in y, and all tiles of a chunk in turn
+  const uint64_t c0 = p.flat ? blockIdx.x : blockIdx.y, cStep = p.flat ? gridDim.x : gridDim.y;
+  const uint64_t t0 = p.flat ? 0 : blockIdx.x, tStep = p.flat ? 1 : gridDim.x;
+  for (uint64_t c = c0; c < p.nchunks; c += cStep) {
     const char *s = LIST == 1 ? l->src[c] : p.src + c * p.srcStride;
     char *d = LIST == 2 ? l->dst[c] : p.dst + c * p.dstStride;
     uint64_t head = (16u - ((uintptr_t)d & 15u)) & 15u;
@@ -112,7 +118,7 @@ __device__ __forceinline__ void copyWaveRaggedBody(const CopyParams &p, const Li
     const char *base = sb - shift;                               // aligned granules that hold the body
     const uint64_t granules = body ? body / 16 + (shift ? 1 : 0) : 0;
     const uint64_t ntiles = (body + lead + 1023) / 1024;
-    for (uint64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    for (uint64_t t = t0; t < ntiles; t += tStep) {
       const uint64_t off = t ? t * 1024 - lead : 0;
       const uint64_t left = body - off;
       const uint32_t cap = t ? 1024u : 1024u - lead;
@@ -138,7 +144,7 @@ __device__ __forceinline__ void copyWaveRaggedBody(const CopyParams &p, const Li
       __builtin_amdgcn_raw_buffer_store_b128(v, rd, lane * 16u, 0, kStoreAux);
     }
     // the chunk's bytes before and after its body: fewer than 32, one lane each
-    if (blockIdx.x == gridDim.x - 1 && lane < head + tail) {
+    if ((p.flat || blockIdx.x == gridDim.x - 1) && lane < head + tail) {
       const uint64_t i = lane < head ? lane : head + body + (lane - head);
       d[i] = s[i];
     }
@@ -197,9 +203,31 @@ static int launchCopyT(const CopyParams &p, const ListParams &l, bool vector, un
     return (int)hipGetLastError();
   }
   if (p.nchunks > 1 && p.chunkBytes >= kRaggedMinBytes) {
-    uint64_t gx = (p.chunkBytes + 127 + 1023) / 1024 + 1; // tiles of the longest possible body, cut at a line
+    // Workgroups per chunk.  Every workgroup pays for the split of its chunk, so short chunks
+    // (up to 16 tiles) get one workgroup each, and a launch of up to 320 MiB in all gives each
+    // workgroup about two tiles; beyond that one tile per workgroup, as the other movers have it.
+    // Measured on MI355X, misaligned packs, percent of peak: 200 000 chunks of 1 / 1.5 / 4 / 9 KB
+    // 54 / 58 / 40 / 62 with a workgroup per tile, 68 / 72 / 76 / 80 with one per chunk; 64 KiB
+    // - 64 MiB chunks, 256 MiB in all: 66-75 with a workgroup per tile, 80-84 with two tiles each;
+    // 1 GiB in all: 78-79 against 70-74 (four tiles each).
+    const uint64_t perChunk = (p.chunkBytes + 127 + 1023) / 1024 + 1; // tiles of the longest possible body, cut at a line
+    uint64_t gx = perChunk;
+    CopyParams q = p;
+    uint64_t gyr = gy;
+    if (perChunk <= 16) {
+      q.flat = 1;
+      gx = p.nchunks < kMaxGridX ? p.nchunks : kMaxGridX;
+      gyr = 1;
+    } else {
+      const uint64_t all = perChunk * p.nchunks;
+      const uint64_t target = all <= 160 * 1024 ? 65536 : all <= 320 * 1024 ? 131072 : 0;
+      if (target) {
+        const uint64_t most = target / gy ? target / gy : 1;
+        if (gx > most) gx = most;
+      }
+    }
     if (gx > kMaxGridX) gx = kMaxGridX;
-    copyWaveRaggedKernel<LIST><<<dim3((unsigned)gx, (unsigned)gy), dim3(64), ldsReservation(launchShapeFor(0, 0).waves), stream>>>(p, l);
+    copyWaveRaggedKernel<LIST><<<dim3((unsigned)gx, (unsigned)gyr), dim3(64), ldsReservation(launchShapeFor(0, 0).waves), stream>>>(q, l);
     return (int)hipGetLastError();
   }
   uint64_t gx = (p.chunkBytes / width + 255) / 256;

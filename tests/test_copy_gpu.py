@@ -112,7 +112,9 @@ def test_pack_unpack_round_trip(L, chunk, stride):
     (64, 70001, 0, 3, 3),       # contiguous chunks, both sides at the same odd offset
     (200, 2049, 77, 1, 2),
     (3, 1 << 20, 16, 8, 0),     # 16-byte strides, the two sides 8 bytes apart
-    (9, 1023, 5, 7, 11),        # under a KiB: the element path
+    (9, 1023, 5, 7, 11),        # one tile per chunk
+    (300, 321, 2, 3, 1),        # many chunks just long enough for the vector body, one workgroup each
+    (9, 300, 5, 7, 11),         # shorter than that: the element path
 ])
 def test_pack_unpack_ragged_chunks(L, nch, cb, gap, so, do):
     """Strided chunks whose size, stride and bases are no multiples of 16: packed, and unpacked
