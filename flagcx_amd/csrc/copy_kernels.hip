@@ -80,7 +80,7 @@ __device__ __forceinline__ void copyWaveBody(const CopyParams &p, const ListPara
   }
 }
 
-// The strided form carries 72 bytes of arguments; only the list forms pay for the
+// The strided form carries 80 bytes of arguments; only the list forms pay for the
 // pointer tables.
 template <int U, bool TILED>
 __global__ void __launch_bounds__(64) copyWaveKernel(CopyParams p) {
