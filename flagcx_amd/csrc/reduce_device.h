@@ -452,8 +452,8 @@ __device__ __forceinline__ void foldBatch(const u32x4 (&in)[NI], Carry<T, OP> &a
 }
 
 // One batch of the aligned kernel for more than eight inputs: C loads, then their fold.
-// INFLIGHT as in reduceWaveBody: the next input is asked for when at most that many
-// earlier ones are outstanding (0: all at once).
+// p.inflight as in reduceWaveBody: a wavefront keeps the loads of at most that many inputs
+// in flight before it asks for the next (0: the whole batch at once).
 template <typename T, int OP, int C, bool FIRST>
 __device__ __forceinline__ void anyBatch(const ReduceParams<FLAGCX_MAX_RANKS> &p, int j0, uint64_t byteOff, uint32_t span,
                                          uint32_t voff, Carry<T, OP> &acc) {
