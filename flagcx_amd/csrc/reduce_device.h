@@ -401,6 +401,7 @@ __global__ void __launch_bounds__(64) reduceBatchKernel(ReduceBatchParams<K> bp)
 // batch length a run-time bound instead, measured on MI355X at 9..16 inputs of
 // 128 MiB: 32-bit integer sum / min / max 65-69 % of the HBM peak and 8-bit min / max
 // 56-62 %, where the other types ran at 84-88 % and all do now.
+//
 // What travels from one batch to the next: the accumulators of one 16-byte position.
 // Where an accumulator has the size of an element (every type but the two 16-bit
 // floating-point ones) they travel packed in four registers, as the inputs do.
