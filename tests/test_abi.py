@@ -260,3 +260,18 @@ def test_device_adaptor_table_layout_and_slots():
     assert local.adaptor_fn(slots, "dmaSupport", C.c_int, C.POINTER(C.c_bool))(C.byref(flag)) == 0 and not flag.value
     assert local.adaptor_fn(slots, "eventElapsedTime", C.c_int, C.c_void_p, C.c_void_p, C.c_void_p)(None, None, None) == 4
     assert local.adaptor_fn(slots, "streamFree", C.c_int, C.c_void_p)(None) == 0
+
+
+def test_build_refuses_a_kernel_with_a_scratch_segment():
+    """The build reads the compiler's resource remarks and stops at a kernel that was given
+    scratch memory (spilled registers, a stack): the text of such a remark, and of a clean one."""
+    from flagcx_amd import build as B
+    tag = " [-Rpass-analysis=kernel-resource-usage]\n"
+    clean = ("k.hip:9:1: remark: Function Name: _Zfine" + tag +
+             "k.hip:9:1: remark:     VGPRs: 64" + tag +
+             "k.hip:9:1: remark:     ScratchSize [bytes/lane]: 0" + tag)
+    B._no_spills("k.hip", [], clean)
+    spilled = clean + ("k.hip:20:1: remark: Function Name: _Zspills" + tag +
+                       "k.hip:20:1: remark:     ScratchSize [bytes/lane]: 48" + tag)
+    with pytest.raises(RuntimeError, match="_Zspills uses 48 bytes of scratch"):
+        B._no_spills("k.hip", ["-DFLAGCX_DT=0"], spilled)
