@@ -122,7 +122,24 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   // a limit on the inputs in flight per wavefront trades latency per wavefront for
   // DRAM efficiency: by default only where the launch runs many rounds of resident
   // wavefronts
-  const LaunchShape shape = launchShapeFor(K, tiles);
+  LaunchShape shape = launchShapeFor(K, tiles);
+  // Buffers at different places inside their cache lines (tiles dealt out in runs per XCD):
+  // from 48 MiB per input on, two, four and five inputs do better with all loads at once, six
+  // and seven with one in flight and more wavefronts.  Measured on MI355X, every source at a
+  // place of its own, fp32 / bf16 at 128 MiB per input, percent of peak, shape of the aligned
+  // case -> this one: 2 inputs 84 / 78 -> 83 / 80, 4: 79 / 76 -> 86 / 86, 5: 78 / 75 -> 82 / 82,
+  // 6: 79 / 76 -> 81 / 76, 7: 77 / 73 -> 79 / 75 (384 MiB: +1 to +5 on the same rows); medians
+  // over random places, sizes and types: 82.0 -> 82.8, 80.6 -> 82.8, 77.7 -> 80.3, 80.2 ->
+  // 80.9, 78.9 -> 79.8.  Three inputs lost a point that way and eight gained nothing: both keep
+  // their shape, and so does a reduce whose output is one of its inputs (five inputs in place:
+  // 69 -> 61 %).  Explicit flagcxLocalTune* settings win.
+  bool inPlace = false;
+  for (int j = 0; j < K; j++) inPlace = inPlace || c.src[j] == c.dst;
+  if (p.run > 1 && tiles >= 48 * 1024 && K >= 2 && K <= 7 && K != 3 && !inPlace && tunedWavesPerCU(K) < 0 &&
+      tunedLoadsInFlight(K) < 0) {
+    shape.loads = K <= 5 ? 0 : 1;
+    shape.waves = K == 2 ? 25 : K <= 5 ? 18 : 25;
+  }
   p.inflight = shape.loads;
   if (tiles < 1) tiles = 1;
   if (p.run > 1) tiles = (tiles + 8ull * p.run - 1) / (8ull * p.run) * (8ull * p.run);
