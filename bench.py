@@ -580,7 +580,8 @@ POSITIONS = [("every buffer on a 128-byte line", lambda j, k: 0, 0),
              ("sources on a line, destination 16 bytes in", lambda j, k: 0, 16),
              ("sources 80 bytes in, destination 16 bytes in", lambda j, k: 80, 16),
              ("sources 2..14 bytes in (another offset modulo 16)", lambda j, k: 2 + 2 * (j % 7), 0),
-             ("the same, destination 16 bytes in", lambda j, k: 2 + 2 * (j % 7), 16)]
+             ("the same, destination 16 bytes in", lambda j, k: 2 + 2 * (j % 7), 16),
+             ("every source at a place of its own, dest. on a line", lambda j, k: 16 * ((3 * j) % 8), 0)]
 
 
 def table_positions(L, args):
