@@ -309,11 +309,19 @@ def c3_queue_ms(L, nranks, descs, warmup=5, iters=20):
                 if it >= warmup:
                     times.append((time.perf_counter() - t0) * 1e3)
             grid = fifo.grid()
+            # what a shard's wall clock holds beside the folding itself: one 4 KiB entry, enqueue -> Wait
+            small = []
+            for it in range(30):
+                t0 = time.perf_counter()
+                fifo._check(enq(fifo._h, arrs[0][0], nranks, arrs[0][1], 2048, C.byref(ticket)))
+                fifo.wait(ticket.value)
+                small.append((time.perf_counter() - t0) * 1e3)
+            small.sort()
     finally:
         fifo.close()
         lib.flagcxLocalSetMaxSpinCount(-1)
     times.sort()
-    return times[len(times) // 2], grid
+    return times[len(times) // 2], grid, small[len(small) // 2]
 
 
 def c3_gated_ms(L, nranks, descs, warmup=5, iters=20):
@@ -326,26 +334,32 @@ def c3_gated_ms(L, nranks, descs, warmup=5, iters=20):
     first = C.c_uint64()
     side = torch.cuda.Stream()
     st = L.Stream(side.cuda_stream)
-    times = []
+    times, dev = [], []
     torch.cuda.synchronize()
     lib.flagcxLocalSetMaxSpinCount(1 << 22)
     gate = L.Gate()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
     try:
         for it in range(warmup + iters):
             t0 = time.perf_counter()
+            e0.record(side)
             L.check(lib.flagcxLocalReduceBatchGated(gate._h, arr, len(descs), nranks, int(L.DataType.Float16),
                                                     int(L.RedOp.Avg), C.byref(st), C.byref(first)))
             for c in range(len(descs)):
                 lib.flagcxLocalGateOpen(gate._h, first.value + c + 1)
+            e1.record(side)
             side.synchronize()
             if it >= warmup:
                 times.append((time.perf_counter() - t0) * 1e3)
+                dev.append(e0.elapsed_time(e1))
         assert gate.query()[2] == 0, "the gated launch gave up waiting"
     finally:
         gate.destroy()
         lib.flagcxLocalSetMaxSpinCount(-1)
     times.sort()
-    return times[len(times) // 2]
+    dev.sort()
+    return times[len(times) // 2], dev[len(dev) // 2]
 
 
 def config_c3(L, full=False, separate=False):
@@ -360,20 +374,44 @@ def config_c3(L, full=False, separate=False):
     ms = timed_ms(lambda: L.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks))
     rows["C3_batch_32x4MiB"] = row(nb, ms, note="32 chunk descriptors, one batch call (needs every chunk present)")
     try:
-        ms, grid = c3_queue_ms(L, nranks, descs)
+        ms, grid, small_ms = c3_queue_ms(L, nranks, descs)
         rows["C3_queue_32x4MiB"] = row(nb, ms, note="chunk by chunk through the resident reduce queue, host wall clock "
-                                                    "first enqueue -> Wait; %d resident wavefronts" % grid)
+                                                    "first enqueue -> Wait; %d resident wavefronts" % grid,
+                                       one_4KiB_entry_enqueue_to_wait_ms=round(small_ms, 5),
+                                       frac_without_that_round_trip=round(
+                                           nb / ((ms - small_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4))
     except Exception as e:   # a row of its own: the others are measured all the same
         rows["C3_queue_32x4MiB"] = {"error": repr(e)}
     try:
-        ms = c3_gated_ms(L, nranks, descs)
+        ms, dev_ms = c3_gated_ms(L, nranks, descs)
         rows["C3_gated_batch_32x4MiB"] = row(nb, ms, note="one batch launched up front, a host store per chunk lets its "
-                                                          "wavefronts go; host wall clock launch -> stream sync")
+                                                          "wavefronts go; host wall clock launch -> stream sync",
+                                             device_ms=round(dev_ms, 5),
+                                             device_frac=round(nb / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                             device_note="between two events on the launch's stream, recorded before the "
+                                                         "launch call and behind it: without the host's wait for the stream")
     except Exception as e:
         rows["C3_gated_batch_32x4MiB"] = {"error": repr(e)}
     ms = timed_ms(lambda: L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE))
     rows["C3_per_chunk_launches"] = row(nb, ms, note="32 launches of 4 MiB chunks on one stream, %.2f us per launch"
                                                      % (ms * 1e3 / 32))
+    try:
+        # the 7 peers' slices staged through a 16 x 4 MiB ring on a second stream, as the proxies move them
+        ring_mem = torch.empty(L.CHUNKSIZE * 16 * (nranks - 1), dtype=torch.uint8, device="cuda")
+        ring = L.Ring(ring_mem, nranks - 1)
+        copy_t = torch.cuda.Stream()
+        staged = nb + 2 * (nranks - 1) * shard * 2
+        ms = timed_ms(lambda: ring.reduce_scatter(send, rank, recv, L.RedOp.Avg, L.Stream(copy_t.cuda_stream),
+                                                  L.current_stream()))
+        rows["C3_staging_ring_2_streams"] = row(nb, ms, hbm_bytes_incl_staging=staged,
+                                                hbm_gbps=round(staged / ms / 1e6, 1),
+                                                hbm_frac=round(staged / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                                                note="every peer slice is copied into a ring slot and read again by the "
+                                                     "reduce: 2.56 x the bytes of the fold alone")
+        ring.close()
+        del ring_mem
+    except Exception as e:
+        rows["C3_staging_ring_2_streams"] = {"error": repr(e)}
     if full:
         # the 32 chunk launches captured once into a HIP graph and replayed
         side = torch.cuda.Stream()
@@ -386,15 +424,11 @@ def config_c3(L, full=False, separate=False):
             L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE)
         rows["C3_per_chunk_launches_hip_graph"] = row(nb, timed_ms(graph.replay))
         del graph
-        # the 7 peers' slices staged through a 16 x 4 MiB ring on a second stream
         ring_mem = torch.empty(L.CHUNKSIZE * 16 * (nranks - 1), dtype=torch.uint8, device="cuda")
         ring = L.Ring(ring_mem, nranks - 1)
         copy_t = torch.cuda.Stream()
-        cs, ms_ = L.Stream(copy_t.cuda_stream), L.current_stream()
+        cs = L.Stream(copy_t.cuda_stream)
         staged = nb + 2 * (nranks - 1) * shard * 2
-        ms = timed_ms(lambda: ring.reduce_scatter(send, rank, recv, L.RedOp.Avg, cs, ms_))
-        rows["C3_staging_ring_2_streams"] = row(nb, ms, hbm_bytes_incl_staging=staged,
-                                                hbm_gbps=round(staged / ms / 1e6, 1))
         L.lib().flagcxLocalSetMaxSpinCount(1 << 22)
         fifo = L.ReduceFifo(64, nranks, L.DataType.Float16, L.RedOp.Avg)
         # a hardware queue of its own for the consumer: the copy stream must never wait behind it
@@ -454,6 +488,163 @@ def config_c4(L, separate=False):
     del bufs, pool
     torch.cuda.empty_cache()
     return rows
+
+
+def config_headline_variants(L, inputs):
+    """The headline fold under three conditions a caller may bring: nine ordinary allocations
+    (whatever addresses the allocator gives), sources two bytes further on than the destination
+    (chunk offsets are elemOffset * dtypeSize, flagcx/core/c2c_algo.cc:313-316, so sources need
+    not agree with the destination modulo 16), and sixteen inputs."""
+    import torch
+    rows = {}
+    n = N_ELEM
+    try:
+        bufs = [torch.empty(n, dtype=torch.bfloat16, device="cuda") for _ in range(K + 1)]
+        for j in range(K):
+            bufs[j].copy_(inputs[j])
+        ms = timed_ms(lambda: L.reduce(bufs[:K], bufs[K], L.RedOp.Sum))
+        rows["headline_allocator_layout"] = row(ALGO_BYTES, ms, note="nine separate torch allocations instead of "
+                                                                      "buffers placed by flagcxLocalPlaceBuffers")
+        del bufs
+        torch.cuda.empty_cache()
+    except Exception as e:
+        rows["headline_allocator_layout"] = {"error": repr(e)}
+    try:
+        pools, pool = placed(L, K + 1, n + 8, torch.bfloat16)
+        srcs = [pools[j][1:n + 1] for j in range(K)]            # + 2 bytes
+        dst = pools[K][:n]
+        for j in range(K):
+            srcs[j].copy_(inputs[j])
+        ms = timed_ms(lambda: L.reduce(srcs, dst, L.RedOp.Sum))
+        rows["headline_sources_plus_2_bytes"] = row(ALGO_BYTES, ms, note="every source 2 bytes past a 16-byte line, the "
+                                                                          "destination on one: aligned loads and lane shifts")
+        del pools, pool, srcs, dst
+        torch.cuda.empty_cache()
+    except Exception as e:
+        rows["headline_sources_plus_2_bytes"] = {"error": repr(e)}
+    try:
+        k16 = 16
+        bufs, pool = placed(L, k16 + 1, n, torch.bfloat16)
+        for j in range(k16):
+            bufs[j].copy_(inputs[j % K])
+        ms = timed_ms(lambda: L.reduce(bufs[:k16], bufs[k16], L.RedOp.Sum), warmup=3, iters=10)
+        rows["K16_bf16_sum_256MiB"] = row((k16 + 1) * n * 2, ms, note="sixteen inputs: two batches of eight loads, "
+                                                                      "accumulators kept in registers")
+        del bufs, pool
+        torch.cuda.empty_cache()
+    except Exception as e:
+        rows["K16_bf16_sum_256MiB"] = {"error": repr(e)}
+    return rows
+
+
+def config_plan_replay(L, mib=128, iters=10):
+    """C2C plan replay: the plan documents under tests/golden/plans (written by the reference's
+    plan DSL) replayed for all ranks on this GPU, the literal way (every refresh a zero-fill, every
+    collective reads all members) and the fused way (sums read the members that hold data).
+    `bytes` of both rows of a pair = the algorithmic bytes of the fused replay, i.e. what has to
+    move; `issued_bytes` = what that replay handed to the kernels."""
+    import torch
+    plans = os.path.join(ROOT, "tests", "golden", "plans")
+    rows = {}
+    cl8 = [0, 0, 0, 0, 1, 1, 1, 1]
+    n = mib * MiB // 4
+    for name, commop, scratch, algo in (("allreduce8", 6, False, 2), ("reducescatter8", 8, True, 0)):
+        try:
+            send = [torch.empty(n, dtype=torch.float32, device="cuda").uniform_(-1, 1) for _ in range(8)]
+            recv = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(8)]
+            scr = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(8)] if scratch else None
+            res, outs = {}, {}
+            for fused in (False, True):
+                plan = L.Plan(cl8, n, commop, L.RedOp.Sum)
+                plan.set_chunks(8)
+                plan.import_xml(os.path.join(plans, name))
+                plan.set_algorithm(algo)
+                plan.set_fused(fused)
+                args = ([t.data_ptr() for t in send], [t.data_ptr() for t in recv],
+                        [t.data_ptr() for t in scr] if scr else None, int(L.DataType.Float32))
+                ms = timed_ms(lambda: plan.execute(*args), warmup=2, iters=iters)
+                res[fused] = (ms,) + plan.traffic()
+                outs[fused] = [t[:n // 8 if commop == 8 else n].clone() for t in recv]
+                plan.close()
+            same = all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(outs[False], outs[True]))
+            need = res[True][1]
+            for fused, tag in ((False, "literal"), (True, "fused")):
+                ms, issued, launches = res[fused]
+                rows["plan_%s_%s" % (name, tag)] = row(need, ms, issued_bytes=int(issued), launches=int(launches),
+                                                       issued_gbps=round(issued / ms / 1e6, 1),
+                                                       issued_frac=round(issued / ms / 1e6 / HBM_PEAK_GBPS, 4))
+            rows["plan_%s_fused" % name]["same_bytes_as_literal"] = bool(same)
+            rows["plan_%s_fused" % name]["speedup_over_literal"] = round(res[False][0] / res[True][0], 3)
+            rows["plan_%s_literal" % name]["note"] = (
+                "8 ranks x %d MiB fp32, 2 clusters of 4, plan %s (algorithm %d)%s; bytes = what the fused replay moves"
+                % (mib, name, algo, ", scratch per rank" if scratch else ""))
+            del send, recv, scr, outs
+            torch.cuda.empty_cache()
+        except Exception as e:
+            rows["plan_%s_error" % name] = repr(e)
+    return rows
+
+
+def perf_driver(*argv, timeout=180):
+    """Lines of flagcx_amd/lib/local_perf (a C++ caller of the C ABI), or None with the reason logged."""
+    import subprocess
+    perf_bin = os.path.join(ROOT, "flagcx_amd", "lib", "local_perf")
+    if not os.path.exists(perf_bin):
+        return None
+    try:
+        r = subprocess.run([perf_bin] + list(argv), capture_output=True, text=True, timeout=timeout)
+        if r.returncode != 0:
+            log("bench.py: local_perf %s failed (%d): %s" % (" ".join(argv), r.returncode, r.stderr[-300:]))
+            return None
+        return r.stdout.splitlines()
+    except Exception as e:
+        log("bench.py: local_perf %s failed: %r" % (" ".join(argv), e))
+        return None
+
+
+def measured_ceiling():
+    """What this GPU's memory gives: read-only streams (the reduce kernels' shape without the
+    store stream), the library's fill, copy and 8-input sum at the same size, in one process."""
+    lines = perf_driver("-C", "1")
+    if not lines:
+        return None
+    out = {"unit": "GB/s", "bytes_walked_per_probe": 16 << 30,
+           "method": "flagcx_amd/lib/local_perf -C 1: bytes moved / time of 10 back-to-back launches between two HIP "
+                     "events after 3 warm-up launches, every probe over 16 GiB (64 x the memory-side cache, which holds part "
+                     "of a smaller walk whatever its order); the 8-input sum at the headline size over 4 sets of "
+                     "buffers; the read-only "
+                     "probe has the reduce kernels' shape without the store stream and is swept over 8 caps on resident "
+                     "wavefronts and 3 load pacings per stream count, best reported"}
+    for l in lines:
+        w = l.split()
+        if len(w) >= 3 and w[0] == "ceiling":
+            out[w[1]] = float(w[2])
+            if len(w) > 3:
+                out[w[1] + "_shape"] = " ".join(w[3:])
+    reads = [v for k, v in out.items() if k.startswith("read_only") and isinstance(v, float)]
+    if reads:
+        out["best_read_only"] = max(reads)
+    return out
+
+
+def latency_floor():
+    lines = perf_driver("-L", "1", "-n", "40")
+    if not lines:
+        return None
+    out = {"columns": "us per call: back to back between two events / one call between its own event pair / "
+                      "call -> hipStreamSynchronize / host time of the call while the stream is busy (medians; "
+                      "flagcx_amd/lib/local_perf -L 1)"}
+    for l in lines:
+        w = l.split()
+        if len(w) == 6 and w[0] == "floor":
+            out[w[1]] = {"back_to_back": float(w[2]), "single_between_events": float(w[3]), "launch_to_sync": float(w[4]),
+                         "host_call": float(w[5])}
+    if "library_reduce2_fp32" in out:
+        for other, key in (("empty_kernel_1x64", "library_above_empty_launch_back_to_back"),
+                           ("minimal_sum_kernel_4x64", "library_above_minimal_sum_kernel_back_to_back")):
+            if other in out:
+                out[key] = round(out["library_reduce2_fp32"]["back_to_back"] - out[other]["back_to_back"], 3)
+    return out
 
 
 def sweep_point(L, size, rotate, g):
@@ -535,7 +726,11 @@ def table_configs(L, args):
     rows.update(config_c1(L, args.allocator_layout)[0])
     rows.update(config_c3(L, full=True, separate=args.allocator_layout))
     rows.update(config_c4(L, args.allocator_layout))
+    rows.update(config_plan_replay(L))
     for name, r in rows.items():
+        if not isinstance(r, dict) or "bytes" not in r:
+            print("%-36s %s" % (name, r), flush=True)
+            continue
         extra = "  ".join("%s=%s" % (k, v) for k, v in r.items() if k not in ("bytes", "ms", "gbps", "frac"))
         print("%-36s %14d B  %9.4f ms  %8.1f GB/s  %5.1f %%  %s" % (name, r["bytes"], r["ms"], r["gbps"],
                                                                       100 * r["frac"], extra), flush=True)
@@ -804,19 +999,13 @@ def main():
         singles.append((time.perf_counter() - s0) * 1e6)
     singles.sort()
 
-    # the same figure as a C caller sees it (no interpreter in the launch path)
+    # the same figure as a C caller sees it (no interpreter in the launch path), beside the runtime's
+    # own floor: an empty kernel and a 4 KiB hipMemcpyAsync timed the same way
     c_lat = None
-    perf_bin = os.path.join(ROOT, "flagcx_amd", "lib", "local_perf")
-    if os.path.exists(perf_bin):
-        import subprocess
-        try:
-            r = subprocess.run([perf_bin, "-b", "4096", "-e", "4096", "-n", "40"], capture_output=True, text=True,
-                               timeout=120)
-            rw = [l.split() for l in r.stdout.splitlines() if l.strip().startswith("4096")]
-            if r.returncode == 0 and rw:
-                c_lat = {"back_to_back_per_launch": float(rw[0][2]), "single_launch_to_sync_median": float(rw[0][4])}
-        except Exception as e:  # the figure is auxiliary: report why it is missing
-            log("bench.py: C latency driver failed: %r" % (e,))
+    floor = latency_floor()
+    if floor and "library_reduce2_fp32" in floor:
+        c_lat = {"back_to_back_per_launch": floor["library_reduce2_fp32"]["back_to_back"],
+                 "single_launch_to_sync_median": floor["library_reduce2_fp32"]["launch_to_sync"]}
 
     result = {
         "metric": "hbm_gbps_reduce8_bf16_sum_256MiB", "value": round(value, 1), "unit": "GB/s",
@@ -837,6 +1026,7 @@ def main():
                      "algorithmic_bytes_per_launch": ALGO_BYTES},
         "latency_us_4KiB": {"workload": "2-input fp32 sum, 4 KiB per buffer",
                             "c_caller": c_lat,
+                            "c_caller_beside_the_runtime_floor": floor,
                             "python_ctypes_caller": {
                                 "back_to_back_per_launch": round(lat_stream_us, 3),
                                 "single_launch_to_sync_median": round(singles[len(singles) // 2], 3)}},
@@ -856,8 +1046,18 @@ def main():
             sys.exit(1)
         del host, dst
 
+    variants = None
+    if not args.no_configs:
+        variants = config_headline_variants(L, inputs)
     del bufs, pool, inputs, out
     torch.cuda.empty_cache()
+
+    # what the memory system of THIS box gives (a child process of its own, nothing else on the GPU meanwhile)
+    ceiling = measured_ceiling()
+    if ceiling:
+        result["roofline"]["ceiling"] = ceiling
+        if ceiling.get("best_read_only"):
+            result["roofline"]["frac_of_best_read_only"] = round(achieved / ceiling["best_read_only"], 4)
 
     if not args.no_configs:
         cfg = {"method": "5 warm-up + 20 timed back-to-back passes per row, HIP events on the launch stream; "
@@ -883,8 +1083,10 @@ def main():
         except Exception as e:
             cfg["C1_error"] = repr(e)
             log("bench.py: configuration C1 failed: %r" % (e,))
+        cfg.update(variants or {})
         for name, fn in (("C3", lambda: config_c3(L, full=False, separate=args.allocator_layout)),
-                         ("C4", lambda: config_c4(L, args.allocator_layout)), ("C5", lambda: config_c5(L))):
+                         ("C4", lambda: config_c4(L, args.allocator_layout)), ("C5", lambda: config_c5(L)),
+                         ("plan", lambda: config_plan_replay(L))):
             try:
                 cfg.update(fn())
             except Exception as e:

@@ -82,7 +82,8 @@ def build(verbose=False, jobs=None):
     # (host-only C++; they reach the GPU through the library)
     for prog in ("local_perf", "local_coll_test", "fifo_perf"):
         src = os.path.join(HERE, "perf", prog + ".cpp")
-        _run([HIPCC, "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", src, "-o",
+        _run([HIPCC, "-O2", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+              "-x", "hip", "--offload-arch=gfx950", src, "-o",
               os.path.join(LIBDIR, prog), "-L" + LIBDIR, "-lflagcx_amd", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", LIB, os.path.getsize(LIB), "bytes")

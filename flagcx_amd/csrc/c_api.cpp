@@ -304,6 +304,7 @@ static flagcxResult_t prepareReduce(const void *const *srcs, int k, void *dst, u
   c.op = op;
   c.stream = stream;
   c.anyOrder = 0;
+  c.plusZero = 0;
   *empty = false;
   return flagcxSuccess;
 }
@@ -451,14 +452,13 @@ static flagcxResult_t launchBatch(ReduceCall *calls, int n, int dtype, const cha
   return fromHip(reduceBatchLauncherFor(dtype)(calls, n), who);
 }
 
-flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int ndescs, int nranks,
-                                      flagcxDataType_t datatype, flagcxRedOp_t op,
-                                      flagcxStream_t stream) {
-  const char *who = "flagcxLocalReduceBatch";
+// `plusZero`: the descriptors list the members of a sum that are read; the member list also
+// holds members that are all zeros (reduce_device.h, kSumZ).
+static flagcxResult_t reduceBatchImpl(const flagcxLocalReduceDesc *descs, int ndescs, int nranks, int dt, int rop,
+                                      int plusZero, flagcxStream_t stream, const char *who) {
   if (ndescs < 0) return fail(flagcxInvalidArgument, "%s: ndescs %d is negative", who, ndescs);
   if (ndescs == 0) return flagcxSuccess;
   if (!descs) return fail(flagcxInvalidArgument, "%s: descs is NULL", who);
-  const int dt = bitsOf(datatype), rop = bitsOf(op);
   const size_t ts = typeSize(dt);
   hipStream_t hs = hipStreamOf(stream);
   constexpr int kGroup = 64;
@@ -474,6 +474,7 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
                                        calls[ncalls], &empty);
       if (r != flagcxSuccess) return r;
       if (empty) continue;
+      calls[ncalls].plusZero = plusZero;
       for (int e = 0; e < ncalls; e++)
         if ((uintptr_t)calls[e].dst < (uintptr_t)d.recvbuff + d.count * ts &&
             (uintptr_t)d.recvbuff < (uintptr_t)calls[e].dst + calls[e].count * ts)
@@ -484,6 +485,25 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
     if (r != flagcxSuccess) return r;
   }
   return finish(stream, 0, who);
+}
+
+flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int ndescs, int nranks,
+                                      flagcxDataType_t datatype, flagcxRedOp_t op,
+                                      flagcxStream_t stream) {
+  return reduceBatchImpl(descs, ndescs, nranks, bitsOf(datatype), bitsOf(op), 0, stream, "flagcxLocalReduceBatch");
+}
+
+flagcxResult_t flagcxLocalReduceBatchSparse(const flagcxLocalReduceDesc *descs, int ndescs, int nlive, int nzero,
+                                            flagcxDataType_t datatype, flagcxRedOp_t op, flagcxStream_t stream) {
+  const char *who = "flagcxLocalReduceBatchSparse";
+  if (nzero < 0) return fail(flagcxInvalidArgument, "%s: nzero %d is negative", who, nzero);
+  if (nzero > 0 && bitsOf(op) != flagcxSum)
+    return fail(flagcxInvalidArgument, "%s: members that hold zeros can only be left out of a sum, not of operation %d", who,
+                bitsOf(op));
+  if (nlive < 1 || nlive > FLAGCX_LOCAL_MAX_RANKS - nzero)
+    return fail(flagcxInvalidArgument, "%s: %d members read + %d zero members outside [1, %d]", who, nlive, nzero,
+                FLAGCX_LOCAL_MAX_RANKS);
+  return reduceBatchImpl(descs, ndescs, nlive, bitsOf(datatype), bitsOf(op), nzero > 0 ? 1 : 0, stream, who);
 }
 
 // ------------------------------------------------------------------ gated batch
@@ -663,47 +683,71 @@ flagcxResult_t flagcxLocalReduceBatchGated(flagcxLocalGate_t gate, const flagcxL
   const int dt = bitsOf(datatype), rop = bitsOf(op);
   const size_t ts = typeSize(dt);
   hipStream_t hs = hipStreamOf(stream);
-  // everything is checked before the first launch: a launch that has gone out waits for its descriptors
-  std::vector<ReduceCall> calls;
-  std::vector<uint64_t> number;
-  calls.reserve((size_t)ndescs);
-  number.reserve((size_t)ndescs);
-  for (int i = 0; i < ndescs; i++) {
-    const flagcxLocalReduceDesc &d = descs[i];
-    if (!d.sendbuffs) return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs is NULL", who, i);
-    ReduceCall c;
-    bool empty;
-    flagcxResult_t r = prepareReduce(d.sendbuffs, nranks, d.recvbuff, d.count, dt, rop, hs, who, c, &empty);
-    if (r != flagcxSuccess) return r;
-    if (empty) continue;
-    if (nranks > 8) return fail(flagcxInvalidArgument, "%s: takes up to 8 inputs, not %d", who, nranks);
-    for (int j = 0; j < nranks; j++)
-      if ((((uintptr_t)c.src[j] ^ (uintptr_t)c.dst) & 15u) != 0)
-        return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs[%d] and recvbuff differ modulo 16", who, i, j);
-    // descriptors of one launch run concurrently
-    const size_t group = calls.size() / kGateBatchMax * kGateBatchMax;
-    for (size_t e = group; e < calls.size(); e++)
-      if ((uintptr_t)calls[e].dst < (uintptr_t)d.recvbuff + d.count * ts &&
-          (uintptr_t)d.recvbuff < (uintptr_t)calls[e].dst + calls[e].count * ts)
-        return fail(flagcxInvalidArgument, "%s: recvbuff of descs[%d] overlaps an earlier one", who, i);
-    calls.push_back(c);
-    number.push_back((uint64_t)i);
-  }
-  const uint64_t base = gate->launched.fetch_add((uint64_t)ndescs);
-  if (first) *first = base;
-  (void)deviceInfo();
-  for (size_t at = 0; at < calls.size(); at += kGateBatchMax) {
-    const int m = (int)(calls.size() - at < (size_t)kGateBatchMax ? calls.size() - at : (size_t)kGateBatchMax);
-    GateArgs a;
-    a.host = gate->host + kGateHostCount;
-    a.dev = gate->dev;
-    a.hostState = gate->host + kGateHostState;
-    a.maxSpin = asyncMaxSpin();
-    a.scalarRead = gate->uncached ? 1 : 0;
-    for (int i = 0; i < kGateBatchMax; i++) a.need[i] = gate->offset + base + number[at + (size_t)(i < m ? i : 0)];
-    a.all = a.need[m - 1] + 1;
-    flagcxResult_t r = fromHip(reduceGatedLauncherFor(dt)(calls.data() + at, m, a), who);
-    if (r != flagcxSuccess) return r;
+  // Two passes over the descriptors, no storage beyond one launch's worth on the stack.  The
+  // first only checks: everything is checked before the first launch goes out, because a
+  // launch that has gone out waits for its descriptors.  The second builds the same groups of
+  // kGateBatchMax non-empty descriptors again and launches each.
+  ReduceCall group[kGateBatchMax];
+  uint64_t number[kGateBatchMax];
+  uint64_t base = 0;
+  bool launchedOne = false;
+  for (int pass = 0; pass < 2; pass++) {
+    int m = 0;
+    auto flush = [&]() -> flagcxResult_t {
+      const int n = m;
+      m = 0;
+      if (pass == 0 || n == 0) return flagcxSuccess;
+      GateArgs a;
+      a.host = gate->host + kGateHostCount;
+      a.dev = gate->dev;
+      a.hostState = gate->host + kGateHostState;
+      a.maxSpin = asyncMaxSpin();
+      a.scalarRead = gate->uncached ? 1 : 0;
+      for (int i = 0; i < kGateBatchMax; i++) a.need[i] = gate->offset + base + number[i < n ? i : 0];
+      a.all = a.need[n - 1] + 1;
+      const flagcxResult_t r = fromHip(reduceGatedLauncherFor(dt)(group, n, a), who);
+      if (r == flagcxSuccess) launchedOne = true;
+      return r;
+    };
+    flagcxResult_t err = flagcxSuccess;
+    for (int i = 0; i < ndescs && err == flagcxSuccess; i++) {
+      const flagcxLocalReduceDesc &d = descs[i];
+      if (pass == 0 && !d.sendbuffs) return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs is NULL", who, i);
+      ReduceCall &c = group[m];
+      bool empty;
+      err = prepareReduce(d.sendbuffs, nranks, d.recvbuff, d.count, dt, rop, hs, who, c, &empty);
+      if (err != flagcxSuccess || empty) continue;
+      if (pass == 0) {
+        if (nranks > 8) return fail(flagcxInvalidArgument, "%s: takes up to 8 inputs, not %d", who, nranks);
+        for (int j = 0; j < nranks; j++)
+          if ((((uintptr_t)c.src[j] ^ (uintptr_t)c.dst) & 15u) != 0)
+            return fail(flagcxInvalidArgument, "%s: descs[%d].sendbuffs[%d] and recvbuff differ modulo 16", who, i, j);
+        // descriptors of one launch run concurrently
+        for (int e = 0; e < m; e++)
+          if ((uintptr_t)group[e].dst < (uintptr_t)d.recvbuff + d.count * ts &&
+              (uintptr_t)d.recvbuff < (uintptr_t)group[e].dst + group[e].count * ts)
+            return fail(flagcxInvalidArgument, "%s: recvbuff of descs[%d] overlaps an earlier one", who, i);
+      }
+      number[m++] = (uint64_t)i;
+      if (m == kGateBatchMax) err = flush();
+    }
+    if (err == flagcxSuccess) err = flush();
+    if (pass == 0) {
+      if (err != flagcxSuccess) return err;
+      // the numbers are handed out only once every descriptor has passed its checks
+      base = gate->launched.fetch_add((uint64_t)ndescs);
+      if (first) *first = base;
+      (void)deviceInfo();
+    } else if (err != flagcxSuccess) {
+      // A launch failed after others had gone out: those wait for numbers the caller will
+      // never open.  The gate is abandoned (as flagcxLocalGateDestroy does): its waiting
+      // workgroups leave without touching data, and later calls on it report that.
+      if (launchedOne) {
+        __atomic_store_n(gate->host + kGateHostState, (uint64_t)kGateTimedOut, __ATOMIC_RELEASE);
+        __atomic_store_n(gate->host + kGateHostCount, ~0ull, __ATOMIC_RELEASE);
+      }
+      return err;
+    }
   }
   return flagcxSuccess;
 }

@@ -299,7 +299,7 @@ int launchCopy2D(const Copy2D &c) {
     if (!vector) {
       // the two sides sit at different offsets modulo 16: a one-input byte "reduce",
       // which reads the source with aligned loads and puts it in place with lane shifts
-      ReduceCall r;
+      ReduceCall r{};
       r.src[0] = src0;
       r.dst = dst0;
       r.count = c.chunkBytes;

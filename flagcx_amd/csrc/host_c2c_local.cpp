@@ -26,15 +26,26 @@
 // homoTypes; for homoType 1 the planner's inter-rank buffer list, which the plan
 // document does not carry, is rebuilt from the rank's hetero receives (the list's
 // isRecv_ entries are exactly those, c2c_algo.cc:386-400,434-452).
-// Not replayed (flagcxNotSupported): AlltoAllv, whose counts and displacements are
-// call arguments, not part of a plan.
+// AlltoAllv takes its counts and displacements, which are arguments of execute() and not
+// part of a plan (c2c_algo.cc:2042-2046), from flagcxLocalPlanSetAlltoAllv.
+//
+// Two ways to replay, with the same bytes in every receive buffer at the end:
+//   - literal: every refresh is a zero-fill and every reduce-type homo function reads all
+//     of its members' buffers, zeros included, as the reference does;
+//   - fused (the default): a refresh only records the ranges it would clear, and a sum
+//     reads the members whose slices hold data (ZeroSet below).  The assembly idiom
+//     "clear everything but the own slice, then all-reduce the buffers"
+//     (c2c_algo.cc:586-608 + 310-336) then moves the live slices only.
 #include "../../include/flagcx_amd.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <iterator>
 #include <map>
 #include <string>
+#include <utility>
 #include <vector>
 
 namespace {
@@ -215,6 +226,8 @@ struct flagcxLocalPlan {
   // AlltoAllv: row r of each matrix is the array rank r hands to execute() (c2c_algo.cc:2042-2046,2083-2094)
   std::vector<size_t> sendCounts, sDispls, recvCounts, rDispls;
   bool loaded = false;
+  bool fused = true; // flagcxLocalPlanSetFused
+  uint64_t lastBytes = 0, lastLaunches = 0; // flagcxLocalPlanGetTraffic
   char err[256] = "";
 };
 
@@ -226,54 +239,268 @@ static flagcxResult_t planFail(flagcxLocalPlan *p, flagcxResult_t code, const ch
   return code;
 }
 
-struct Bufs {
-  const void *const *send;
-  void *const *recv;
-  void *const *scratch;
-};
-
-static char *pick(const Bufs &b, int rank, int type) {
-  // sendType_: 0 user send, 1 recv, 2 scratch; recvType_: 1 recv, else scratch (c2c_algo.cc:297-300)
-  if (type == 0) return (char *)const_cast<void *>(b.send[rank]);
-  if (type == 1) return (char *)b.recv[rank];
-  return b.scratch ? (char *)b.scratch[rank] : nullptr;
-}
-
 #define LCHECK(call)                                                           \
   do {                                                                         \
     flagcxResult_t r_ = (call);                                                \
     if (r_ != flagcxSuccess) return r_;                                        \
   } while (0)
 
-// n blocks of `bytes` from the pointers in `src` into dst, back to back: one launch
-// unless a block already lies inside the destination (in-place all-gather,
-// flagcx/include/flagcx.h:373), which the list copy refuses; then block by block,
-// where a copy onto itself is nothing.
-static flagcxResult_t gatherBlocks(char *dst, const std::vector<const void *> &src, size_t bytes, flagcxStream_t stream) {
-  const int n = (int)src.size();
-  bool inside = n > 64;
-  for (int j = 0; j < n && !inside; j++) {
-    const char *s = (const char *)src[j];
-    inside = s < dst + (size_t)n * bytes && dst < s + bytes;
+// Byte ranges of device memory that hold zeros by definition but have not been written.
+// The reference assembles a sum across a cluster by clearing, in every member's buffer,
+// all but the member's own slice (flagcxC2cRefreshFunc::run, c2c_algo.cc:586-608) and
+// then all-reducing the whole buffers (c2c_algo.cc:310-336): most of what that collective
+// reads are the zeros just written.  The fused replay keeps those ranges here instead:
+// a refresh adds ranges, a write removes them, a copy out of them moves them, a sum leaves
+// out the members that lie in them, and what is left when the plan ends is written then.
+class ZeroSet {
+  std::map<uintptr_t, uintptr_t> r_; // begin -> end: disjoint, never adjacent
+ public:
+  bool empty() const { return r_.empty(); }
+  void add(uintptr_t b, uintptr_t e) {
+    if (b >= e) return;
+    auto it = r_.upper_bound(b);
+    if (it != r_.begin()) {
+      auto pv = std::prev(it);
+      if (pv->second >= b) {
+        b = pv->first;
+        if (pv->second > e) e = pv->second;
+        it = r_.erase(pv);
+      }
+    }
+    while (it != r_.end() && it->first <= e) {
+      if (it->second > e) e = it->second;
+      it = r_.erase(it);
+    }
+    r_[b] = e;
   }
-  if (!inside) return flagcxLocalPackList(dst, src.data(), n, bytes, stream);
-  for (int j = 0; j < n; j++) {
-    const flagcxResult_t r = flagcxLocalMemcpy(dst + (size_t)j * bytes, src[j], bytes, stream);
-    if (r != flagcxSuccess) return r;
+  void remove(uintptr_t b, uintptr_t e) {
+    if (b >= e) return;
+    auto it = r_.upper_bound(b);
+    if (it != r_.begin()) --it;
+    while (it != r_.end() && it->first < e) {
+      const uintptr_t rb = it->first, re = it->second;
+      if (re <= b) {
+        ++it;
+        continue;
+      }
+      it = r_.erase(it);
+      if (rb < b) r_[rb] = b;
+      if (re > e) r_[e] = re;
+    }
   }
-  return flagcxSuccess;
-}
+  bool touches(uintptr_t b, uintptr_t e) const {
+    if (b >= e) return false;
+    auto it = r_.upper_bound(b);
+    if (it != r_.begin() && std::prev(it)->second > b) return true;
+    return it != r_.end() && it->first < e;
+  }
+  bool covers(uintptr_t b, uintptr_t e) const {
+    auto it = r_.upper_bound(b);
+    if (it == r_.begin()) return false;
+    --it;
+    return it->second >= e;
+  }
+  // where zero ranges begin or end strictly inside (b, e), as offsets from b, ascending
+  void cuts(uintptr_t b, uintptr_t e, std::vector<size_t> &out) const {
+    auto it = r_.upper_bound(b);
+    if (it != r_.begin()) --it;
+    for (; it != r_.end() && it->first < e; ++it) {
+      if (it->first > b) out.push_back(it->first - b);
+      if (it->second > b && it->second < e) out.push_back(it->second - b);
+    }
+  }
+  std::vector<std::pair<uintptr_t, uintptr_t>> ranges() const {
+    return std::vector<std::pair<uintptr_t, uintptr_t>>(r_.begin(), r_.end());
+  }
+};
 
-static flagcxResult_t runSendRecv(flagcxLocalPlan *p, int cl, const std::vector<const HomoFunc *> &fn, const Bufs &b,
-                                  size_t ts, int root, flagcxStream_t stream);
+// One reduction of a collective: dst = fold of src[0..n) over `count` elements.
+struct Red {
+  char *dst;
+  std::vector<const char *> src;
+  size_t count;
+};
 
-// One homo function slot (step s, index i of one table) across all ranks.  `root`
-// is the collective's root as a rank of its cluster, globalrank2homorank[root]
-// (c2c_algo.cc:2147,2170).
-static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const HomoFunc *> &fn, const Bufs &b,
-                                  flagcxDataType_t dt, int root, flagcxStream_t stream) {
-  const size_t ts = flagcxLocalGetDataTypeSize(dt);
+// One flagcxLocalPlanExecute call.
+struct Exec {
+  flagcxLocalPlan *p;
+  const void *const *send;
+  void *const *recv;
+  void *const *scratch;
+  flagcxDataType_t dt;
+  size_t ts;
+  int homoRoot;
+  flagcxStream_t stream;
+  bool fused;
+  ZeroSet zeros;
+  std::vector<char> ownsScratch; // per rank: the reference allocates a scratch buffer for this call (c2c_algo.cc:2122-2129)
+  std::vector<char *> recvTmp, sendTmp;
+  uint64_t bytes = 0, launches = 0; // algorithmic traffic handed to the kernels
+
+  char *pick(int rank, int type) const {
+    // sendType_: 0 user send, 1 recv, 2 scratch; recvType_: 1 recv, else scratch (c2c_algo.cc:297-300)
+    if (type == 0) return (char *)const_cast<void *>(send[rank]);
+    if (type == 1) return (char *)recv[rank];
+    return scratch ? (char *)scratch[rank] : nullptr;
+  }
+  flagcxResult_t needScratch() { return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", ""); }
+
+  flagcxResult_t memcpyNow(char *dst, const char *src, size_t n) {
+    bytes += 2 * n;
+    launches++;
+    return flagcxLocalMemcpy(dst, src, n, stream);
+  }
+  flagcxResult_t memsetNow(char *dst, size_t n) {
+    bytes += n;
+    launches++;
+    return flagcxLocalMemset(dst, 0, n, stream);
+  }
+
+  // dst[0, n) = src[0, n), zeros that were never written included.
+  flagcxResult_t copy(char *dst, const char *src, size_t n) {
+    if (!n || dst == src) return flagcxSuccess;
+    const uintptr_t s = (uintptr_t)src, d = (uintptr_t)dst;
+    if (!fused || zeros.empty()) return memcpyNow(dst, src, n);
+    if (!zeros.touches(s, s + n)) {
+      zeros.remove(d, d + n);
+      return memcpyNow(dst, src, n);
+    }
+    if (d < s + n && s < d + n) return planFail(p, flagcxInvalidArgument, "a copy's buffers overlap%s", "");
+    std::vector<size_t> cut{0};
+    zeros.cuts(s, s + n, cut);
+    cut.push_back(n);
+    std::vector<char> isZero(cut.size() - 1);
+    for (size_t i = 0; i + 1 < cut.size(); i++) isZero[i] = zeros.covers(s + cut[i], s + cut[i + 1]);
+    for (size_t i = 0; i + 1 < cut.size(); i++) {
+      const size_t at = cut[i], len = cut[i + 1] - cut[i];
+      if (isZero[i]) {
+        zeros.add(d + at, d + at + len);
+      } else {
+        zeros.remove(d + at, d + at + len);
+        LCHECK(memcpyNow(dst + at, src + at, len));
+      }
+    }
+    return flagcxSuccess;
+  }
+
+  // n blocks of `n` bytes from the pointers in `src` into dst, back to back: one launch
+  // unless a block already lies inside the destination (in-place all-gather,
+  // flagcx/include/flagcx.h:373), which the list copy refuses; then block by block,
+  // where a copy onto itself is nothing.
+  flagcxResult_t gather(char *dst, const std::vector<const void *> &src, size_t n) {
+    const int m = (int)src.size();
+    if (!n || !m) return flagcxSuccess;
+    bool single = m <= 64;
+    for (int j = 0; j < m && single; j++) {
+      const char *s = (const char *)src[j];
+      single = !(s < dst + (size_t)m * n && dst < s + n);
+      if (fused && zeros.touches((uintptr_t)s, (uintptr_t)s + n)) single = false;
+    }
+    if (!single) {
+      for (int j = 0; j < m; j++) LCHECK(copy(dst + (size_t)j * n, (const char *)src[j], n));
+      return flagcxSuccess;
+    }
+    if (fused) zeros.remove((uintptr_t)dst, (uintptr_t)dst + (size_t)m * n);
+    bytes += 2 * (uint64_t)m * n;
+    launches++;
+    return flagcxLocalPackList(dst, src.data(), m, n, stream);
+  }
+
+  // Zeros that are due in [b, e) are written now.
+  flagcxResult_t materialize(uintptr_t b, uintptr_t e) {
+    if (!fused || !zeros.touches(b, e)) return flagcxSuccess;
+    std::vector<size_t> cut{0};
+    zeros.cuts(b, e, cut);
+    cut.push_back(e - b);
+    for (size_t i = 0; i + 1 < cut.size(); i++)
+      if (zeros.covers(b + cut[i], b + cut[i + 1])) LCHECK(memsetNow((char *)b + cut[i], cut[i + 1] - cut[i]));
+    zeros.remove(b, e);
+    return flagcxSuccess;
+  }
+
+  flagcxResult_t reduceNow(const std::vector<Red> &reds, int nzero) {
+    const int nlive = (int)reds[0].src.size();
+    const flagcxRedOp_t rop = (flagcxRedOp_t)p->redOp;
+    std::vector<flagcxLocalReduceDesc> descs(reds.size());
+    for (size_t i = 0; i < reds.size(); i++) {
+      descs[i] = {(const void *const *)reds[i].src.data(), reds[i].dst, reds[i].count};
+      bytes += (uint64_t)(nlive + 1) * reds[i].count * ts;
+    }
+    launches += (reds.size() + 31) / 32;
+    if (nzero) return flagcxLocalReduceBatchSparse(descs.data(), (int)descs.size(), nlive, nzero, dt, rop, stream);
+    if (reds.size() == 1) return flagcxLocalReduce(descs[0].sendbuffs, nlive, descs[0].recvbuff, descs[0].count, dt, rop, stream);
+    return flagcxLocalReduceBatch(descs.data(), (int)descs.size(), nlive, dt, rop, stream);
+  }
+
+  // The reductions of one collective (same member count; they run concurrently).  Members
+  // whose slice lies in zeros that were never written are not read: a sum over the rest,
+  // with +0.0 added once, has the bytes of the sum over all of them (the zero members turn
+  // a -0.0 result into +0.0 and change nothing else).
+  flagcxResult_t reduce(const std::vector<Red> &reds) {
+    if (reds.empty()) return flagcxSuccess;
+    bool plain = !fused || zeros.empty();
+    if (!plain) {
+      plain = true;
+      for (auto &r : reds)
+        for (auto s : r.src)
+          if (zeros.touches((uintptr_t)s, (uintptr_t)s + r.count * ts)) plain = false;
+    }
+    if (!plain && p->redOp != flagcxSum) {
+      // for a maximum or a minimum a zero is a value like any other
+      for (auto &r : reds)
+        for (auto s : r.src) LCHECK(materialize((uintptr_t)s, (uintptr_t)s + r.count * ts));
+      plain = true;
+    }
+    if (plain) {
+      if (fused)
+        for (auto &r : reds) zeros.remove((uintptr_t)r.dst, (uintptr_t)r.dst + r.count * ts);
+      return reduceNow(reds, 0);
+    }
+    const int n = (int)reds[0].src.size();
+    std::map<int, std::vector<Red>> byLive; // members read -> pieces (n: no member left out)
+    std::vector<std::pair<uintptr_t, uintptr_t>> written, cleared;
+    for (auto &r : reds) {
+      const size_t len = r.count * ts;
+      std::vector<size_t> cut{0, len};
+      for (auto s : r.src) zeros.cuts((uintptr_t)s, (uintptr_t)s + len, cut);
+      std::sort(cut.begin(), cut.end());
+      cut.erase(std::unique(cut.begin(), cut.end()), cut.end());
+      for (size_t i = 0; i + 1 < cut.size(); i++) {
+        const size_t a = cut[i], b = cut[i + 1];
+        if (a % ts || b % ts) return planFail(p, flagcxInternalError, "a cleared range ends inside an element%s", "");
+        Red piece{r.dst + a, {}, (b - a) / ts};
+        for (auto s : r.src)
+          if (!zeros.covers((uintptr_t)s + a, (uintptr_t)s + b)) piece.src.push_back(s + a);
+        if (piece.src.empty()) {
+          cleared.push_back({(uintptr_t)r.dst + a, (uintptr_t)r.dst + b}); // 0 + 0 + ... = +0
+        } else {
+          written.push_back({(uintptr_t)r.dst + a, (uintptr_t)r.dst + b});
+          byLive[(int)piece.src.size()].push_back(std::move(piece));
+        }
+      }
+    }
+    for (auto &w : written) zeros.remove(w.first, w.second);
+    for (auto &c : cleared) zeros.add(c.first, c.second);
+    for (auto &g : byLive) LCHECK(reduceNow(g.second, n - g.first));
+    return flagcxSuccess;
+  }
+
+  flagcxResult_t refresh(const std::vector<char> *only);
+  flagcxResult_t homoSlot(const std::vector<const HomoFunc *> &fn);
+  flagcxResult_t sendRecv(int cl, const std::vector<const HomoFunc *> &fn);
+  flagcxResult_t homoStep(std::vector<std::vector<HomoFunc>> RankPlan::*table, int s, int onlyIndex = -1,
+                          const std::vector<char> *only = nullptr, bool refreshBeforeEach = false);
+  flagcxResult_t heteroSlot(int s, int i);
+  flagcxResult_t run();
+  flagcxResult_t finish();
+};
+
+// One homo function slot (step s, index i of one table) across all ranks; fn[r] is rank
+// r's function or NULL.  The collective's root reaches the functions as a rank of its
+// cluster, globalrank2homorank[root] (c2c_algo.cc:2147,2170).
+flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
   const int ncl = (int)p->clusterRanks.size();
+  const int root = homoRoot;
   for (int cl = 0; cl < ncl; cl++) {
     // members that hold a function in this slot; homoType 1 runs on inter-ranks only
     std::vector<int> mem;
@@ -291,21 +518,20 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
     if (op == kLocCpy || op == kLocRed) {
       for (int r : mem) {
         const HomoFunc *f = fn[r];
-        char *s = pick(b, r, f->sendType_), *d = pick(b, r, f->recvType_ == 1 ? 1 : 2);
-        if (!s || !d) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+        char *s = pick(r, f->sendType_), *d = pick(r, f->recvType_ == 1 ? 1 : 2);
+        if (!s || !d) return needScratch();
         s += f->sendOffset_ * ts;
         d += f->recvOffset_ * ts;
         if (op == kLocCpy) {
-          LCHECK(flagcxLocalMemcpy(d, s, f->count_ * ts, stream));
+          LCHECK(copy(d, s, f->count_ * ts));
         } else {
-          const void *srcs[2] = {d, s}; // acc = recv slice; acc = OP(send slice, acc)
-          LCHECK(flagcxLocalReduce(srcs, 2, d, f->count_, dt, (flagcxRedOp_t)p->redOp, stream));
+          LCHECK(reduce({Red{d, {d, s}, f->count_}})); // acc = recv slice; acc = OP(send slice, acc)
         }
       }
       continue;
     }
     if (op == flagcxCommOpSend || op == flagcxCommOpRecv) {
-      LCHECK(runSendRecv(p, cl, fn, b, ts, root, stream));
+      LCHECK(sendRecv(cl, fn));
       continue;
     }
     if (op == flagcxCommOpAlltoAllv) {
@@ -316,8 +542,8 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
         return planFail(p, flagcxInvalidArgument, "AlltoAllv needs counts and displacements (flagcxLocalPlanSetAlltoAllv)%s", "");
       for (int r : mem) {
         const HomoFunc *f = fn[r];
-        char *src = pick(b, r, f->sendType_);
-        if (!src) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+        char *src = pick(r, f->sendType_);
+        if (!src) return needScratch();
         for (int i : p->clusterRanks[cl]) {
           const size_t cnt = p->sendCounts[r * n + i];
           const HomoFunc *g = fn[i];
@@ -325,9 +551,9 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
           if (cnt != (recvs ? p->recvCounts[i * n + r] : 0))
             return planFail(p, flagcxInvalidUsage, "AlltoAllv: rank %s%lld sends to rank %lld what that rank does not receive", "", r, i);
           if (!cnt) continue;
-          char *dst = pick(b, i, g->recvType_ == 1 ? 1 : 2);
-          if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
-          LCHECK(flagcxLocalMemcpy(dst + p->rDispls[i * n + r] * ts, src + p->sDispls[r * n + i] * ts, cnt * ts, stream));
+          char *dst = pick(i, g->recvType_ == 1 ? 1 : 2);
+          if (!dst) return needScratch();
+          LCHECK(copy(dst + p->rDispls[i * n + r] * ts, src + p->sDispls[r * n + i] * ts, cnt * ts));
         }
       }
       // a receive nobody sends would hang the reference
@@ -349,67 +575,68 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
       const HomoFunc *f = fn[r];
       if (!f || f->commOp_ != op)
         return planFail(p, flagcxInvalidUsage, "rank %s%lld has no matching homo function (commOp %lld)", "", r, op);
-      char *s = pick(b, r, f->sendType_), *d = pick(b, r, f->recvType_ == 1 ? 1 : 2);
-      if (!s || !d) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+      char *s = pick(r, f->sendType_), *d = pick(r, f->recvType_ == 1 ? 1 : 2);
+      if (!s || !d) return needScratch();
       S[h] = s + f->sendOffset_ * ts;
       D[h] = d + f->recvOffset_ * ts;
       cnt[h] = f->count_;
     }
     const size_t count = cnt[0];
-    auto homoRoot = [&](const HomoFunc *f) { return f->rootRank_ == -1 ? root : f->rootRank_; };
-    const flagcxRedOp_t rop = (flagcxRedOp_t)p->redOp;
+    auto homoRootOf = [&](const HomoFunc *f) { return f->rootRank_ == -1 ? root : f->rootRank_; };
+    auto badRoot = [&](int rt) { return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt); };
+    const std::vector<const char *> members(S.begin(), S.end());
     switch (op) {
       case flagcxCommOpReduce: {
-        const int rt = homoRoot(first);
-        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
-        LCHECK(flagcxLocalReduce((const void *const *)S.data(), n, D[rt], count, dt, rop, stream));
+        const int rt = homoRootOf(first);
+        if (rt < 0 || rt >= n) return badRoot(rt);
+        LCHECK(reduce({Red{D[rt], members, count}}));
         break;
       }
       case flagcxCommOpAllReduce: {
         // every member ends with the same bytes: reduce once, then copy
-        LCHECK(flagcxLocalReduce((const void *const *)S.data(), n, D[0], count, dt, rop, stream));
-        for (int h = 1; h < n; h++) LCHECK(flagcxLocalMemcpy(D[h], D[0], count * ts, stream));
+        LCHECK(reduce({Red{D[0], members, count}}));
+        for (int h = 1; h < n; h++) LCHECK(copy(D[h], D[0], count * ts));
         break;
       }
       case flagcxCommOpReduceScatter: {
         // member h receives the fold of everybody's h-th block; one batch launch
-        std::vector<std::vector<const void *>> srcs(n, std::vector<const void *>(n));
-        std::vector<flagcxLocalReduceDesc> descs(n);
+        std::vector<Red> reds(n);
         for (int h = 0; h < n; h++) {
-          for (int j = 0; j < n; j++) srcs[h][j] = S[j] + (size_t)h * count * ts;
-          descs[h] = {srcs[h].data(), D[h], count};
+          reds[h].dst = D[h];
+          reds[h].count = count;
+          for (int j = 0; j < n; j++) reds[h].src.push_back(S[j] + (size_t)h * count * ts);
         }
-        LCHECK(flagcxLocalReduceBatch(descs.data(), n, n, dt, rop, stream));
+        LCHECK(reduce(reds));
         break;
       }
       case flagcxCommOpAllGather: {
         const std::vector<const void *> blocks(S.begin(), S.end());
-        for (int h = 0; h < n; h++) LCHECK(gatherBlocks(D[h], blocks, count * ts, stream));
+        for (int h = 0; h < n; h++) LCHECK(gather(D[h], blocks, count * ts));
         break;
       }
       case flagcxCommOpGather: {
-        const int rt = homoRoot(first);
-        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
-        LCHECK(gatherBlocks(D[rt], std::vector<const void *>(S.begin(), S.end()), count * ts, stream));
+        const int rt = homoRootOf(first);
+        if (rt < 0 || rt >= n) return badRoot(rt);
+        LCHECK(gather(D[rt], std::vector<const void *>(S.begin(), S.end()), count * ts));
         break;
       }
       case flagcxCommOpScatter: {
-        const int rt = homoRoot(first);
-        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
-        for (int h = 0; h < n; h++) LCHECK(flagcxLocalMemcpy(D[h], S[rt] + (size_t)h * count * ts, count * ts, stream));
+        const int rt = homoRootOf(first);
+        if (rt < 0 || rt >= n) return badRoot(rt);
+        for (int h = 0; h < n; h++) LCHECK(copy(D[h], S[rt] + (size_t)h * count * ts, count * ts));
         break;
       }
       case flagcxCommOpBroadcast: {
-        const int rt = homoRoot(first);
-        if (rt < 0 || rt >= n) return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
-        for (int h = 0; h < n; h++) LCHECK(flagcxLocalMemcpy(D[h], S[rt], count * ts, stream));
+        const int rt = homoRootOf(first);
+        if (rt < 0 || rt >= n) return badRoot(rt);
+        for (int h = 0; h < n; h++) LCHECK(copy(D[h], S[rt], count * ts));
         break;
       }
       case flagcxCommOpAlltoAll: {
         std::vector<const void *> blocks(n);
         for (int h = 0; h < n; h++) {
           for (int j = 0; j < n; j++) blocks[j] = S[j] + (size_t)h * count * ts;
-          LCHECK(gatherBlocks(D[h], blocks, count * ts, stream));
+          LCHECK(gather(D[h], blocks, count * ts));
         }
         break;
       }
@@ -422,36 +649,37 @@ static flagcxResult_t runHomoSlot(flagcxLocalPlan *p, const std::vector<const Ho
   return flagcxSuccess;
 }
 
-static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream,
-                                 const std::vector<char> *only = nullptr);
-
-static flagcxResult_t runHomoStep(flagcxLocalPlan *p, std::vector<std::vector<HomoFunc>> RankPlan::*table, int s,
-                                  const Bufs &b, flagcxDataType_t dt, int root, flagcxStream_t stream,
-                                  int onlyIndex = -1, bool refreshBeforeEach = false) {
+// Functions i (all of them, or `onlyIndex`) of step s of one table.  `only`: the ranks that
+// take part (a rank leaves a loop of the reference when ITS table runs out); with
+// refreshBeforeEach every rank that runs function i refreshes first (c2c_algo.cc:2276-2282).
+flagcxResult_t Exec::homoStep(std::vector<std::vector<HomoFunc>> RankPlan::*table, int s, int onlyIndex,
+                              const std::vector<char> *only, bool refreshBeforeEach) {
   size_t width = 0;
   for (auto &rp : p->ranks) {
     auto &t = rp.*table;
     if (s < (int)t.size() && t[s].size() > width) width = t[s].size();
   }
+  std::vector<char> has(p->nranks);
   for (size_t i = 0; i < width; i++) {
     if (onlyIndex >= 0 && (int)i != onlyIndex) continue;
-    if (refreshBeforeEach) LCHECK(runRefresh(p, b, dt, stream));
     std::vector<const HomoFunc *> fn(p->nranks, nullptr);
+    bool any = false;
     for (int r = 0; r < p->nranks; r++) {
       auto &t = p->ranks[r].*table;
-      if (s < (int)t.size() && i < t[s].size()) fn[r] = &t[s][i];
+      has[r] = (!only || (*only)[r]) && s < (int)t.size() && i < t[s].size();
+      if (has[r]) fn[r] = &t[s][i];
+      any = any || has[r];
     }
-    LCHECK(runHomoSlot(p, fn, b, dt, root, stream));
+    if (!any) continue;
+    if (refreshBeforeEach) LCHECK(refresh(&has));
+    LCHECK(homoSlot(fn));
   }
   return flagcxSuccess;
 }
 
 // Hetero function i of step s on every rank: match each send with the peer's
 // next unmatched receive from that sender (order of appearance).
-static flagcxResult_t runHeteroSlot(flagcxLocalPlan *p, int s, int i, const std::vector<char *> &sendTmp,
-                                    const std::vector<char *> &recvTmp, flagcxDataType_t dt,
-                                    flagcxStream_t stream) {
-  const size_t ts = flagcxLocalGetDataTypeSize(dt);
+flagcxResult_t Exec::heteroSlot(int s, int i) {
   std::map<std::pair<int, int>, std::vector<const P2pOp *>> recvs; // (receiver, sender) -> ops
   for (int r = 0; r < p->nranks; r++) {
     auto &t = p->ranks[r].heteroFuncSteps_;
@@ -475,7 +703,10 @@ static flagcxResult_t runHeteroSlot(flagcxLocalPlan *p, int s, int i, const std:
       const P2pOp *rv = it->second[u++];
       if (rv->count_ != op.count_)
         return planFail(p, flagcxInvalidUsage, "send/recv count mismatch between ranks %s%lld and %lld", "", r, peer);
-      LCHECK(flagcxLocalMemcpy(recvTmp[peer] + rv->offset_ * ts, sendTmp[r] + op.offset_ * ts, op.count_ * ts, stream));
+      if (!recvTmp[peer] || !sendTmp[r])
+        return planFail(p, flagcxInvalidArgument, "rank %s%lld stages its hetero functions in scratch and was given none", "",
+                        recvTmp[peer] ? r : peer);
+      LCHECK(copy(recvTmp[peer] + rv->offset_ * ts, sendTmp[r] + op.offset_ * ts, op.count_ * ts));
     }
   }
   for (auto &kv : recvs)
@@ -484,35 +715,41 @@ static flagcxResult_t runHeteroSlot(flagcxLocalPlan *p, int s, int i, const std:
   return flagcxSuccess;
 }
 
-static size_t heteroWidth(flagcxLocalPlan *p, int s) {
-  size_t w = 0;
-  for (auto &rp : p->ranks)
-    if (s < (int)rp.heteroFuncSteps_.size() && rp.heteroFuncSteps_[s].size() > w) w = rp.heteroFuncSteps_[s].size();
-  return w;
-}
-
 // The refresh function of every rank (only: of the ranks marked).
-static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataType_t dt, flagcxStream_t stream,
-                                 const std::vector<char> *only) {
+flagcxResult_t Exec::refresh(const std::vector<char> *only) {
   for (int r = 0; r < p->nranks; r++) {
     if (only && !(*only)[r]) continue;
     const RefreshFunc &f = p->ranks[r].refreshFunc_;
-    // bufftype -1 resolves to recv (1) without scratch, scratch (2) with it, and under the
-    // pipeline algorithm a reduce-type collective starts at its cluster's part (c2c_algo.cc:2156-2164)
+    // bufftype -1 resolves to scratch (2) on a rank the reference gives a scratch buffer and to
+    // recv (1) on every other, and under the pipeline algorithm a reduce-type collective starts
+    // at its cluster's part (c2c_algo.cc:2156-2164)
     int bt = f.bufftype_;
     size_t start = f.start_;
     if (bt == -1) {
-      bt = (b.scratch && b.scratch[r]) ? 2 : 1;
+      bt = ownsScratch[r] ? 2 : 1;
       if ((p->commOp == flagcxCommOpReduceScatter || p->commOp == flagcxCommOpAllReduce) && p->algorithm == 1) {
         size_t clusterOffset = 0;
         for (int c = 0; c < p->clusterOf[r]; c++) clusterOffset += p->clusterRanks[c].size();
         start = clusterOffset * p->totalCount / (size_t)p->nranks;
       }
     }
-    void *buff = bt == 1 ? b.recv[r] : (b.scratch ? b.scratch[r] : nullptr);
+    void *buff = bt == 1 ? recv[r] : (scratch ? scratch[r] : nullptr);
     if (f.totalCount_ == 0) continue;
     if (!buff) return planFail(p, flagcxInvalidArgument, "refresh needs a scratch buffer%s", "");
-    LCHECK(flagcxLocalRefresh(buff, start, f.offset_, f.count_, f.totalCount_, dt, (flagcxRedOp_t)f.redOp_, stream));
+    if (!fused) {
+      if (f.redOp_ == flagcxSum && f.count_ < f.totalCount_) {
+        bytes += (f.totalCount_ - f.count_) * ts;
+        launches++;
+      }
+      LCHECK(flagcxLocalRefresh(buff, start, f.offset_, f.count_, f.totalCount_, dt, (flagcxRedOp_t)f.redOp_, stream));
+      continue;
+    }
+    if (f.offset_ + f.count_ > f.totalCount_ || f.offset_ + f.count_ < f.offset_)
+      return planFail(p, flagcxInvalidArgument, "refresh: offset + count exceeds totalCount%s", "");
+    if (f.redOp_ != flagcxSum) continue; // c2c_algo.cc:596
+    const uintptr_t base = (uintptr_t)buff + start * ts;
+    zeros.add(base, base + f.offset_ * ts);
+    zeros.add(base + (f.offset_ + f.count_) * ts, base + f.totalCount_ * ts);
   }
   return flagcxSuccess;
 }
@@ -525,9 +762,9 @@ static flagcxResult_t runRefresh(flagcxLocalPlan *p, const Bufs &b, flagcxDataTy
 //               clusters, piece by piece at the pieces' own offsets;
 //   homoType 2: inter-rank 0 sends to the root unless it is the root itself.
 // Roots are ranks inside the cluster.
-static flagcxResult_t runSendRecv(flagcxLocalPlan *p, int cl, const std::vector<const HomoFunc *> &fn, const Bufs &b,
-                                  size_t ts, int root, flagcxStream_t stream) {
+flagcxResult_t Exec::sendRecv(int cl, const std::vector<const HomoFunc *> &fn) {
   const std::vector<int> &members = p->clusterRanks[cl], &inters = p->clusterInterRanks[cl];
+  const int root = homoRoot;
   auto recvOf = [&](int r) -> const HomoFunc * {
     const HomoFunc *g = fn[r];
     return (g && g->commOp_ == flagcxCommOpRecv) ? g : nullptr;
@@ -538,23 +775,23 @@ static flagcxResult_t runSendRecv(flagcxLocalPlan *p, int cl, const std::vector<
     const int rt = f->rootRank_ == -1 ? root : f->rootRank_;
     if (rt < 0 || rt >= (int)members.size())
       return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt);
-    char *src = pick(b, r, f->sendType_);
-    if (!src) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+    char *src = pick(r, f->sendType_);
+    if (!src) return needScratch();
     if (f->homoType_ == 0) {
       if (p->homoRank[r] != rt) continue;
       for (int peer : inters) {
         const HomoFunc *g = recvOf(peer);
         if (peer == r || !g || p->homoRank[peer] == rt) continue;
-        char *dst = pick(b, peer, g->recvType_ == 1 ? 1 : 2);
-        if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
-        LCHECK(flagcxLocalMemcpy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts, stream));
+        char *dst = pick(peer, g->recvType_ == 1 ? 1 : 2);
+        if (!dst) return needScratch();
+        LCHECK(copy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts));
       }
     } else if (f->homoType_ == 1) {
       if (p->homoInterRank[r] <= 0 || inters.empty()) continue;
       const HomoFunc *g = recvOf(inters[0]);
       if (!g) continue;
-      char *dst = pick(b, inters[0], g->recvType_ == 1 ? 1 : 2);
-      if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
+      char *dst = pick(inters[0], g->recvType_ == 1 ? 1 : 2);
+      if (!dst) return needScratch();
       // what rank r received from other clusters: every receive of its hetero functions
       std::vector<std::pair<size_t, size_t>> pieces;
       for (auto &step : p->ranks[r].heteroFuncSteps_)
@@ -565,18 +802,110 @@ static flagcxResult_t runSendRecv(flagcxLocalPlan *p, int cl, const std::vector<
             for (auto &q : pieces) seen = seen || (q.first == o.offset_ && q.second == o.count_);
             if (!seen) pieces.push_back({o.offset_, o.count_});
           }
-      for (auto &q : pieces)
-        LCHECK(flagcxLocalMemcpy(dst + q.first * ts, src + q.first * ts, q.second * ts, stream));
+      for (auto &q : pieces) LCHECK(copy(dst + q.first * ts, src + q.first * ts, q.second * ts));
     } else if (f->homoType_ == 2) {
       if (p->homoInterRank[r] != 0 || p->homoRank[r] == rt) continue;
       const int peer = members[rt];
       const HomoFunc *g = recvOf(peer);
       if (!g) continue;
-      char *dst = pick(b, peer, g->recvType_ == 1 ? 1 : 2);
-      if (!dst) return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", "");
-      LCHECK(flagcxLocalMemcpy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts, stream));
+      char *dst = pick(peer, g->recvType_ == 1 ? 1 : 2);
+      if (!dst) return needScratch();
+      LCHECK(copy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts));
     }
   }
+  return flagcxSuccess;
+}
+
+// flagcxC2cPlanner::execute from its first step on (c2c_algo.cc:2142-2290).
+flagcxResult_t Exec::run() {
+  const RankPlan &c = p->ranks[0];
+  const int nr = p->nranks;
+  const bool anyPipe = c.nPipePreSteps_ > 0 || c.nPipePostSteps_ > 0;
+  // when the reference refreshes around sequential steps (c2c_algo.cc:2205-2208,2226-2229,2276-2279)
+  const bool refreshSeq = p->algorithm == 0 || !anyPipe;
+  const bool refreshAfterInter = p->algorithm == 1 && anyPipe;
+  // Every rank walks ITS OWN tables: it runs hetero function i of a step while
+  // i < heteroFuncSteps_[s].size() for itself, and behind it homoInter function i if its own
+  // homoInterFuncSteps_[s] holds one (c2c_algo.cc:2177-2194,2204-2231,2247-2267).
+  std::vector<char> in(nr), has(nr);
+  auto heteroAt = [&](int hs, size_t i) {
+    bool any = false;
+    for (int r = 0; r < nr; r++) {
+      auto &t = p->ranks[r].heteroFuncSteps_;
+      in[r] = hs < (int)t.size() && i < t[hs].size();
+      any = any || in[r];
+    }
+    return any;
+  };
+  auto interAt = [&](int hs, size_t i) {
+    bool any = false;
+    for (int r = 0; r < nr; r++) {
+      auto &t = p->ranks[r].homoInterFuncSteps_;
+      has[r] = in[r] && hs < (int)t.size() && i < t[hs].size();
+      any = any || has[r];
+    }
+    return any;
+  };
+  auto heteroWidth = [&](int hs) {
+    size_t w = 0;
+    for (auto &rp : p->ranks)
+      if (hs < (int)rp.heteroFuncSteps_.size() && rp.heteroFuncSteps_[hs].size() > w) w = rp.heteroFuncSteps_[hs].size();
+    return w;
+  };
+
+  // sequential preHomoFunc steps
+  for (int s = 0; s < c.nSeqPreSteps_; s++) LCHECK(homoStep(&RankPlan::preHomoFuncSteps_, s));
+  LCHECK(refresh(nullptr));
+  // pipelined preHomoFunc + heteroFunc steps
+  for (int s = 0; s < c.nPipePreSteps_; s++) {
+    LCHECK(homoStep(&RankPlan::preHomoFuncSteps_, c.nSeqPreSteps_ + s));
+    for (size_t i = 0; i < heteroWidth(s); i++) {
+      if (!heteroAt(s, i)) continue;
+      LCHECK(heteroSlot(s, (int)i));
+      if (interAt(s, i)) {
+        LCHECK(homoStep(&RankPlan::homoInterFuncSteps_, s, (int)i, &has));
+        LCHECK(refresh(&has));
+      }
+    }
+  }
+  // sequential heteroFunc steps
+  for (int s = 0; s < c.nSeqInterSteps_; s++) {
+    const int hs = c.nPipePreSteps_ + s;
+    for (size_t i = 0; i < heteroWidth(hs); i++) {
+      if (!heteroAt(hs, i)) continue;
+      if (refreshSeq) LCHECK(refresh(&in));
+      LCHECK(heteroSlot(hs, (int)i));
+      if (interAt(hs, i)) {
+        LCHECK(homoStep(&RankPlan::homoInterFuncSteps_, hs, (int)i, &has));
+        if (refreshAfterInter) LCHECK(refresh(&has));
+      }
+    }
+  }
+  // pipelined heteroFunc + postHomoFunc steps
+  for (int s = 0; s < c.nPipePostSteps_; s++) {
+    LCHECK(homoStep(&RankPlan::postHomoFuncSteps_, s));
+    const int hs = c.nPipePreSteps_ + c.nSeqInterSteps_ + s;
+    for (size_t i = 0; i < heteroWidth(hs); i++) {
+      if (!heteroAt(hs, i)) continue;
+      LCHECK(heteroSlot(hs, (int)i));
+      if (interAt(hs, i)) LCHECK(homoStep(&RankPlan::homoInterFuncSteps_, hs, (int)i, &has));
+    }
+  }
+  // sequential postHomoFunc steps
+  for (int s = 0; s < c.nSeqPostSteps_; s++)
+    LCHECK(homoStep(&RankPlan::postHomoFuncSteps_, c.nPipePostSteps_ + s, -1, nullptr, refreshSeq));
+  return finish();
+}
+
+// Zeros that are still due are written, except into the scratch buffers that the reference
+// allocates for the call and frees when it ends (c2c_algo.cc:2122-2129,2292-2295): nobody
+// reads those again.
+flagcxResult_t Exec::finish() {
+  if (!fused) return flagcxSuccess;
+  for (int r = 0; r < p->nranks; r++)
+    if (ownsScratch[r] && scratch && scratch[r])
+      zeros.remove((uintptr_t)scratch[r], (uintptr_t)scratch[r] + p->totalCount * ts);
+  for (auto &z : zeros.ranges()) LCHECK(memsetNow((char *)z.first, z.second - z.first));
   return flagcxSuccess;
 }
 
@@ -590,7 +919,9 @@ flagcxResult_t flagcxLocalPlanCreate(flagcxLocalPlan **plan, int nranks, const i
                                      flagcxRedOp_t redOp) {
   if (!plan || nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS || !clusterIds || totalCount == 0)
     return flagcxInvalidArgument;
-  flagcxLocalPlan *p = new flagcxLocalPlan();
+  flagcxLocalPlan *p = nullptr;
+  try {
+  p = new flagcxLocalPlan();
   p->nranks = nranks;
   p->totalCount = totalCount;
   memcpy(&p->commOp, &commOp, sizeof(int)); // enum bits as they came from the caller
@@ -632,6 +963,10 @@ flagcxResult_t flagcxLocalPlanCreate(flagcxLocalPlan **plan, int nranks, const i
   p->ranks.resize(nranks);
   *plan = p;
   return flagcxSuccess;
+  } catch (...) {
+    delete p;
+    return flagcxSystemError;
+  }
 }
 
 // Number of chunks of plan documents that carry no <nChunks> (those written by
@@ -654,10 +989,14 @@ flagcxResult_t flagcxLocalPlanSetAlltoAllv(flagcxLocalPlan *p, const size_t *sen
   if (!sendCounts || !sDispls || !recvCounts || !rDispls)
     return planFail(p, flagcxInvalidArgument, "sendrecv counts and displacements need to be set for AlltoAllv%s", "");
   const size_t n = (size_t)p->nranks * (size_t)p->nranks;
-  p->sendCounts.assign(sendCounts, sendCounts + n);
-  p->sDispls.assign(sDispls, sDispls + n);
-  p->recvCounts.assign(recvCounts, recvCounts + n);
-  p->rDispls.assign(rDispls, rDispls + n);
+  try {
+    p->sendCounts.assign(sendCounts, sendCounts + n);
+    p->sDispls.assign(sDispls, sDispls + n);
+    p->recvCounts.assign(recvCounts, recvCounts + n);
+    p->rDispls.assign(rDispls, rDispls + n);
+  } catch (...) {
+    return planFail(p, flagcxSystemError, "out of memory%s", "");
+  }
   return flagcxSuccess;
 }
 
@@ -677,9 +1016,38 @@ flagcxResult_t flagcxLocalPlanSetAlgorithm(flagcxLocalPlan *plan, int algorithm)
   return flagcxSuccess;
 }
 
+// 1 (the default): a refresh records the ranges it clears and sums leave out the members
+// that lie in them; 0: every refresh is a zero-fill and every collective reads all of its
+// members, as the reference does.  The receive buffers end with the same bytes either way.
+flagcxResult_t flagcxLocalPlanSetFused(flagcxLocalPlan *plan, int fused) {
+  if (!plan || fused < 0 || fused > 1) return flagcxInvalidArgument;
+  plan->fused = fused != 0;
+  return flagcxSuccess;
+}
+
+// What the last flagcxLocalPlanExecute handed to the kernels: algorithmic bytes (2 B per
+// copied byte, (k + 1) * n * size per k-input reduction, B per cleared byte) and launches.
+flagcxResult_t flagcxLocalPlanGetTraffic(flagcxLocalPlan *plan, uint64_t *bytes, uint64_t *launches) {
+  if (!plan) return flagcxInvalidArgument;
+  if (bytes) *bytes = plan->lastBytes;
+  if (launches) *launches = plan->lastLaunches;
+  return flagcxSuccess;
+}
+
+static flagcxResult_t importXml(flagcxLocalPlan *p, const char *prefix);
+static flagcxResult_t exportXml(flagcxLocalPlan *p, const char *prefix);
+
 // Reads <prefix>_<rank>.xml for every rank (file naming of importXml, c2c_algo.cc:975-976).
 flagcxResult_t flagcxLocalPlanImportXml(flagcxLocalPlan *p, const char *prefix) {
   if (!p || !prefix) return flagcxInvalidArgument;
+  try {
+    return importXml(p, prefix);
+  } catch (...) {
+    return planFail(p, flagcxSystemError, "out of memory while reading %s", prefix);
+  }
+}
+
+static flagcxResult_t importXml(flagcxLocalPlan *p, const char *prefix) {
   for (int r = 0; r < p->nranks; r++) {
     char filename[512];
     snprintf(filename, sizeof(filename), "%s_%d.xml", prefix, r);
@@ -747,6 +1115,14 @@ flagcxResult_t flagcxLocalPlanImportXml(flagcxLocalPlan *p, const char *prefix) 
 // Writes <prefix>_<rank>.xml in the layout of exportXml (c2c_algo.cc:1050-1087).
 flagcxResult_t flagcxLocalPlanExportXml(flagcxLocalPlan *p, const char *prefix) {
   if (!p || !prefix || !p->loaded) return flagcxInvalidArgument;
+  try {
+    return exportXml(p, prefix);
+  } catch (...) {
+    return planFail(p, flagcxSystemError, "out of memory while writing %s", prefix);
+  }
+}
+
+static flagcxResult_t exportXml(flagcxLocalPlan *p, const char *prefix) {
   for (int r = 0; r < p->nranks; r++) {
     char filename[512];
     snprintf(filename, sizeof(filename), "%s_%d.xml", prefix, r);
@@ -799,91 +1175,56 @@ flagcxResult_t flagcxLocalPlanExportXml(flagcxLocalPlan *p, const char *prefix) 
 }
 
 // sendbuffs / recvbuffs / scratchbuffs: host arrays with one device pointer per
-// rank (scratchbuffs may be NULL when no function or refresh names scratch).
+// rank (scratchbuffs, or entries of it, may be NULL for ranks that need none).
 flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan *p, const void *const *sendbuffs, void *const *recvbuffs,
                                       void *const *scratchbuffs, flagcxDataType_t datatype, int root,
                                       flagcxStream_t stream) {
   if (!p || !sendbuffs || !recvbuffs) return flagcxInvalidArgument;
-  if (!p->loaded) return planFail(p, flagcxInvalidUsage, "no plan imported%s", "");
-  // redOp validation of flagcxC2cPlanner::execute (c2c_algo.cc:2047-2053)
-  if (p->redOp != flagcxRedNoOp && p->redOp != flagcxSum && p->redOp != flagcxMax && p->redOp != flagcxMin)
-    return planFail(p, flagcxNotSupported, "Unsupported reduction operation %s%lld", "", p->redOp);
-  if (!flagcxLocalGetDataTypeSize(datatype)) return planFail(p, flagcxInvalidArgument, "unsupported data type%s", "");
-  for (int r = 0; r < p->nranks; r++)
-    if (!sendbuffs[r] || !recvbuffs[r]) return planFail(p, flagcxInvalidArgument, "rank %s%lld has a NULL buffer", "", r);
-  const Bufs b{sendbuffs, recvbuffs, scratchbuffs};
-  const RankPlan &c = p->ranks[0];
-  // staging buffers of the hetero functions (c2c_algo.cc:2129-2137)
-  std::vector<char *> recvTmp(p->nranks), sendTmp(p->nranks);
-  for (int r = 0; r < p->nranks; r++) {
-    char *scratch = scratchbuffs ? (char *)scratchbuffs[r] : nullptr;
-    recvTmp[r] = scratch ? scratch : (char *)recvbuffs[r];
-    const bool fromSend = p->commOp == flagcxCommOpAlltoAll || p->commOp == flagcxCommOpAlltoAllv ||
-                          (p->commOp == flagcxCommOpScatter && r == root) ||
-                          (p->commOp == flagcxCommOpAllGather && p->eachNicPerRank && p->multiNic);
-    sendTmp[r] = fromSend ? (char *)const_cast<void *>(sendbuffs[r]) : recvTmp[r];
-  }
-  // what the homo functions get as root: the root's rank inside its cluster (c2c_algo.cc:2147,2170)
-  const int homoRoot = (root >= 0 && root < p->nranks) ? p->homoRank[root] : root;
-  const bool anyPipe = c.nPipePreSteps_ > 0 || c.nPipePostSteps_ > 0;
-  // when the reference refreshes around sequential steps (c2c_algo.cc:2205-2208,2226-2229,2276-2279)
-  const bool refreshSeq = p->algorithm == 0 || !anyPipe;
-  const bool refreshAfterInter = p->algorithm == 1 && anyPipe;
-  // ranks whose own homoInter table holds a function i in step hs: every rank decides
-  // `homoInterFuncSteps_[s].size() > i` for itself (c2c_algo.cc:2181,2219,2258)
-  std::vector<char> has(p->nranks);
-  auto interAt = [&](int hs, size_t i) {
-    bool any = false;
+  try {
+    if (!p->loaded) return planFail(p, flagcxInvalidUsage, "no plan imported%s", "");
+    // redOp validation of flagcxC2cPlanner::execute (c2c_algo.cc:2047-2053)
+    if (p->redOp != flagcxRedNoOp && p->redOp != flagcxSum && p->redOp != flagcxMax && p->redOp != flagcxMin)
+      return planFail(p, flagcxNotSupported, "Unsupported reduction operation %s%lld", "", p->redOp);
+    if (!flagcxLocalGetDataTypeSize(datatype)) return planFail(p, flagcxInvalidArgument, "unsupported data type%s", "");
+    for (int r = 0; r < p->nranks; r++)
+      if (!sendbuffs[r] || !recvbuffs[r]) return planFail(p, flagcxInvalidArgument, "rank %s%lld has a NULL buffer", "", r);
+    Exec x;
+    x.p = p;
+    x.send = sendbuffs;
+    x.recv = recvbuffs;
+    x.scratch = scratchbuffs;
+    x.dt = datatype;
+    x.ts = flagcxLocalGetDataTypeSize(datatype);
+    x.stream = stream;
+    x.fused = p->fused;
+    // what the homo functions get as root: the root's rank inside its cluster (c2c_algo.cc:2147,2170)
+    x.homoRoot = (root >= 0 && root < p->nranks) ? p->homoRank[root] : root;
+    // Staging buffers of the hetero functions.  The reference allocates a scratch buffer for a
+    // ReduceScatter, a Scatter and on the non-root ranks of a Gather, and nowhere else
+    // (c2c_algo.cc:2121-2129); where it does, hetero receives land there, everywhere else in
+    // recvbuff (c2c_algo.cc:2131-2137).  A scratch pointer handed over for a rank that has none
+    // in the reference is only what functions that name scratch explicitly get.
+    x.ownsScratch.assign(p->nranks, 0);
+    x.recvTmp.resize(p->nranks);
+    x.sendTmp.resize(p->nranks);
     for (int r = 0; r < p->nranks; r++) {
-      auto &t = p->ranks[r].homoInterFuncSteps_;
-      has[r] = hs < (int)t.size() && i < t[hs].size();
-      any = any || has[r];
+      x.ownsScratch[r] = p->commOp == flagcxCommOpReduceScatter || p->commOp == flagcxCommOpScatter ||
+                         (p->commOp == flagcxCommOpGather && r != root);
+      char *scratch = scratchbuffs ? (char *)scratchbuffs[r] : nullptr;
+      // (a plan that never stages anything there runs without one; what needs it says so when it gets there)
+      x.recvTmp[r] = x.ownsScratch[r] ? scratch : (char *)recvbuffs[r];
+      const bool fromSend = p->commOp == flagcxCommOpAlltoAll || p->commOp == flagcxCommOpAlltoAllv ||
+                            (p->commOp == flagcxCommOpScatter && r == root) ||
+                            (p->commOp == flagcxCommOpAllGather && p->eachNicPerRank && p->multiNic);
+      x.sendTmp[r] = fromSend ? (char *)const_cast<void *>(sendbuffs[r]) : x.recvTmp[r];
     }
-    return any;
-  };
-
-  // sequential preHomoFunc steps
-  for (int s = 0; s < c.nSeqPreSteps_; s++)
-    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, s, b, datatype, homoRoot, stream));
-  LCHECK(runRefresh(p, b, datatype, stream));
-  // pipelined preHomoFunc + heteroFunc steps
-  for (int s = 0; s < c.nPipePreSteps_; s++) {
-    LCHECK(runHomoStep(p, &RankPlan::preHomoFuncSteps_, c.nSeqPreSteps_ + s, b, datatype, homoRoot, stream));
-    for (size_t i = 0; i < heteroWidth(p, s); i++) {
-      LCHECK(runHeteroSlot(p, s, (int)i, sendTmp, recvTmp, datatype, stream));
-      if (interAt(s, i)) {
-        LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, s, b, datatype, homoRoot, stream, (int)i));
-        LCHECK(runRefresh(p, b, datatype, stream, &has));
-      }
-    }
+    const flagcxResult_t res = x.run();
+    p->lastBytes = x.bytes;
+    p->lastLaunches = x.launches;
+    return res;
+  } catch (...) {
+    return planFail(p, flagcxSystemError, "out of memory while replaying the plan%s", "");
   }
-  // sequential heteroFunc steps
-  for (int s = 0; s < c.nSeqInterSteps_; s++) {
-    const int hs = c.nPipePreSteps_ + s;
-    for (size_t i = 0; i < heteroWidth(p, hs); i++) {
-      if (refreshSeq) LCHECK(runRefresh(p, b, datatype, stream));
-      LCHECK(runHeteroSlot(p, hs, (int)i, sendTmp, recvTmp, datatype, stream));
-      if (interAt(hs, i)) {
-        LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, homoRoot, stream, (int)i));
-        if (refreshAfterInter) LCHECK(runRefresh(p, b, datatype, stream, &has));
-      }
-    }
-  }
-  // pipelined heteroFunc + postHomoFunc steps
-  for (int s = 0; s < c.nPipePostSteps_; s++) {
-    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, s, b, datatype, homoRoot, stream));
-    const int hs = c.nPipePreSteps_ + c.nSeqInterSteps_ + s;
-    for (size_t i = 0; i < heteroWidth(p, hs); i++) {
-      LCHECK(runHeteroSlot(p, hs, (int)i, sendTmp, recvTmp, datatype, stream));
-      if (interAt(hs, i))
-        LCHECK(runHomoStep(p, &RankPlan::homoInterFuncSteps_, hs, b, datatype, homoRoot, stream, (int)i));
-    }
-  }
-  // sequential postHomoFunc steps
-  for (int s = 0; s < c.nSeqPostSteps_; s++)
-    LCHECK(runHomoStep(p, &RankPlan::postHomoFuncSteps_, c.nPipePostSteps_ + s, b, datatype, homoRoot, stream, -1,
-                       refreshSeq));
-  return flagcxSuccess;
 }
 
 } // extern "C"

@@ -18,6 +18,7 @@ struct ReduceCall {
   int op;         // flagcxRedOp_t value
   hipStream_t stream;
   int anyOrder;   // this launch need not wait for the launch before it on the stream to finish (chunks of one call)
+  int plusZero;   // op is a sum and the fold also holds members, not listed in src, that are all zeros (kSumZ)
 };
 
 // Cached per-process facts about the device the library runs on.

@@ -27,6 +27,14 @@ namespace flagcx_amd {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 enum : int { kSum = 0, kProd = 1, kMax = 2, kMin = 3, kAvg = 4 };
+// Internal to the library (no flagcxRedOp_t value): the sum of a member list of which only
+// some members are read because the others are known to hold nothing but zeros.  The fold
+// over the full list differs from the fold over the members read in one thing only: a sum
+// whose addends are all -0.0 comes out +0.0 once a +0.0 takes part, wherever in the list it
+// stands.  So the members read are summed in their order and +0.0 is added once at the end,
+// before the one rounding of the 16-bit types.  Floating-point types only; an integer
+// sum needs nothing of the kind.
+enum : int { kSumZ = 5 };
 
 // Element tags for the two 16-bit float formats (raw bit carriers).
 struct f16 { uint16_t bits; };
@@ -118,6 +126,7 @@ struct Fold<T, OP, false, false> {
     return (OP == kProd) ? (acc_t)((acc_t)a * b) : (acc_t)((acc_t)a + b);
   }
   static __device__ __forceinline__ T fin(acc_t acc, int k) {
+    if (OP == kSumZ) acc = (acc_t)(acc + (acc_t)0); // -0.0 -> +0.0, every other value unchanged
     return (OP == kAvg) ? (T)((T)acc / (T)k) : (T)acc;
   }
 };
@@ -132,6 +141,7 @@ struct Fold<T, OP, true, false> {
   }
   static __device__ __forceinline__ T fin(acc_t acc, int k) {
     if (OP == kAvg) acc = acc / (float)k;
+    if (OP == kSumZ) acc = acc + 0.0f;
     T out;
     narrow(acc, out);
     return out;

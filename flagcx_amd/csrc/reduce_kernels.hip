@@ -144,7 +144,8 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   if (tiles < 1) tiles = 1;
   if (p.run > 1) tiles = (tiles + 8ull * p.run - 1) / (8ull * p.run) * (8ull * p.run);
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  const int lds = ldsReservation(shape.waves);
+  // a launch of fewer workgroups than there are CUs cannot exceed any cap: no reservation to set up
+  const int lds = tiles <= (uint64_t)deviceInfo().numCU ? 0 : ldsReservation(shape.waves);
   if (c.anyOrder) {
     if (p.lead == 0 && p.run == 1)
       hipExtLaunchKernelGGL((reduceWaveKernel<elem_t, OP, K, U, false>), dim3((unsigned)tiles), dim3(64), lds, c.stream,
@@ -456,9 +457,18 @@ int FLAGCX_CAT(launchReduceGated_, FLAGCX_DT)(const ReduceCall *calls, int n, co
   }
 }
 
+// Sums whose member list holds all-zero members that are not read: floating-point types
+// add +0.0 once (kSumZ); for integers the sum of the members read is already the result.
+#if FLAGCX_DT >= 6
+#define FLAGCX_SUM_WITH_ZEROS kSumZ
+#else
+#define FLAGCX_SUM_WITH_ZEROS kSum
+#endif
+
 // n reductions that share k, op and stream.
 int FLAGCX_CAT(launchReduceBatch_, FLAGCX_DT)(const ReduceCall *calls, int n) {
   if (n <= 0) return 0;
+  if (calls[0].plusZero) return calls[0].op == kSum ? launchBatchOp<FLAGCX_SUM_WITH_ZEROS>(calls, n) : (int)hipErrorInvalidValue;
   switch (calls[0].op) {
     case kSum: return launchBatchOp<kSum>(calls, n);
     case kProd: return launchBatchOp<kProd>(calls, n);
@@ -519,6 +529,7 @@ int FLAGCX_CAT(launchReduceQueue_, FLAGCX_DT)(int op, const QueueKernelArgs &q, 
 }
 
 int FLAGCX_CAT(launchReduce_, FLAGCX_DT)(const ReduceCall &c) {
+  if (c.plusZero) return c.op == kSum ? launchOp<FLAGCX_SUM_WITH_ZEROS>(c) : (int)hipErrorInvalidValue;
   switch (c.op) {
     case kSum: return launchOp<kSum>(c);
     case kProd: return launchOp<kProd>(c);

@@ -120,7 +120,7 @@ EXPORTS = [
     "flagcxLocalRefresh", "flagcxLocalPack", "flagcxLocalUnpack", "flagcxLocalPackList",
     "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
     "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
-    "flagcxLocalReduceBatch", "flagcxLocalReduceTriggers",
+    "flagcxLocalReduceBatch", "flagcxLocalReduceBatchSparse", "flagcxLocalReduceTriggers",
     "flagcxLocalGateCreate", "flagcxLocalGateDestroy", "flagcxLocalReduceBatchGated", "flagcxLocalGateOpen",
     "flagcxLocalGateQuery", "flagcxLocalGateOwnStream",
     "flagcxLocalFifoInit", "flagcxLocalFifoDestroy", "flagcxLocalFifoDequeue", "flagcxLocalP2pDemo",
@@ -128,7 +128,7 @@ EXPORTS = [
     "flagcxLocalRingReduceScatter",
     "flagcxLocalGetDeviceAdaptor", "flagcxLocalDeviceAdaptorLayout",
     "flagcxLocalPlanCreate", "flagcxLocalPlanDestroy", "flagcxLocalPlanImportXml", "flagcxLocalPlanExportXml",
-    "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanSetChunks", "flagcxLocalPlanSetAlltoAllv", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
+    "flagcxLocalPlanSetAlgorithm", "flagcxLocalPlanSetFused", "flagcxLocalPlanGetTraffic", "flagcxLocalPlanSetChunks", "flagcxLocalPlanSetAlltoAllv", "flagcxLocalPlanExecute", "flagcxLocalPlanGetLastError",
     "flagcxLocalReduceFifoCreate", "flagcxLocalReduceFifoDestroy", "flagcxLocalReduceFifoStart",
     "flagcxLocalReduceFifoStop", "flagcxLocalReduceFifoEnqueue", "flagcxLocalReduceFifoEnqueueReduce",
     "flagcxLocalReduceFifoQuery", "flagcxLocalReduceFifoWait", "flagcxLocalReduceFifoGetGrid",
@@ -188,6 +188,7 @@ def lib():
         L.flagcxLocalCopyFunc.restype = None
         L.flagcxLocalCopyFunc.argtypes = [sp, C.POINTER(CopyArgs)]
         L.flagcxLocalReduceBatch.argtypes = [C.POINTER(ReduceDesc), i, i, i, i, sp]
+        L.flagcxLocalReduceBatchSparse.argtypes = [C.POINTER(ReduceDesc), i, i, i, i, i, sp]
         L.flagcxLocalReduceTriggers.argtypes = [C.POINTER(ReduceTrigger), i, sp]
         L.flagcxLocalFifoInit.argtypes = [C.POINTER(vp)]
         L.flagcxLocalFifoDestroy.argtypes = [vp]
@@ -206,6 +207,8 @@ def lib():
         L.flagcxLocalPlanImportXml.argtypes = [vp, C.c_char_p]
         L.flagcxLocalPlanExportXml.argtypes = [vp, C.c_char_p]
         L.flagcxLocalPlanSetAlgorithm.argtypes = [vp, i]
+        L.flagcxLocalPlanSetFused.argtypes = [vp, i]
+        L.flagcxLocalPlanGetTraffic.argtypes = [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         L.flagcxLocalPlanSetChunks.argtypes = [vp, sz]
         szp = C.POINTER(C.c_size_t)
         L.flagcxLocalPlanSetAlltoAllv.argtypes = [vp, szp, szp, szp, szp]
@@ -347,6 +350,14 @@ def reduce_batch(descs, op, dtype, nranks, stream="current"):
     check(lib().flagcxLocalReduceBatch(arr, len(descs), nranks, int(dtype), int(op), _sref(st)))
 
 
+def reduce_batch_sparse(descs, op, dtype, nlive, nzero, stream="current"):
+    """descs as reduce_batch, each listing the nlive members that hold data; nzero more members hold zeros."""
+    st = current_stream() if stream == "current" else stream
+    keep = [_ptr_array(list(d[0])) for d in descs]
+    arr = (ReduceDesc * len(descs))(*[ReduceDesc(keep[i], d[1], d[2]) for i, d in enumerate(descs)])
+    check(lib().flagcxLocalReduceBatchSparse(arr, len(descs), nlive, nzero, int(dtype), int(op), _sref(st)))
+
+
 def reduce_triggers(triggers, stream="current"):
     st = current_stream() if stream == "current" else stream
     arr = (ReduceTrigger * len(triggers))(*triggers)
@@ -435,6 +446,16 @@ class Plan:
 
     def set_algorithm(self, algo):
         self._check(lib().flagcxLocalPlanSetAlgorithm(self._h, algo))
+
+    def set_fused(self, fused):
+        """True (default): refreshes are recorded and sums skip the cleared members; False: literal replay."""
+        self._check(lib().flagcxLocalPlanSetFused(self._h, 1 if fused else 0))
+
+    def traffic(self):
+        """(algorithmic bytes, kernel launches) of the last execute."""
+        b, n = C.c_uint64(), C.c_uint64()
+        self._check(lib().flagcxLocalPlanGetTraffic(self._h, C.byref(b), C.byref(n)))
+        return b.value, n.value
 
     def execute(self, send_ptrs, recv_ptrs, scratch_ptrs, dtype, root=-1, stream="current"):
         st = current_stream() if stream == "current" else stream

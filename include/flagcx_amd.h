@@ -250,6 +250,21 @@ flagcxResult_t flagcxLocalReduceBatch(const flagcxLocalReduceDesc *descs, int nd
                                       int nranks, flagcxDataType_t datatype,
                                       flagcxRedOp_t op, flagcxStream_t stream);
 
+/* A batch of sums over member lists of which `nzero` members are known to hold only
+ * zeros and are not read: each descriptor lists the `nlive` members that hold data,
+ * in fold order.  The result has the bytes that flagcxLocalReduceBatch gives over
+ * the full lists with zero-filled buffers in the other places, wherever those stand:
+ * for integers the sum of the members read; for floating-point types that sum plus
+ * +0.0, added once before the rounding of the 16-bit types (zero members change a
+ * sum in one way only: addends that are all -0.0 give +0.0).  This is the call
+ * behind the fused replay of "clear all but the own slice, then all-reduce"
+ * (flagcx/core/c2c_algo.cc:586-608 + 310-336).  nzero == 0 is
+ * flagcxLocalReduceBatch; nzero > 0 with an op other than flagcxSum is
+ * flagcxInvalidArgument. */
+flagcxResult_t flagcxLocalReduceBatchSparse(const flagcxLocalReduceDesc *descs, int ndescs,
+                                            int nlive, int nzero, flagcxDataType_t datatype,
+                                            flagcxRedOp_t op, flagcxStream_t stream);
+
 /* The same batch, launched BEFORE its inputs have arrived: the pipeline chunks of a
  * collective are known when it starts, only their arrival times are not.  Where the
  * reference's proxy would fold a chunk each time a receive completes (the loop
@@ -577,8 +592,9 @@ flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing_t ring, flagcxLo
  * local slice into recvbuff, in the ring's order rank+1, ..., rank - the same
  * bytes as flagcxLocalRingReduceScatter and flagcxLocalReduceScatter.  Calls no
  * hipMalloc / hipFree and creates no stream or event.
- * Limit: (nranks - 1) * roundUp(recvcount * elementSize + (recvbuff mod 16), 256)
- * <= FLAGCX_LOCAL_STATIC_STAGING_BYTES, else flagcxInvalidArgument.  Every call on
+ * Limit: (nranks - 1) * roundUp(recvcount * elementSize + (recvbuff mod 128), 256)
+ * <= FLAGCX_LOCAL_STATIC_STAGING_BYTES, else flagcxInvalidArgument (a staged slice
+ * sits as far into its 128-byte line as recvbuff does into its own).  Every call on
  * a GPU uses that GPU's one staging area: calls on one stream follow one another;
  * calls that overlap in time on different streams of one GPU race on it. */
 #define FLAGCX_LOCAL_STATIC_STAGING_BYTES (8ULL * 1024 * 1024)
@@ -600,9 +616,14 @@ flagcxResult_t flagcxLocalStagedReduceScatterNoAlloc(const void *const *sendbuff
  * three homoTypes and hetero P2P ops become device copies between the ranks'
  * buffers; the refresh function is flagcxLocalRefresh.  `root` of Execute is a
  * global rank and reaches the homo functions as its rank inside its cluster, like
- * globalrank2homorank[root] (c2c_algo.cc:2147,2170).  AlltoAllv is
- * flagcxNotSupported (its counts are call arguments, not part of a plan); a
- * document with negative offsets or counts is flagcxInvalidArgument at import.
+ * globalrank2homorank[root] (c2c_algo.cc:2147,2170).  An AlltoAllv plan takes its
+ * counts and displacements, which are call arguments and not part of a plan, from
+ * flagcxLocalPlanSetAlltoAllv; a document with negative offsets or counts is
+ * flagcxInvalidArgument at import.  Every rank walks its own step tables, as in the
+ * reference: a rank whose table for a step is shorter than its peers' takes no part
+ * in their later functions of that step (c2c_algo.cc:2177,2204,2247,2277), and a
+ * collective that then lacks a member is flagcxInvalidUsage where the reference
+ * would hang.
  * commOp 12 (LocCpy) and 13 (LocRed), reserved by the reference's plan DSL
  * (flagcx/tools/utils.py:43-44), are rank-local copy and
  * recv = OP(send, recv).  Host-side errors of a plan are reported through
@@ -637,8 +658,31 @@ flagcxResult_t flagcxLocalPlanSetAlltoAllv(flagcxLocalPlan_t plan, const size_t 
                                            const size_t *rDispls);
 /* 0 sequential, 1 pipeline, 2 input (default after import). */
 flagcxResult_t flagcxLocalPlanSetAlgorithm(flagcxLocalPlan_t plan, int algorithm);
-/* Host arrays of one device pointer per rank; scratchbuffs may be NULL when the
- * plan never names scratch.  Enqueues everything on `stream`. */
+/* How the refresh function and the sums behind it are replayed.  The reference
+ * assembles a sum across a cluster by clearing, in every member's buffer, all but
+ * the member's own slice (flagcxC2cRefreshFunc::run, c2c_algo.cc:586-608) and then
+ * reducing the whole buffers with the vendor CCL (c2c_algo.cc:310-336), which reads
+ * the zeros back.
+ *   fused = 1 (default): a refresh only records the ranges it clears; copies out of
+ *     such a range move the record, a write ends it, a sum reads only the members
+ *     whose slice holds data (flagcxLocalReduceBatchSparse) and what is still
+ *     recorded for a receive buffer when the plan ends is written then.  Ranges in a
+ *     scratch buffer that the reference allocates for the call and frees at its end
+ *     (c2c_algo.cc:2122-2129,2292-2295) are never written.
+ *   fused = 0: every refresh is a zero-fill (flagcxLocalRefresh) and every
+ *     collective reads all of its members, as the reference does.
+ * Every receive buffer ends with the same bytes either way, signed zeros included. */
+flagcxResult_t flagcxLocalPlanSetFused(flagcxLocalPlan_t plan, int fused);
+/* Algorithmic bytes (2 per copied byte, (k + 1) * count * size per k-input
+ * reduction, 1 per cleared byte) and kernel launches of the last Execute. */
+flagcxResult_t flagcxLocalPlanGetTraffic(flagcxLocalPlan_t plan, uint64_t *bytes, uint64_t *launches);
+/* Host arrays of one device pointer per rank.  Scratch is used where the reference
+ * allocates one for the call - every rank of a ReduceScatter or Scatter, the
+ * non-root ranks of a Gather (c2c_algo.cc:2121-2129): there hetero receives and a
+ * refresh of buffType -1 go to scratchbuffs[rank], which must not be NULL; on every
+ * other rank they go to recvbuffs[rank] (c2c_algo.cc:2131,2157-2158) and the scratch
+ * pointer, which may be NULL, is only what functions that name scratch explicitly
+ * (sendType / recvType / buffType 2) get.  Enqueues everything on `stream`. */
 flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan_t plan, const void *const *sendbuffs,
                                       void *const *recvbuffs, void *const *scratchbuffs,
                                       flagcxDataType_t datatype, int root, flagcxStream_t stream);

@@ -127,7 +127,7 @@ class Model:
             typ = p.rf_type
             start = p.rf_start
             if typ == -1:                                    # c2c_algo.cc:2156-2164
-                typ = 1 if self.scratch[r] is None else 2
+                typ = 2 if self.owns_scratch[r] else 1
                 if self.comm_op in (REDUCESCATTER, ALLREDUCE) and self.algorithm == ALGO_PIPELINE:
                     cl = self.cluster_of[r]
                     start = sum(len(self.members[c]) for c in range(cl)) * self.total // self.n
@@ -137,11 +137,13 @@ class Model:
             b[start:start + p.rf_off] = 0
             b[start + p.rf_off + p.rf_count:start + p.rf_total] = 0
 
-    def _homo(self, table, s, i, root):
-        """Function i of step s of one table on every rank that has it."""
+    def _homo(self, table, s, i, root, only=None):
+        """Function i of step s of one table on every rank that has it (only: and is in that set)."""
         fn = {}
         for r, p in enumerate(self.plans):
             t = getattr(p, table)
+            if only is not None and r not in only:
+                continue
             if s < len(t) and i < len(t[s]):
                 f = t[s][i]
                 if f.homo_type == 1 and not self.is_inter[r]:
@@ -289,13 +291,21 @@ class Model:
 
     def execute(self, send, recv, scratch, root=-1, algorithm=ALGO_INPUT, v_args=None):
         """flagcxC2cPlanner::execute, c2c_algo.cc:2121-2298; buffers are modified in place.
-        v_args: (sendCounts, sDispls, recvCounts, rDispls) of an AlltoAllv, row r = rank r's arrays."""
+        v_args: (sendCounts, sDispls, recvCounts, rDispls) of an AlltoAllv, row r = rank r's arrays.
+        Every rank walks its own tables: it runs hetero function i of a step while i is below the
+        length of ITS hetero table for that step, homoInter function i behind it if its own table
+        holds one, and refreshes where its own loop stands (c2c_algo.cc:2177-2194,2204-2231,
+        2247-2267,2276-2288)."""
         self.v_args = v_args
         self.send, self.recv = send, recv
         self.scratch = scratch if scratch is not None else [None] * self.n
         self.algorithm = algorithm
         homo_root = self._homo_rank(root) if 0 <= root < self.n else root     # globalrank2homorank[root]
-        recv_tmp = [self.recv[r] if self.scratch[r] is None else self.scratch[r] for r in range(self.n)]
+        # the ranks the reference gives a scratch buffer for the call (c2c_algo.cc:2121-2129); hetero
+        # receives land there, and in recvbuff on every other rank (c2c_algo.cc:2131)
+        self.owns_scratch = [self.comm_op in (REDUCESCATTER, SCATTER) or (self.comm_op == GATHER and r != root)
+                             for r in range(self.n)]
+        recv_tmp = [self.scratch[r] if self.owns_scratch[r] else self.recv[r] for r in range(self.n)]
         send_tmp = []
         for r in range(self.n):
             from_send = self.comm_op in (ALLTOALL, ALLTOALLV) or (self.comm_op == SCATTER and r == root) or \
@@ -312,29 +322,33 @@ class Model:
                 self._homo("pre", c.n_seq_pre + s, i, homo_root)
             for i in range(self._width("hetero", s)):
                 self._hetero(s, i, send_tmp, recv_tmp)
-                if self._has("inter", s, i):
-                    self._homo("inter", s, i, homo_root)
-                    self._refresh(self._has("inter", s, i))
+                has = self._has("hetero", s, i) & self._has("inter", s, i)
+                if has:
+                    self._homo("inter", s, i, homo_root, has)
+                    self._refresh(has)
         for s in range(c.n_seq_inter):
             hs = c.n_pipe_pre + s
             for i in range(self._width("hetero", hs)):
+                at = self._has("hetero", hs, i)
                 if algorithm == ALGO_SEQUENTIAL or not any_pipe:
-                    self._refresh()
+                    self._refresh(at)
                 self._hetero(hs, i, send_tmp, recv_tmp)
-                if self._has("inter", hs, i):
-                    self._homo("inter", hs, i, homo_root)
+                has = at & self._has("inter", hs, i)
+                if has:
+                    self._homo("inter", hs, i, homo_root, has)
                     if algorithm == ALGO_PIPELINE and any_pipe:
-                        self._refresh(self._has("inter", hs, i))
+                        self._refresh(has)
         for s in range(c.n_pipe_post):
             for i in range(self._width("post", s)):
                 self._homo("post", s, i, homo_root)
             hs = c.n_pipe_pre + c.n_seq_inter + s
             for i in range(self._width("hetero", hs)):
                 self._hetero(hs, i, send_tmp, recv_tmp)
-                if self._has("inter", hs, i):
-                    self._homo("inter", hs, i, homo_root)
+                has = self._has("hetero", hs, i) & self._has("inter", hs, i)
+                if has:
+                    self._homo("inter", hs, i, homo_root, has)
         for s in range(c.n_seq_post):
             for i in range(self._width("post", c.n_pipe_post + s)):
                 if algorithm == ALGO_SEQUENTIAL or not any_pipe:
-                    self._refresh()
+                    self._refresh(self._has("post", c.n_pipe_post + s, i))
                 self._homo("post", c.n_pipe_post + s, i, homo_root)

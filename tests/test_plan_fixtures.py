@@ -113,10 +113,98 @@ def test_model_gives_the_alltoallv_closed_form():
         assert np.array_equal(recv[r], want[r]), r
 
 
+CL4 = [0, 0, 1, 1]
+
+
+def int_inputs(nr, n, seed, npdt=np.int32):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(-2**26, 2**26, n).astype(npdt) for _ in range(nr)]
+
+
+def junk(n, npdt, byte):
+    return np.frombuffer(bytes([byte]) * (n * np.dtype(npdt).itemsize), dtype=npdt).copy()
+
+
+@pytest.mark.parametrize("algo", [M.ALGO_SEQUENTIAL, M.ALGO_INPUT])
+def test_model_gives_the_reducescatter_closed_form(algo):
+    """2 clusters of 4 as findStrategy lays the sequential reduce-scatter out: every staging
+    step in scratch, rank r ends with the sum of everybody's r-th block and nothing else of
+    its receive buffer is touched.  Under `sequential` the refreshes run where
+    c2c_algo.cc:2205-2208 and 2276-2282 put them, which the closed form needs: without the one
+    before the post function every block would come out four times too large."""
+    rc = 33
+    n = 8 * rc
+    hosts = int_inputs(8, n, 21)
+    m = M.Model(fixture("reducescatter8"), CL8, n, M.REDUCESCATTER, M.SUM, default_chunks=8)
+    recv = [junk(n, np.int32, 0x55) for _ in range(8)]
+    m.execute([h.copy() for h in hosts], recv, [junk(n, np.int32, 0x33) for _ in range(8)], algorithm=algo)
+    total = sum(hosts)
+    for r in range(8):
+        assert np.array_equal(recv[r][:rc], total[r * rc:(r + 1) * rc]), r
+        assert np.array_equal(recv[r][rc:], junk(n - rc, np.int32, 0x55)), r
+    # the reference's own reduce-scatter pattern, floor(i / recvcount) on every rank: shard r = 8 r
+    pat = [(np.arange(n) // rc).astype(np.float32) for _ in range(8)]
+    recv = [np.full(n, -1, dtype=np.float32) for _ in range(8)]
+    m.execute(pat, recv, [np.full(n, -2, dtype=np.float32) for _ in range(8)], algorithm=algo)
+    for r in range(8):
+        assert np.array_equal(recv[r][:rc], np.full(rc, 8.0 * r, dtype=np.float32)), r
+
+
+@pytest.mark.parametrize("root", [6, 4])
+def test_model_gives_the_reduce_closed_form(root):
+    n = 4 * 29
+    hosts = int_inputs(8, n, 22)
+    m = M.Model(fixture("reduce8"), CL8, n, M.REDUCE, M.SUM, default_chunks=4)
+    recv = [junk(n, np.int32, 0x55) for _ in range(8)]
+    m.execute([h.copy() for h in hosts], recv, None, root=root, algorithm=M.ALGO_SEQUENTIAL)
+    assert np.array_equal(recv[root], sum(hosts))
+
+
+def test_model_gives_the_gather_closed_form():
+    """Root 3 sits in the second cluster and stages its hetero receive in its RECEIVE buffer, the
+    other ranks in scratch (c2c_algo.cc:2122-2131): the model, given scratch for every rank, must
+    still take recv on the root, or block 1 of the result is not rank 1's."""
+    s_ = 17
+    n = 4 * s_
+    hosts = int_inputs(4, n, 23)
+    m = M.Model(fixture("gather4"), CL4, n, M.GATHER, 5, default_chunks=4)
+    recv = [junk(n, np.int32, 0x55) for _ in range(4)]
+    m.execute([h.copy() for h in hosts], recv, [junk(n, np.int32, 0x33) for _ in range(4)], root=3)
+    assert np.array_equal(recv[3], np.concatenate([h[:s_] for h in hosts]))
+    for r in range(3):
+        assert np.array_equal(recv[r], junk(n, np.int32, 0x55)), r
+
+
+def uneven4_expected(hosts, c):
+    """By hand.  T = sum over the four ranks, halves T0 = T[:2c], T1 = T[2c:].  After hetero
+    function 0 and the all-reduce behind it every rank holds T.  Function 1 exists on ranks 0
+    and 2 only: they alone refresh again (keep their first half) and swap it into each other's
+    second half: [T0, T0].  The post function exists in cluster 0 only: ranks 0 and 1 refresh
+    (rank 1 keeps its second half) and rank 1 broadcasts: both end with [0, T1].  Ranks 2 and 3
+    are not refreshed again: [T0, T0] and T."""
+    t = sum(hosts)
+    t0, t1, z = t[:2 * c], t[2 * c:], np.zeros(2 * c, dtype=t.dtype)
+    return [np.concatenate([z, t1]), np.concatenate([z, t1]), np.concatenate([t0, t0]), t]
+
+
+@pytest.mark.parametrize("algo", [M.ALGO_SEQUENTIAL, M.ALGO_PIPELINE, M.ALGO_INPUT])
+def test_model_walks_every_ranks_own_tables(algo):
+    """Ranks with fewer functions in a step leave its loop earlier (c2c_algo.cc:2204,2277) and are
+    not refreshed again; a lock-step replay would wipe rank 3's first half."""
+    c = 11
+    n = 4 * c
+    hosts = int_inputs(4, n, 24)
+    m = M.Model(fixture("uneven4"), CL4, n, M.ALLREDUCE, M.SUM, default_chunks=4)
+    recv = [junk(n, np.int32, 0x55) for _ in range(4)]
+    m.execute([h.copy() for h in hosts], recv, None, algorithm=algo)
+    for r, want in enumerate(uneven4_expected(hosts, c)):
+        assert np.array_equal(recv[r], want), r
+
+
 # ------------------------------------------------------------------ GPU: replay
 
 def run_both(prefix, clusters, n, commop, redop, hosts, dt, algo, root=-1, chunks=None, scratch=False, is_inter=None,
-             recv_fill=0x55):
+             recv_fill=0x55, fused=True):
     """Replays the plan on the GPU and in the numpy model from the same inputs;
     returns (gpu recv arrays, model recv arrays, gpu send arrays after the run)."""
     import torch
@@ -128,9 +216,10 @@ def run_both(prefix, clusters, n, commop, redop, hosts, dt, algo, root=-1, chunk
         plan.set_chunks(chunks)
     plan.import_xml(prefix)
     plan.set_algorithm(algo)
+    plan.set_fused(fused)
     send = [to_dev(h) for h in hosts]
-    recv = [dev_empty(n, ts, fill=recv_fill) for _ in range(nr)]
-    scr = [dev_empty(n, ts, fill=0x33) for _ in range(nr)] if scratch else None
+    recv = [to_dev(np.frombuffer(bytes([recv_fill]) * (n * ts), dtype=npdt)) for _ in range(nr)]     # the byte, repeated
+    scr = [to_dev(np.frombuffer(bytes([0x33]) * (n * ts), dtype=npdt)) for _ in range(nr)] if scratch else None
     plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv],
                  [s.data_ptr() for s in scr] if scr else None, dt, root=root)
     torch.cuda.synchronize()
@@ -282,7 +371,8 @@ def send_recv_plan(prefix):
         if r == 0:
             pre, inter = [[PX.homo(SEND, 0, 1, 0, 0, 1, 0, rootRank=0)]], [[PX.homo(RECV, 1, 1, 0, 0, 6, 1)]]
             post = [[PX.homo(SEND, 1, 1, 2, 0, 2, 2, rootRank=1)]]
-            het = [[]]
+            het = [[[]]]    # a hetero function without P2P ops, as findStrategy pushes one for every rank
+                            # (c2c_algo.cc:1763-1766): with none at all the rank would never reach its inter function
         elif r == 1:
             pre, inter = [[PX.homo(RECV, 0, 1, 0, 4, 1, 0, rootRank=0)]], [[PX.homo(SEND, 1, 1, 0, 0, 6, 1)]]
             post = [[PX.homo(RECV, 1, 1, 0, 0, 2, 2, rootRank=1)]]
@@ -295,8 +385,9 @@ def send_recv_plan(prefix):
 
 @pytest.mark.gpu
 def test_send_recv_homo_functions_of_all_three_types(tmp_path):
-    """Send / Recv homo functions (c2c_algo.cc:364-463).  The hetero sends read the recv
-    buffer (sendTmp = recvTmp for a gather), so ranks 2 and 3 send their recv fill."""
+    """Send / Recv homo functions (c2c_algo.cc:364-463).  The collective is a gather to rank 1:
+    every other rank stages its hetero functions in scratch (c2c_algo.cc:2122-2137), so ranks 2
+    and 3 send what their scratch buffers hold, and the root receives into its receive buffer."""
     import torch
     prefix = str(tmp_path / "sr")
     send_recv_plan(prefix)
@@ -309,24 +400,129 @@ def test_send_recv_homo_functions_of_all_three_types(tmp_path):
     send = [to_dev(h) for h in hosts]
     fills = [np.full(n, 1000 + r, dtype=np.int32) for r in range(4)]
     recv = [to_dev(f) for f in fills]
-    plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, O.INT32, root=1)
+    scr = [to_dev(np.full(n, 2000 + r, dtype=np.int32)) for r in range(4)]
+    # without scratch the ranks that stage there cannot run their hetero functions
+    with pytest.raises(local.FlagcxError) as e:
+        plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], None, O.INT32, root=1)
+    assert e.value.code == int(local.Result.InvalidArgument) and "scratch" in str(e.value)
+    recv = [to_dev(f) for f in fills]
+    plan.execute([s.data_ptr() for s in send], [r.data_ptr() for r in recv], [s.data_ptr() for s in scr], O.INT32, root=1)
     torch.cuda.synchronize()
     got = [from_dev(r, np.int32) for r in recv]
     # by hand: rank 1 gets send_0's first chunk at chunk 4, the two hetero pieces at chunks 2 and 3
-    # (the senders' recv fill), rank 0 gets those two pieces at the same place, and finally rank 1
+    # (the senders' scratch fill), rank 0 gets those two pieces at the same place, and finally rank 1
     # gets them at chunks 0 and 1
     want0 = fills[0].copy()
-    want0[2 * c:3 * c], want0[3 * c:4 * c] = 1002, 1003
+    want0[2 * c:3 * c], want0[3 * c:4 * c] = 2002, 2003
     want1 = fills[1].copy()
     want1[4 * c:5 * c] = hosts[0][:c]
-    want1[2 * c:3 * c], want1[3 * c:4 * c] = 1002, 1003
-    want1[0:c], want1[c:2 * c] = 1002, 1003
+    want1[2 * c:3 * c], want1[3 * c:4 * c] = 2002, 2003
+    want1[0:c], want1[c:2 * c] = 2002, 2003
     assert same(got[0], want0)
     assert same(got[1], want1)
     assert same(got[2], fills[2]) and same(got[3], fills[3])
     # and the same from the model
     m = M.Model(prefix, [0, 0, 1, 1], n, M.GATHER, M.SUM)
     mrecv = [f.copy() for f in fills]
-    m.execute([h.copy() for h in hosts], mrecv, None, root=1)
+    m.execute([h.copy() for h in hosts], mrecv, [np.full(n, 2000 + r, dtype=np.int32) for r in range(4)], root=1)
     for r in range(4):
         assert same(got[r], mrecv[r]), r
+
+
+def case_inputs(dt, nr, n, seed):
+    """Random inputs, the numpy carrier type, and whether sums are exact (closed form usable)."""
+    rng = np.random.default_rng(seed)
+    if dt == O.FP32:
+        return [rng.standard_normal(n).astype(np.float32) for _ in range(nr)], False
+    if dt == O.INT32:
+        return [rng.integers(-2**26, 2**26, n).astype(np.int32) for _ in range(nr)], True
+    raise ValueError(dt)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "literal"])
+@pytest.mark.parametrize("algo", [0, 2], ids=["sequential", "input"])
+@pytest.mark.parametrize("dt", [O.FP32, O.INT32])
+def test_reducescatter8_fixture_with_scratch(dt, algo, fused):
+    """The sequential reduce-scatter of findStrategy for 2 clusters of 4, replayed with scratch:
+    cluster sums into scratch, quarters across, all-reduce of the scratch buffers (2 of 4 members
+    hold data per quarter), refresh, reduce-scatter out of scratch (1 of 4).  Same bytes as the
+    numpy model, the closed form for integers, recv beyond the shard untouched."""
+    rc = 20011
+    n = 8 * rc
+    hosts, exact = case_inputs(dt, 8, n, 31 + dt)
+    got, want, sent = run_both(fixture("reducescatter8"), CL8, n, 8, local.RedOp.Sum, hosts, dt, algo, chunks=8,
+                               scratch=True, fused=fused)
+    total = sum(hosts)
+    for r in range(8):
+        assert same(got[r], want[r]), (algo, r)
+        assert same(sent[r], hosts[r])
+        assert same(got[r][rc:], junk(n - rc, hosts[0].dtype, 0x55)), r
+        if exact:
+            assert same(got[r][:rc], total[r * rc:(r + 1) * rc]), r
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "literal"])
+@pytest.mark.parametrize("root", [6, 5])
+@pytest.mark.parametrize("dt", [O.FP32, O.INT32])
+def test_reduce8_fixture_root_in_the_second_cluster(dt, root, fused):
+    n = 4 * 15013
+    hosts, exact = case_inputs(dt, 8, n, 41 + dt)
+    got, want, sent = run_both(fixture("reduce8"), CL8, n, 5, local.RedOp.Sum, hosts, dt, 0, root=root, chunks=4,
+                               fused=fused)
+    for r in range(8):
+        assert same(got[r], want[r]), r
+        assert same(sent[r], hosts[r])
+    if exact:
+        assert same(got[root], sum(hosts))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "literal"])
+def test_gather4_fixture_root_stages_in_its_receive_buffer(fused):
+    """Root 3 in the second cluster; scratch handed over for EVERY rank.  The reference gives the
+    root no scratch buffer (c2c_algo.cc:2122-2129), so its hetero receive lands in recvbuff, where
+    its Send function of homoType 1 then reads it."""
+    s_ = 9001
+    n = 4 * s_
+    hosts = int_inputs(4, n, 51)
+    got, want, sent = run_both(fixture("gather4"), CL4, n, 3, 5, hosts, O.INT32, 0, root=3, chunks=4, scratch=True,
+                               fused=fused)
+    assert same(got[3], np.concatenate([h[:s_] for h in hosts]))
+    for r in range(4):
+        assert same(got[r], want[r]), r
+        assert same(sent[r], hosts[r])
+        if r != 3:
+            assert same(got[r], junk(n, np.int32, 0x55)), r
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "literal"])
+@pytest.mark.parametrize("algo", [0, 1, 2], ids=["sequential", "pipeline", "input"])
+def test_uneven4_fixture_every_rank_walks_its_own_tables(algo, fused):
+    c = 7001
+    n = 4 * c
+    hosts = int_inputs(4, n, 61)
+    got, want, _ = run_both(fixture("uneven4"), CL4, n, 6, local.RedOp.Sum, hosts, O.INT32, algo, chunks=4, fused=fused)
+    for r, by_hand in enumerate(uneven4_expected(hosts, c)):
+        assert same(got[r], by_hand), r
+        assert same(got[r], want[r]), r
+
+
+@pytest.mark.gpu
+def test_a_collective_that_lacks_a_member_is_refused(tmp_path):
+    """Rank 1 has no hetero function in the sequential step, so in the reference it never reaches
+    the all-reduce behind it, which its cluster then waits for forever; here: flagcxInvalidUsage."""
+    prefix = str(tmp_path / "lack")
+    for r in range(4):
+        het = [[]] if r == 1 else [[[]]]                  # <Step/> against a step with one empty function
+        inter = [[PX.homo(PX.ALLREDUCE, 1, 1, 0, 0, 4, 0)]]
+        PX.write_rank(prefix, r, 4, (0, 0, 1, 0, 0), PX.NO_REFRESH, [], het, inter, [])
+    n = 4 * 100
+    plan = local.Plan(CL4, n, 6, local.RedOp.Sum)
+    plan.import_xml(prefix)
+    bufs = [dev_empty(n, 4, fill=1) for _ in range(8)]
+    with pytest.raises(local.FlagcxError) as e:
+        plan.execute([b.data_ptr() for b in bufs[:4]], [b.data_ptr() for b in bufs[4:]], None, O.INT32)
+    assert e.value.code == int(local.Result.InvalidUsage) and "rank 1" in str(e.value)
