@@ -33,6 +33,7 @@ Tables (human-readable, no JSON line; the summaries under profiles/ come from th
   --table sweep         C5: 1 KiB .. 1 GiB, 2-input fp32 sum, pack, unpack, copy, fill
   --table sweep-rotate  the same over several sets of buffers in turn, from --min on
   --table configs       every C1 / C3 / C4 row incl. HIP graph, staging ring, gather
+  --table plan          C2C plan replay, literal and fused (--plan-name, --plan-mode, --plan-iters)
   --table dtypes        every element type x operation, --k inputs of --mib MiB
   --table stride        k-input reduce against the inputs' relative placement,
                         wavefronts per CU and inputs in flight
@@ -537,7 +538,7 @@ def config_headline_variants(L, inputs):
     return rows
 
 
-def config_plan_replay(L, mib=128, iters=10):
+def config_plan_replay(L, mib=128, iters=10, only=None, modes=(False, True)):
     """C2C plan replay: the plan documents under tests/golden/plans (written by the reference's
     plan DSL) replayed for all ranks on this GPU, the literal way (every refresh a zero-fill, every
     collective reads all members) and the fused way (sums read the members that hold data).
@@ -549,12 +550,14 @@ def config_plan_replay(L, mib=128, iters=10):
     cl8 = [0, 0, 0, 0, 1, 1, 1, 1]
     n = mib * MiB // 4
     for name, commop, scratch, algo in (("allreduce8", 6, False, 2), ("reducescatter8", 8, True, 0)):
+        if only and name != only:
+            continue
         try:
             send = [torch.empty(n, dtype=torch.float32, device="cuda").uniform_(-1, 1) for _ in range(8)]
             recv = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(8)]
             scr = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(8)] if scratch else None
             res, outs = {}, {}
-            for fused in (False, True):
+            for fused in modes:
                 plan = L.Plan(cl8, n, commop, L.RedOp.Sum)
                 plan.set_chunks(8)
                 plan.import_xml(os.path.join(plans, name))
@@ -566,6 +569,10 @@ def config_plan_replay(L, mib=128, iters=10):
                 res[fused] = (ms,) + plan.traffic()
                 outs[fused] = [t[:n // 8 if commop == 8 else n].clone() for t in recv]
                 plan.close()
+            if len(res) < 2:      # one mode only (profiling runs): its own bytes
+                for fused, (ms, issued, launches) in res.items():
+                    rows["plan_%s_%s" % (name, "fused" if fused else "literal")] = row(issued, ms, launches=int(launches))
+                continue
             same = all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(outs[False], outs[True]))
             need = res[True][1]
             for fused, tag in ((False, "literal"), (True, "fused")):
@@ -736,6 +743,20 @@ def table_configs(L, args):
                                                                       100 * r["frac"], extra), flush=True)
 
 
+def table_plan(L, args):
+    """C2C plan replay rows only: --plan-name allreduce8|reducescatter8, --plan-mode literal|fused|both."""
+    modes = {"literal": (False,), "fused": (True,), "both": (False, True)}[args.plan_mode]
+    rows = config_plan_replay(L, mib=args.mib if args.mib != 256 else 128, iters=args.plan_iters, only=args.plan_name,
+                              modes=modes)
+    for name, r in rows.items():
+        if not isinstance(r, dict) or "bytes" not in r:
+            print("%-36s %s" % (name, r), flush=True)
+            continue
+        extra = "  ".join("%s=%s" % (k, v) for k, v in r.items() if k not in ("bytes", "ms", "gbps", "frac", "note"))
+        print("%-32s %14d B  %9.4f ms  %8.1f GB/s  %5.1f %%  %s" % (name, r["bytes"], r["ms"], r["gbps"],
+                                                                      100 * r["frac"], extra), flush=True)
+
+
 def table_dtypes(L, args):
     import torch
     lib = L.lib()
@@ -883,7 +904,10 @@ def main():
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also run N flagcxLocalMemcpy launches of 256 MiB (a copy of known size "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--table", choices=["sweep", "sweep-rotate", "configs", "dtypes", "stride", "positions"],
+    ap.add_argument("--plan-name", default=None, help="plan table: allreduce8 or reducescatter8 (default both)")
+    ap.add_argument("--plan-mode", default="both", choices=["literal", "fused", "both"], help="plan table: which replay")
+    ap.add_argument("--plan-iters", type=int, default=10, help="plan table: timed replays per row")
+    ap.add_argument("--table", choices=["sweep", "sweep-rotate", "configs", "dtypes", "stride", "positions", "plan"],
                     help="print one of the tables instead of the JSON line")
     ap.add_argument("--min", type=int, default=1 << 10, help="sweep tables: smallest size")
     ap.add_argument("--max", type=int, default=1 << 30, help="sweep tables: largest size")
@@ -909,7 +933,7 @@ def main():
 
     if args.table:
         {"sweep": table_sweep, "sweep-rotate": table_sweep, "configs": table_configs, "dtypes": table_dtypes,
-         "stride": table_stride, "positions": table_positions}[args.table](L, args)
+         "stride": table_stride, "positions": table_positions, "plan": table_plan}[args.table](L, args)
         return
 
     # The 8 input buffers and the output live in one allocation, at the addresses
@@ -999,6 +1023,26 @@ def main():
         singles.append((time.perf_counter() - s0) * 1e6)
     singles.sort()
 
+    # what the GPU itself takes per launch: 1000 of them captured once into a HIP graph and replayed
+    graph_us = None
+    try:
+        side = torch.cuda.Stream()
+        sst = L.Stream(side.cuda_stream)
+        ssref = C.byref(sst)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(10):
+                fn(ptrs, 2, cptr, 1024, f32, opsum, ssref)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(1000):
+                fn(ptrs, 2, cptr, 1024, f32, opsum, ssref)
+        graph_us = timed_ms(graph.replay, warmup=3, iters=5)
+        del graph
+    except Exception as e:
+        log("bench.py: graph replay of small launches failed: %r" % (e,))
+
     # the same figure as a C caller sees it (no interpreter in the launch path), beside the runtime's
     # own floor: an empty kernel and a 4 KiB hipMemcpyAsync timed the same way
     c_lat = None
@@ -1027,6 +1071,10 @@ def main():
         "latency_us_4KiB": {"workload": "2-input fp32 sum, 4 KiB per buffer",
                             "c_caller": c_lat,
                             "c_caller_beside_the_runtime_floor": floor,
+                            "hip_graph_replay_per_launch": None if graph_us is None else round(graph_us, 3),
+                            "note": "back to back from a caller, every launch costs what the runtime takes on the host "
+                                    "to launch ANY kernel with arguments (minimal_sum_kernel_4x64, hipMemcpyAsync_d2d); "
+                                    "the GPU itself takes such launches as fast as empty ones (hip_graph_replay_per_launch)",
                             "python_ctypes_caller": {
                                 "back_to_back_per_launch": round(lat_stream_us, 3),
                                 "single_launch_to_sync_median": round(singles[len(singles) // 2], 3)}},

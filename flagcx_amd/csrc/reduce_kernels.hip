@@ -117,6 +117,21 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   p.tail = s.tail;
   p.k = K;
   const uint64_t tileBytes = 64ull * U * 16ull;
+  // Small messages: a launch of no more workgroups than there are CUs is over in one round of
+  // wavefronts, whatever its shape, and what it costs is the host's time per launch (the GPU
+  // takes such launches back to back as fast as empty ones).  So no tiling arithmetic, no shape
+  // lookup, no LDS reservation (nothing to cap), and one runtime call whose return value is the
+  // launch's status.
+  if (!c.anyOrder && (s.nvec * 16 + tileBytes - 1) / tileBytes <= (uint64_t)deviceInfo().numCU) {
+    p.inflight = 0;
+    p.lead = 0;
+    p.run = 1;
+    uint64_t few = (s.nvec * 16 + tileBytes - 1) / tileBytes;
+    if (few < 1) few = 1;
+    void *args[] = {&p};
+    return (int)hipLaunchKernel(reinterpret_cast<const void *>(&reduceWaveKernel<elem_t, OP, K, U, false>), dim3((unsigned)few),
+                                dim3(64), args, 0, c.stream);
+  }
   setTiling(p, c, s);
   uint64_t tiles = (s.nvec * 16 + p.lead + tileBytes - 1) / tileBytes;
   // a limit on the inputs in flight per wavefront trades latency per wavefront for
@@ -144,8 +159,7 @@ static int launchFixed(const ReduceCall &c, const Split &s) {
   if (tiles < 1) tiles = 1;
   if (p.run > 1) tiles = (tiles + 8ull * p.run - 1) / (8ull * p.run) * (8ull * p.run);
   if (tiles > kMaxGrid) tiles = kMaxGrid;
-  // a launch of fewer workgroups than there are CUs cannot exceed any cap: no reservation to set up
-  const int lds = tiles <= (uint64_t)deviceInfo().numCU ? 0 : ldsReservation(shape.waves);
+  const int lds = ldsReservation(shape.waves);
   if (c.anyOrder) {
     if (p.lead == 0 && p.run == 1)
       hipExtLaunchKernelGGL((reduceWaveKernel<elem_t, OP, K, U, false>), dim3((unsigned)tiles), dim3(64), lds, c.stream,

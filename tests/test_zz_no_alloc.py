@@ -129,3 +129,46 @@ def test_no_alloc_entry_point_rejects_what_does_not_fit(L):
     assert call([p, p + 1024], 2, 0, p + 8, 16) == inv           # output overlaps a slice that is read
     assert call([p, p + 1024], 2, 0, p + 2048, 0) == 0           # nothing to do
     torch.cuda.synchronize()
+
+
+def test_no_alloc_entry_point_under_stream_capture_and_without_taking_memory(L):
+    """What the entry point is for.  Captured between hipStreamBeginCapture and
+    hipStreamEndCapture (a call that allocated, freed or synchronised there would end the
+    capture with an error: the capture mode is the strict one), then replayed four times over
+    new inputs with eager work in between, every replay against the oracle, the second shape
+    smaller than the first; and the device's free memory is the same before and after the calls."""
+    import torch
+    dt, op, nranks = O.BF16, O.SUM, 8
+    ts = O.type_size(dt)
+    side = torch.cuda.Stream()
+    for rcount in (200000 + 5, 4099):
+        send_h = make_inputs(dt, nranks, nranks * rcount, seed=91 + rcount % 7, op=op)
+        send = [to_dev(h) for h in send_h]
+        out = dev_empty(rcount + 8, ts, fill=0x5A)
+        rank = 5
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            staged(L, send, rank, out[:rcount], op, dt)        # eager once on the capture stream
+        side.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side, capture_error_mode="global"):
+            staged(L, send, rank, out[:rcount], op, dt)
+        for rep in range(4):
+            perm = np.roll(np.arange(nranks), rep + 1)
+            for j in range(nranks):
+                send[j].copy_(to_dev(send_h[perm[j]]))
+            out.fill_(0x5A5A)
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            rc, want = O.reduce_scatter_rank([send_h[perm[j]] for j in range(nranks)], rank, rcount, dt, op)
+            assert rc == 0
+            assert same(from_dev(out[:rcount], np.uint16), want, nan_class=True, dtype=dt), (rcount, rep)
+            assert bool((out[rcount:] == 0x5A5A).all()), "wrote past the shard"
+        # eager calls take no device memory either
+        for _ in range(3):
+            staged(L, send, rank, out[:rcount], op, dt)
+        torch.cuda.synchronize()
+        del g
+        assert torch.cuda.mem_get_info()[0] >= free_before, "the calls took device memory"
