@@ -190,9 +190,14 @@ def cpu_c1_reference_path():
                                        partial.size, 1)
         assert rc == 0
 
+    evict = np.zeros(96 * 1024 * 1024, dtype=np.float32)     # 384 MiB: larger than the host's caches
+
     def one_pass(threads):
         # rank 0 ends with chunk 0 = in1[0:half] (received) + in0[0:half] (local); rank 1 with chunk 1
         p0, p1 = b[:half].copy(), a[half:].copy()
+        # the reference's partial arrives over a socket, not from a copy made a moment ago: walk
+        # another buffer so that nothing of the operands is left in the caches when the fold starts
+        evict.__iadd__(1.0)
         jobs = [(a[:half], p0), (b[half:], p1)]
         t0 = time.perf_counter()
         if threads == 1:
@@ -219,7 +224,8 @@ def cpu_c1_reference_path():
         "config": "C1: 2-input fp32 sum, 64 MiB per buffer, uniform[-1,1) seed 0, as the reference's 2-rank host "
                   "ring all-reduce folds it (two sum<float> calls over 8 Mi elements each)",
         "value": round(nbytes / res[1] / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind,
-        "sample": "the whole configuration (192 MiB of traffic), median of 5 passes after 1 warm-up",
+        "sample": "the whole configuration (192 MiB of traffic), median of 5 passes after 1 warm-up; operands evicted "
+                  "from the host's caches before every timed fold (a 384 MiB buffer is walked in between)",
         "threads_2": {"value": round(nbytes / res[2] / 1e9, 3), "threads": 2,
                       "note": "one thread per simulated rank, each folding its own chunk"},
         "result_equals_in0_plus_in1": ok,
@@ -285,8 +291,10 @@ def c3_chunk_descs(L, nranks, shard, send, recv, rank):
 
 
 def c3_queue_ms(L, nranks, descs, warmup=5, iters=20):
-    """The shard chunk by chunk through the resident reduce queue: host wall clock from
-    the first enqueue to the return of Wait on the last ticket."""
+    """The shard chunk by chunk through the resident reduce queue.  Returns (ms per shard when
+    `iters` shards are enqueued back to back and the last ticket is waited for, as the other rows
+    are timed; median ms of one shard alone, first enqueue -> return of Wait; resident wavefronts;
+    ms of one 4 KiB entry, enqueue -> Wait)."""
     import torch
     lib = L.lib()
     fifo = L.ReduceFifo(64, nranks, L.DataType.Float16, L.RedOp.Avg)
@@ -296,19 +304,28 @@ def c3_queue_ms(L, nranks, descs, warmup=5, iters=20):
     times = []
     torch.cuda.synchronize()
     lib.flagcxLocalSetMaxSpinCount(1 << 22)
+
+    def shard():
+        for srcs, dst, cnt in arrs:
+            while True:
+                rc = enq(fifo._h, srcs, nranks, dst, cnt, C.byref(ticket))
+                if rc != L.Result.InProgress:
+                    break
+            fifo._check(rc)
+
     try:
         with fifo:
             for it in range(warmup + iters):
                 t0 = time.perf_counter()
-                for srcs, dst, cnt in arrs:
-                    while True:
-                        rc = enq(fifo._h, srcs, nranks, dst, cnt, C.byref(ticket))
-                        if rc != L.Result.InProgress:
-                            break
-                    fifo._check(rc)
+                shard()
                 fifo.wait(ticket.value)
                 if it >= warmup:
                     times.append((time.perf_counter() - t0) * 1e3)
+            t0 = time.perf_counter()
+            for it in range(iters):
+                shard()
+            fifo.wait(ticket.value)
+            steady = (time.perf_counter() - t0) * 1e3 / iters
             grid = fifo.grid()
             # what a shard's wall clock holds beside the folding itself: one 4 KiB entry, enqueue -> Wait
             small = []
@@ -322,12 +339,15 @@ def c3_queue_ms(L, nranks, descs, warmup=5, iters=20):
         fifo.close()
         lib.flagcxLocalSetMaxSpinCount(-1)
     times.sort()
-    return times[len(times) // 2], grid, small[len(small) // 2]
+    return steady, times[len(times) // 2], grid, small[len(small) // 2]
 
 
 def c3_gated_ms(L, nranks, descs, warmup=5, iters=20):
     """The shard as ONE batch launched before any chunk is said to be there, its descriptors opened
-    chunk by chunk: host wall clock from the launch call to the end of the stream synchronisation."""
+    chunk by chunk.  Returns (ms per shard when `iters` shards are launched and opened back to back
+    with one synchronisation at the end, as the other rows are timed; median ms of one shard alone by
+    the host's clock, launch call -> end of the stream synchronisation; the same between two events on
+    the launch's stream)."""
     import torch
     lib = L.lib()
     keep = [(C.c_void_p * nranks)(*d[0]) for d in descs]
@@ -341,26 +361,35 @@ def c3_gated_ms(L, nranks, descs, warmup=5, iters=20):
     gate = L.Gate()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
+
+    def shard():
+        L.check(lib.flagcxLocalReduceBatchGated(gate._h, arr, len(descs), nranks, int(L.DataType.Float16),
+                                                int(L.RedOp.Avg), C.byref(st), C.byref(first)))
+        for c in range(len(descs)):
+            lib.flagcxLocalGateOpen(gate._h, first.value + c + 1)
+
     try:
         for it in range(warmup + iters):
             t0 = time.perf_counter()
             e0.record(side)
-            L.check(lib.flagcxLocalReduceBatchGated(gate._h, arr, len(descs), nranks, int(L.DataType.Float16),
-                                                    int(L.RedOp.Avg), C.byref(st), C.byref(first)))
-            for c in range(len(descs)):
-                lib.flagcxLocalGateOpen(gate._h, first.value + c + 1)
+            shard()
             e1.record(side)
             side.synchronize()
             if it >= warmup:
                 times.append((time.perf_counter() - t0) * 1e3)
                 dev.append(e0.elapsed_time(e1))
+        t0 = time.perf_counter()
+        for it in range(iters):
+            shard()
+        side.synchronize()
+        steady = (time.perf_counter() - t0) * 1e3 / iters
         assert gate.query()[2] == 0, "the gated launch gave up waiting"
     finally:
         gate.destroy()
         lib.flagcxLocalSetMaxSpinCount(-1)
     times.sort()
     dev.sort()
-    return times[len(times) // 2], dev[len(dev) // 2]
+    return steady, times[len(times) // 2], dev[len(dev) // 2]
 
 
 def config_c3(L, full=False, separate=False):
@@ -374,23 +403,26 @@ def config_c3(L, full=False, separate=False):
     descs = c3_chunk_descs(L, nranks, shard, send, recv, rank)
     ms = timed_ms(lambda: L.reduce_batch(descs, L.RedOp.Avg, L.DataType.Float16, nranks))
     rows["C3_batch_32x4MiB"] = row(nb, ms, note="32 chunk descriptors, one batch call (needs every chunk present)")
+    frac_of = lambda t: round(nb / (t * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
     try:
-        ms, grid, small_ms = c3_queue_ms(L, nranks, descs)
-        rows["C3_queue_32x4MiB"] = row(nb, ms, note="chunk by chunk through the resident reduce queue, host wall clock "
-                                                    "first enqueue -> Wait; %d resident wavefronts" % grid,
-                                       one_4KiB_entry_enqueue_to_wait_ms=round(small_ms, 5),
-                                       frac_without_that_round_trip=round(
-                                           nb / ((ms - small_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4))
+        ms, single, grid, small_ms = c3_queue_ms(L, nranks, descs)
+        rows["C3_queue_32x4MiB"] = row(nb, ms, note="chunk by chunk through the resident reduce queue: 20 shards enqueued back "
+                                                    "to back, host wall clock to the return of Wait on the last ticket, per "
+                                                    "shard; %d resident wavefronts" % grid,
+                                       one_shard_enqueue_to_wait_ms=round(single, 5), one_shard_frac=frac_of(single),
+                                       one_4KiB_entry_enqueue_to_wait_ms=round(small_ms, 5))
     except Exception as e:   # a row of its own: the others are measured all the same
         rows["C3_queue_32x4MiB"] = {"error": repr(e)}
     try:
-        ms, dev_ms = c3_gated_ms(L, nranks, descs)
+        ms, single, dev_ms = c3_gated_ms(L, nranks, descs)
         rows["C3_gated_batch_32x4MiB"] = row(nb, ms, note="one batch launched up front, a host store per chunk lets its "
-                                                          "wavefronts go; host wall clock launch -> stream sync",
-                                             device_ms=round(dev_ms, 5),
-                                             device_frac=round(nb / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                                             device_note="between two events on the launch's stream, recorded before the "
-                                                         "launch call and behind it: without the host's wait for the stream")
+                                                          "wavefronts go: 20 shards launched and opened back to back, host wall "
+                                                          "clock to the end of one stream synchronisation, per shard",
+                                             one_shard_launch_to_sync_ms=round(single, 5), one_shard_frac=frac_of(single),
+                                             one_shard_device_ms=round(dev_ms, 5), one_shard_device_frac=frac_of(dev_ms),
+                                             device_note="device: between two events on the launch's stream, recorded before "
+                                                         "the launch call and behind the last Open; launch_to_sync also holds "
+                                                         "the host's wake-up from the synchronisation (about 10 us)")
     except Exception as e:
         rows["C3_gated_batch_32x4MiB"] = {"error": repr(e)}
     ms = timed_ms(lambda: L.reduce_scatter(send, rank, recv, L.RedOp.Avg, chunkbytes=L.CHUNKSIZE))

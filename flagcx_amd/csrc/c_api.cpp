@@ -534,7 +534,7 @@ struct GateWord {
 static std::mutex gGateWordsMutex;
 static std::map<int, std::vector<GateWord>> gGateWords;
 
-static GateWord takeUncachedWord(int device) {
+static GateWord takeUncachedWord(int device) try {
   std::lock_guard<std::mutex> lock(gGateWordsMutex);
   std::vector<GateWord> &pool = gGateWords[device];
   if (pool.empty()) {
@@ -549,10 +549,13 @@ static GateWord takeUncachedWord(int device) {
   const GateWord w = pool.back();
   pool.pop_back();
   return w;
+} catch (...) { // out of host memory: the gate then keeps its count in ordinary device memory
+  return GateWord{nullptr, 0};
 }
-static void returnUncachedWord(int device, GateWord w) {
+static void returnUncachedWord(int device, GateWord w) try {
   std::lock_guard<std::mutex> lock(gGateWordsMutex);
   gGateWords[device].push_back(w);
+} catch (...) { // the word is lost to later gates, nothing else
 }
 
 flagcxResult_t flagcxLocalGateCreate(flagcxLocalGate_t *gate) {

@@ -345,12 +345,53 @@ struct Exec {
   }
   flagcxResult_t needScratch() { return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", ""); }
 
+  // Copies wait here until something depends on them, and then go out together: the P2P ops of a
+  // hetero function run as one group in the reference (flagcxC2cHeteroFunc::run,
+  // c2c_algo.cc:554-568), and so do the sends of a homo function; on one GPU a group is one launch
+  // of the batch kernel with one input per segment (a sum of one input is a copy) instead of a
+  // launch per copy, which for chunk-sized copies runs at the rate of a large launch.
+  struct Pending {
+    char *dst;
+    const char *src;
+    size_t n;
+  };
+  std::vector<Pending> pending;
+  static bool hit(const char *a, size_t an, const char *b, size_t bn) { return a < b + bn && b < a + an; }
+
+  flagcxResult_t flushCopies() {
+    if (pending.empty()) return flagcxSuccess;
+    flagcxResult_t r;
+    if (pending.size() == 1) {
+      launches++;
+      r = flagcxLocalMemcpy(pending[0].dst, pending[0].src, pending[0].n, stream);
+    } else {
+      std::vector<const void *> src(pending.size());
+      std::vector<flagcxLocalReduceDesc> descs(pending.size());
+      for (size_t i = 0; i < pending.size(); i++) {
+        src[i] = pending[i].src;
+        descs[i] = {&src[i], pending[i].dst, pending[i].n};
+      }
+      launches += (pending.size() + 31) / 32;
+      r = flagcxLocalReduceBatch(descs.data(), (int)descs.size(), 1, flagcxUint8, flagcxSum, stream);
+    }
+    pending.clear();
+    return r;
+  }
   flagcxResult_t memcpyNow(char *dst, const char *src, size_t n) {
+    if (hit(dst, n, src, n)) return planFail(p, flagcxInvalidArgument, "a copy's buffers overlap%s", "");
+    // a copy that touches what a waiting copy writes, or writes what one reads, must follow it
+    for (auto &c : pending)
+      if (hit(dst, n, c.dst, c.n) || hit(dst, n, c.src, c.n) || hit(src, n, c.dst, c.n)) {
+        LCHECK(flushCopies());
+        break;
+      }
     bytes += 2 * n;
-    launches++;
-    return flagcxLocalMemcpy(dst, src, n, stream);
+    pending.push_back({dst, src, n});
+    if (pending.size() >= 64) return flushCopies();
+    return flagcxSuccess;
   }
   flagcxResult_t memsetNow(char *dst, size_t n) {
+    LCHECK(flushCopies());
     bytes += n;
     launches++;
     return flagcxLocalMemset(dst, 0, n, stream);
@@ -401,6 +442,7 @@ struct Exec {
       return flagcxSuccess;
     }
     if (fused) zeros.remove((uintptr_t)dst, (uintptr_t)dst + (size_t)m * n);
+    LCHECK(flushCopies());
     bytes += 2 * (uint64_t)m * n;
     launches++;
     return flagcxLocalPackList(dst, src.data(), m, n, stream);
@@ -419,6 +461,7 @@ struct Exec {
   }
 
   flagcxResult_t reduceNow(const std::vector<Red> &reds, int nzero) {
+    LCHECK(flushCopies());
     const int nlive = (int)reds[0].src.size();
     const flagcxRedOp_t rop = (flagcxRedOp_t)p->redOp;
     std::vector<flagcxLocalReduceDesc> descs(reds.size());
@@ -737,6 +780,7 @@ flagcxResult_t Exec::refresh(const std::vector<char> *only) {
     if (f.totalCount_ == 0) continue;
     if (!buff) return planFail(p, flagcxInvalidArgument, "refresh needs a scratch buffer%s", "");
     if (!fused) {
+      LCHECK(flushCopies());
       if (f.redOp_ == flagcxSum && f.count_ < f.totalCount_) {
         bytes += (f.totalCount_ - f.count_) * ts;
         launches++;
@@ -901,12 +945,12 @@ flagcxResult_t Exec::run() {
 // allocates for the call and frees when it ends (c2c_algo.cc:2122-2129,2292-2295): nobody
 // reads those again.
 flagcxResult_t Exec::finish() {
-  if (!fused) return flagcxSuccess;
+  if (!fused) return flushCopies();
   for (int r = 0; r < p->nranks; r++)
     if (ownsScratch[r] && scratch && scratch[r])
       zeros.remove((uintptr_t)scratch[r], (uintptr_t)scratch[r] + p->totalCount * ts);
   for (auto &z : zeros.ranges()) LCHECK(memsetNow((char *)z.first, z.second - z.first));
-  return flagcxSuccess;
+  return flushCopies();
 }
 
 } // namespace

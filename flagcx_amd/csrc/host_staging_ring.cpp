@@ -79,13 +79,19 @@ flagcxResult_t flagcxLocalRingCreate(flagcxLocalRing **ring, void *ringBuffer, s
   if (steps == 0) steps = FLAGCX_LOCAL_STEPS;
   if (steps < 1 || steps > 1024 || (chunkBytes & 15u)) return flagcxInvalidArgument;
   if (ringBytes < (size_t)steps * (size_t)npeers * chunkBytes) return flagcxInvalidArgument;
-  flagcxLocalRing *r = new flagcxLocalRing();
+  flagcxLocalRing *r = nullptr;
+  try { // nothing may leave an extern "C" function by exception
+    r = new flagcxLocalRing();
+    r->filled.resize(steps);
+    r->freed.resize(steps);
+  } catch (...) {
+    delete r;
+    return flagcxSystemError;
+  }
   r->buffer = static_cast<char *>(ringBuffer);
   r->chunkBytes = chunkBytes;
   r->steps = steps;
   r->npeers = npeers;
-  r->filled.resize(steps);
-  r->freed.resize(steps);
   bool ok = hipEventCreateWithFlags(&r->start, hipEventDisableTiming) == hipSuccess;
   for (int i = 0; ok && i < steps; i++) {
     ok = hipEventCreateWithFlags(&r->filled[i], hipEventDisableTiming) == hipSuccess &&
@@ -216,8 +222,8 @@ flagcxResult_t flagcxLocalRingReduceScatterFifo(flagcxLocalRing *r, flagcxLocalR
   const size_t size = recvcount * ts;
   const size_t nsteps = (size + r->chunkBytes - 1) / r->chunkBytes;
   const size_t depth = (size_t)r->steps;
-  std::vector<uint64_t> ticket(depth, 0); // per slot: ticket of the entry that reads it
-  std::vector<int> lead(depth, 0);        // per slot: the slot whose `filled` event covers its copy
+  uint64_t ticket[1024] = {0}; // per slot (a ring has at most 1024): ticket of the entry that reads it
+  int lead[1024] = {0};        // per slot: the slot whose `filled` event covers its copy
   const void *peerSrc[kGroup * FLAGCX_LOCAL_MAX_RANKS];
   const void *ordered[FLAGCX_LOCAL_MAX_RANKS];
   size_t copied = 0, handed = 0; // steps whose copy is issued / whose reduce is enqueued
