@@ -61,7 +61,7 @@ MiB = 1 << 20
 # (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a copy of
 # known size; not measured by this program.
 TRAFFIC_SOURCE = "profiles/reduce8_bf16_sum_256MiB_pmc.txt"
-TRAFFIC_BYTES = 2415742279
+TRAFFIC_BYTES = 2415742177
 
 
 def log(*a):

@@ -227,18 +227,32 @@ int main(int argc, char **argv) {
     CK(hipMemset(a, 1, 4096));
     CK(hipMemset(b, 2, 4096));
     const void *two[2] = {a, b};
-    double lib[4], empty[4], copy[4], minimal[4];
-    if (threeWays([&]() { (void)flagcxLocalReduce(two, 2, c, 1024, flagcxFloat, flagcxSum, &st); }, st.base, e0, e1, iters, lib)) return 1;
-    if (threeWays([&]() { emptyKernel<<<1, 64, 0, st.base>>>(); }, st.base, e0, e1, iters, empty)) return 1;
-    if (threeWays([&]() { minimalSumKernel<<<4, 64, 0, st.base>>>((const float4 *)a, (const float4 *)b, (float4 *)c); }, st.base,
-                  e0, e1, iters, minimal))
-      return 1;
-    if (threeWays([&]() { (void)hipMemcpyAsync(c, a, 4096, hipMemcpyDeviceToDevice, st.base); }, st.base, e0, e1, iters, copy)) return 1;
+    // the four are timed in turn, five rounds, and the median round of each is reported: the host's
+    // clock and caches drift over a run, and whoever goes first would carry that
+    const char *names[4] = {"library_reduce2_fp32", "empty_kernel_1x64", "minimal_sum_kernel_4x64", "hipMemcpyAsync_d2d"};
+    std::vector<double> res[4][4];
+    for (int round = 0; round < 5; round++) {
+      double t[4];
+      if (threeWays([&]() { (void)flagcxLocalReduce(two, 2, c, 1024, flagcxFloat, flagcxSum, &st); }, st.base, e0, e1, iters, t)) return 1;
+      for (int i = 0; i < 4; i++) res[0][i].push_back(t[i]);
+      if (threeWays([&]() { emptyKernel<<<1, 64, 0, st.base>>>(); }, st.base, e0, e1, iters, t)) return 1;
+      for (int i = 0; i < 4; i++) res[1][i].push_back(t[i]);
+      if (threeWays([&]() { minimalSumKernel<<<4, 64, 0, st.base>>>((const float4 *)a, (const float4 *)b, (float4 *)c); }, st.base,
+                    e0, e1, iters, t))
+        return 1;
+      for (int i = 0; i < 4; i++) res[2][i].push_back(t[i]);
+      if (threeWays([&]() { (void)hipMemcpyAsync(c, a, 4096, hipMemcpyDeviceToDevice, st.base); }, st.base, e0, e1, iters, t)) return 1;
+      for (int i = 0; i < 4; i++) res[3][i].push_back(t[i]);
+    }
     printf("# 4 KiB: us per call, back to back / one call between events / call -> stream synchronise / host time of the call\n");
-    printf("floor library_reduce2_fp32 %.3f %.3f %.3f %.3f\n", lib[0], lib[1], lib[2], lib[3]);
-    printf("floor empty_kernel_1x64 %.3f %.3f %.3f %.3f\n", empty[0], empty[1], empty[2], empty[3]);
-    printf("floor minimal_sum_kernel_4x64 %.3f %.3f %.3f %.3f\n", minimal[0], minimal[1], minimal[2], minimal[3]);
-    printf("floor hipMemcpyAsync_d2d %.3f %.3f %.3f %.3f\n", copy[0], copy[1], copy[2], copy[3]);
+    for (int k = 0; k < 4; k++) {
+      double m[4];
+      for (int i = 0; i < 4; i++) {
+        std::sort(res[k][i].begin(), res[k][i].end());
+        m[i] = res[k][i][res[k][i].size() / 2];
+      }
+      printf("floor %s %.3f %.3f %.3f %.3f\n", names[k], m[0], m[1], m[2], m[3]);
+    }
     return 0;
   }
   if (ceilingMode) {
