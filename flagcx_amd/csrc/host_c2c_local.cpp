@@ -344,6 +344,16 @@ struct Exec {
     return scratch ? (char *)scratch[rank] : nullptr;
   }
   flagcxResult_t needScratch() { return planFail(p, flagcxInvalidArgument, "plan needs a scratch buffer%s", ""); }
+  // [offset, offset + blocks * count) in elements lies inside the totalCount elements that the
+  // largest buffer of the collective holds
+  bool fits(size_t offset, size_t count, size_t blocks) const {
+    if (offset > p->totalCount) return false;
+    const size_t room = p->totalCount - offset;
+    return blocks == 0 || count <= room / blocks;
+  }
+  flagcxResult_t outside(int r) {
+    return planFail(p, flagcxInvalidArgument, "rank %s%lld: a function reaches past totalCount elements", "", r);
+  }
 
   // Copies wait here until something depends on them, and then go out together: the P2P ops of a
   // hetero function run as one group in the reference (flagcxC2cHeteroFunc::run,
@@ -563,6 +573,7 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
         const HomoFunc *f = fn[r];
         char *s = pick(r, f->sendType_), *d = pick(r, f->recvType_ == 1 ? 1 : 2);
         if (!s || !d) return needScratch();
+        if (!fits(f->sendOffset_, f->count_, 1) || !fits(f->recvOffset_, f->count_, 1)) return outside(r);
         s += f->sendOffset_ * ts;
         d += f->recvOffset_ * ts;
         if (op == kLocCpy) {
@@ -627,6 +638,22 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
     const size_t count = cnt[0];
     auto homoRootOf = [&](const HomoFunc *f) { return f->rootRank_ == -1 ? root : f->rootRank_; };
     auto badRoot = [&](int rt) { return planFail(p, flagcxInvalidArgument, "root %s%lld outside the communicator", "", rt); };
+    {
+      // every range a member reads or writes lies inside totalCount elements, the most any
+      // buffer of the collective holds (c2c_algo.cc:623,2124): blocks per member, and whether
+      // only the root's range is touched
+      const bool sBlocks = op == flagcxCommOpReduceScatter || op == flagcxCommOpScatter || op == flagcxCommOpAlltoAll;
+      const bool dBlocks = op == flagcxCommOpAllGather || op == flagcxCommOpGather || op == flagcxCommOpAlltoAll;
+      const bool sRootOnly = op == flagcxCommOpScatter || op == flagcxCommOpBroadcast;
+      const bool dRootOnly = op == flagcxCommOpReduce || op == flagcxCommOpGather;
+      const int rt = (sRootOnly || dRootOnly) ? homoRootOf(first) : -1;
+      if (op != flagcxCommNoOp)
+        for (int h = 0; h < n; h++) {
+          const HomoFunc *f = fn[comm[h]];
+          if (!(sRootOnly && h != rt) && !fits(f->sendOffset_, count, sBlocks ? (size_t)n : 1)) return outside(comm[h]);
+          if (!(dRootOnly && h != rt) && !fits(f->recvOffset_, count, dBlocks ? (size_t)n : 1)) return outside(comm[h]);
+        }
+    }
     const std::vector<const char *> members(S.begin(), S.end());
     switch (op) {
       case flagcxCommOpReduce: {
@@ -749,6 +776,8 @@ flagcxResult_t Exec::heteroSlot(int s, int i) {
       if (!recvTmp[peer] || !sendTmp[r])
         return planFail(p, flagcxInvalidArgument, "rank %s%lld stages its hetero functions in scratch and was given none", "",
                         recvTmp[peer] ? r : peer);
+      if (!fits(op.offset_, op.count_, 1)) return outside(r);
+      if (!fits(rv->offset_, rv->count_, 1)) return outside(peer);
       LCHECK(copy(recvTmp[peer] + rv->offset_ * ts, sendTmp[r] + op.offset_ * ts, op.count_ * ts));
     }
   }
@@ -779,6 +808,7 @@ flagcxResult_t Exec::refresh(const std::vector<char> *only) {
     void *buff = bt == 1 ? recv[r] : (scratch ? scratch[r] : nullptr);
     if (f.totalCount_ == 0) continue;
     if (!buff) return planFail(p, flagcxInvalidArgument, "refresh needs a scratch buffer%s", "");
+    if (f.redOp_ == flagcxSum && !fits(start, f.totalCount_, 1)) return outside(r);
     if (!fused) {
       LCHECK(flushCopies());
       if (f.redOp_ == flagcxSum && f.count_ < f.totalCount_) {
@@ -828,6 +858,8 @@ flagcxResult_t Exec::sendRecv(int cl, const std::vector<const HomoFunc *> &fn) {
         if (peer == r || !g || p->homoRank[peer] == rt) continue;
         char *dst = pick(peer, g->recvType_ == 1 ? 1 : 2);
         if (!dst) return needScratch();
+        if (!fits(f->sendOffset_, f->count_, 1)) return outside(r);
+        if (!fits(g->recvOffset_, f->count_, 1)) return outside(peer);
         LCHECK(copy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts));
       }
     } else if (f->homoType_ == 1) {
@@ -846,7 +878,10 @@ flagcxResult_t Exec::sendRecv(int cl, const std::vector<const HomoFunc *> &fn) {
             for (auto &q : pieces) seen = seen || (q.first == o.offset_ && q.second == o.count_);
             if (!seen) pieces.push_back({o.offset_, o.count_});
           }
-      for (auto &q : pieces) LCHECK(copy(dst + q.first * ts, src + q.first * ts, q.second * ts));
+      for (auto &q : pieces) {
+        if (!fits(q.first, q.second, 1)) return outside(r);
+        LCHECK(copy(dst + q.first * ts, src + q.first * ts, q.second * ts));
+      }
     } else if (f->homoType_ == 2) {
       if (p->homoInterRank[r] != 0 || p->homoRank[r] == rt) continue;
       const int peer = members[rt];
@@ -854,6 +889,8 @@ flagcxResult_t Exec::sendRecv(int cl, const std::vector<const HomoFunc *> &fn) {
       if (!g) continue;
       char *dst = pick(peer, g->recvType_ == 1 ? 1 : 2);
       if (!dst) return needScratch();
+      if (!fits(f->sendOffset_, f->count_, 1)) return outside(r);
+      if (!fits(g->recvOffset_, f->count_, 1)) return outside(peer);
       LCHECK(copy(dst + g->recvOffset_ * ts, src + f->sendOffset_ * ts, f->count_ * ts));
     }
   }

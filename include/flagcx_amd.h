@@ -682,7 +682,10 @@ flagcxResult_t flagcxLocalPlanGetTraffic(flagcxLocalPlan_t plan, uint64_t *bytes
  * refresh of buffType -1 go to scratchbuffs[rank], which must not be NULL; on every
  * other rank they go to recvbuffs[rank] (c2c_algo.cc:2131,2157-2158) and the scratch
  * pointer, which may be NULL, is only what functions that name scratch explicitly
- * (sendType / recvType / buffType 2) get.  Enqueues everything on `stream`. */
+ * (sendType / recvType / buffType 2) get.  No buffer is taken to hold more than
+ * totalCount elements (c2c_algo.cc:623,2124): a function or refresh that reaches past
+ * that returns flagcxInvalidArgument before it is launched (what was enqueued ahead of
+ * it still runs).  Enqueues everything on `stream`. */
 flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan_t plan, const void *const *sendbuffs,
                                       void *const *recvbuffs, void *const *scratchbuffs,
                                       flagcxDataType_t datatype, int root, flagcxStream_t stream);
