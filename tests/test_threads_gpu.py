@@ -207,3 +207,47 @@ def test_queue_gate_and_plain_launches_side_by_side():
         rc, want = O.reduce(ins, dt, op)
         assert rc == 0
         assert same(from_dev(out, ins[0].dtype), want, nan_class=dt != O.INT32, dtype=dt), (dt, op)
+
+
+@pytest.mark.gpu
+def test_two_gates_waiting_at_once_and_a_plain_launch_behind_them():
+    """Two gated batches wait on the GPU at the same time, each on its gate's own stream and each large
+    enough to fill its share of every CU's wavefront slots (8 chunks of 1024 tiles), and a plain launch is
+    enqueued on a third stream while both wait.  The host opens the gates chunk by chunk, the second gate
+    first; nothing the GPU holds can keep the host from doing so, so all three finish, with the oracle's
+    bytes.  The waits are bounded by the spin limit, as in every test of a waiting kernel."""
+    import ctypes as C
+    import torch
+    from flagcx_amd import local as L
+    assert L.lib().flagcxLocalInit() == 0
+    L.lib().flagcxLocalSetMaxSpinCount(1 << 22)
+    try:
+        n, chunks = 1 << 19, 8
+        ai, bi, pi = (make_inputs(dt, k, n * chunks, seed=s, op=op) for dt, k, s, op in
+                      ((O.FP16, 4, 11, O.AVG), (O.BF16, 8, 12, O.SUM), (O.INT32, 3, 13, O.MIN)))
+        ad, bd, pd = ([to_dev(a) for a in x] for x in (ai, bi, pi))
+        ao, bo, po = dev_empty(n * chunks, 2, fill=0), dev_empty(n * chunks, 2, fill=0), dev_empty(n * chunks, 4, fill=0)
+        plain = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        sync = L.adaptor_fn(L.device_adaptor()[1], "streamSynchronize", C.c_int, C.c_void_p)
+        with L.Gate() as ga, L.Gate() as gb:
+            sa, sb = ga.own_stream(), gb.own_stream()
+            fa = ga.reduce_batch([([d.data_ptr() + c * n * 2 for d in ad], ao.data_ptr() + c * n * 2, n)
+                                  for c in range(chunks)], O.AVG, O.FP16, 4, stream=sa)
+            fb = gb.reduce_batch([([d.data_ptr() + c * n * 2 for d in bd], bo.data_ptr() + c * n * 2, n)
+                                  for c in range(chunks)], O.SUM, O.BF16, 8, stream=sb)
+            L.reduce(pd, po, O.MIN, dtype=O.INT32, stream=L.Stream(plain.cuda_stream))
+            for c in range(chunks):
+                gb.open(fb + c + 1)
+                if c % 2:
+                    ga.open(fa + c + 1)            # the first gate two chunks at a time
+            assert sync(C.addressof(sb)) == 0 and sync(C.addressof(sa)) == 0
+            plain.synchronize()
+            assert ga.query()[2] == 0 and gb.query()[2] == 0
+        torch.cuda.synchronize()
+        for ins, out, dt, op in ((ai, ao, O.FP16, O.AVG), (bi, bo, O.BF16, O.SUM), (pi, po, O.INT32, O.MIN)):
+            rc, want = O.reduce(ins, dt, op)
+            assert rc == 0
+            assert same(from_dev(out, ins[0].dtype), want, nan_class=dt != O.INT32, dtype=dt), (dt, op)
+    finally:
+        L.lib().flagcxLocalSetMaxSpinCount(-1)
