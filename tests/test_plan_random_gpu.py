@@ -33,7 +33,7 @@ def disjoint(a, an, b, bn):
 def homo_for_cluster(rnd, m, allow_scratch):
     """One homo function per member of a cluster of m ranks (a list of m dicts), or None."""
     op = rnd.choice([PX.ALLREDUCE, PX.ALLREDUCE, PX.REDUCE, PX.REDUCESCATTER, PX.REDUCESCATTER, PX.BROADCAST, PX.ALLGATHER,
-                     NOP, PX.LOCRED, PX.LOCCPY])
+                     NOP, PX.LOCRED, PX.LOCCPY, PX.GATHER, PX.SCATTER, PX.ALLTOALL])
     st = rnd.choice([0, 1, 1, 2] if allow_scratch else [0, 1, 1])
     rt = rnd.choice([1, 1, 2] if allow_scratch else [1])
     root = rnd.randrange(m)
@@ -53,6 +53,24 @@ def homo_for_cluster(rnd, m, allow_scratch):
         return [PX.homo(op, st, rt, so, ro, cnt, 0, rootRank=root if op in (PX.REDUCE, PX.BROADCAST) else -1) for _ in range(m)]
     cnt = rnd.randint(1, NCH // m)
     big = rnd.randint(0, NCH - m * cnt)
+    if op == PX.ALLTOALL:                                  # S = m blocks, D = m blocks, never the same range
+        for _ in range(50):
+            ro = rnd.randint(0, NCH - m * cnt)
+            if st != rt or disjoint(big, m * cnt, ro, m * cnt):
+                return [PX.homo(op, st, rt, big, ro, cnt, 0) for _ in range(m)]
+        return None
+    if op == PX.SCATTER:                                   # the root's S = m blocks, D = one block
+        for _ in range(50):
+            ro = rnd.randint(0, NCH - cnt)
+            if st != rt or disjoint(big, m * cnt, ro, cnt):
+                return [PX.homo(op, st, rt, big, ro, cnt, 0, rootRank=root) for _ in range(m)]
+        return None
+    if op == PX.GATHER:                                    # S = one block, the root's D = m blocks
+        for _ in range(50):
+            so = rnd.randint(0, NCH - cnt)
+            if st != rt or disjoint(big, m * cnt, so, cnt):
+                return [PX.homo(op, st, rt, so, big, cnt, 0, rootRank=root) for _ in range(m)]
+        return None
     if op == PX.REDUCESCATTER:                             # S = m blocks, D = one block
         if st == rt and rnd.random() < 0.5:
             return [PX.homo(op, st, rt, big, big + h * cnt, cnt, 0) for h in range(m)]      # in place: own block
