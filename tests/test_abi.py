@@ -275,3 +275,16 @@ def test_build_refuses_a_kernel_with_a_scratch_segment():
                        "k.hip:20:1: remark:     ScratchSize [bytes/lane]: 48" + tag)
     with pytest.raises(RuntimeError, match="_Zspills uses 48 bytes of scratch"):
         B._no_spills("k.hip", ["-DFLAGCX_DT=0"], spilled)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The build runs on one GPU (the k ranks are k HBM buffers on it): bench.py says so and
+    exits instead of printing a figure for several, under a launcher that sets WORLD_SIZE too."""
+    import subprocess
+    import sys
+    bench = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")
+    for argv, env in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "2"})):
+        r = subprocess.run([sys.executable, bench] + argv, capture_output=True, text=True, timeout=120,
+                           env=dict(os.environ, **env))
+        assert r.returncode == 2, (argv, env, r.returncode)
+        assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
