@@ -624,6 +624,48 @@ def config_plan_replay(L, mib=128, iters=10, only=None, modes=(False, True)):
     return rows
 
 
+def plan_replay_small(L, sizes_kib=(64, 1024, 8192), iters=50):
+    """Small collectives are bound by the launches of a replay, not by bytes.  flagcxLocalPlanExecute
+    only launches kernels, so one Execute captured into a HIP graph stands for every later one with
+    the same buffers: microseconds per fused replay of the allreduce8 plan, eager and from a graph."""
+    import torch
+    plans = os.path.join(ROOT, "tests", "golden", "plans")
+    cl8 = [0, 0, 0, 0, 1, 1, 1, 1]
+    rows = {}
+    for kib in sizes_kib:
+        try:
+            n = kib * 1024 // 4
+            send = [torch.empty(n, dtype=torch.float32, device="cuda").uniform_(-1, 1) for _ in range(8)]
+            recv = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(8)]
+            plan = L.Plan(cl8, n, 6, L.RedOp.Sum)
+            plan.set_chunks(8)
+            plan.import_xml(os.path.join(plans, "allreduce8"))
+            plan.set_algorithm(2)
+            args = ([t.data_ptr() for t in send], [t.data_ptr() for t in recv], None, int(L.DataType.Float32))
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                eager_ms = timed_ms(lambda: plan.execute(*args), warmup=5, iters=iters)
+                want = [t.clone() for t in recv]
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side, capture_error_mode="global"):
+                    plan.execute(*args)
+                for t in recv:
+                    t.zero_()
+                graph_ms = timed_ms(g.replay, warmup=5, iters=iters)
+                same = all(torch.equal(a.view(torch.int32), b.view(torch.int32)) for a, b in zip(want, recv))
+            issued, launches = plan.traffic()
+            rows["plan_allreduce8_fused_%dKiB" % kib] = {
+                "bytes": int(issued), "launches": int(launches), "eager_us": round(eager_ms * 1e3, 2),
+                "graph_us": round(graph_ms * 1e3, 2), "graph_same_bytes_as_eager": bool(same),
+                "note": "8 ranks x %d KiB fp32, back-to-back replays between two HIP events" % kib}
+            plan.close()
+            del g
+        except Exception as e:
+            rows["plan_allreduce8_fused_%dKiB" % kib] = {"error": repr(e)}
+    return rows
+
+
 def perf_driver(*argv, timeout=180):
     """Lines of flagcx_amd/lib/local_perf (a C++ caller of the C ABI), or None with the reason logged."""
     import subprocess
@@ -787,6 +829,9 @@ def table_plan(L, args):
         extra = "  ".join("%s=%s" % (k, v) for k, v in r.items() if k not in ("bytes", "ms", "gbps", "frac", "note"))
         print("%-32s %14d B  %9.4f ms  %8.1f GB/s  %5.1f %%  %s" % (name, r["bytes"], r["ms"], r["gbps"],
                                                                       100 * r["frac"], extra), flush=True)
+    if args.plan_name in (None, "allreduce8") and args.plan_mode in ("fused", "both"):
+        for name, r in plan_replay_small(L).items():
+            print("%-32s %s" % (name, "  ".join("%s=%s" % kv for kv in r.items() if kv[0] != "note")), flush=True)
 
 
 def table_dtypes(L, args):

@@ -64,3 +64,54 @@ def test_chunked_reduce_scatter_pipeline_replays_from_a_graph():
         assert same(from_dev(mirror, np.uint16), want_rep, nan_class=True, dtype=dt), rep
         s = from_dev(scratch, np.uint16)
         assert not s[:n // 2].any() and not s[n // 2 + n:].any() and (s[n // 2:n // 2 + n] == 0x1234).all(), rep
+
+
+@pytest.mark.parametrize("name,commop,scratch", [("allreduce8", 6, False), ("reducescatter8", 8, True)])
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "literal"])
+def test_plan_replay_is_captured_once_and_replayed_on_new_inputs(name, commop, scratch, fused):
+    """flagcxLocalPlanExecute only launches kernels (a refresh is a fill kernel, copies are the
+    batch kernel), and the fused replay decides on the host, from the plan alone, which members a
+    sum reads: so one Execute captured into a HIP graph stands for every later one with the same
+    buffers.  Four replays on new inputs, the receive and scratch buffers refilled with junk in
+    between, each compared with the numpy model of flagcxC2cPlanner::execute."""
+    import torch
+    from flagcx_amd import local as L
+    from oracle import c2c_plan_model as M
+    from tests.test_plan_fixtures import CL8, fixture
+    assert L.lib().flagcxLocalInit() == 0
+    nr, n = 8, 8 * 3001
+    plan = L.Plan(CL8, n, commop, L.RedOp.Sum)
+    plan.set_chunks(8)
+    plan.import_xml(fixture(name))
+    plan.set_algorithm(2)
+    plan.set_fused(fused)
+    send = [torch.zeros(n, dtype=torch.int32, device="cuda") for _ in range(nr)]
+    recv = [torch.zeros(n, dtype=torch.int32, device="cuda") for _ in range(nr)]
+    scr = [torch.zeros(n, dtype=torch.int32, device="cuda") for _ in range(nr)] if scratch else None
+    ptrs = ([s.data_ptr() for s in send], [r.data_ptr() for r in recv], [s.data_ptr() for s in scr] if scr else None)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        plan.execute(*ptrs, O.INT32)                # eager warm-up on the capture stream
+    side.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side, capture_error_mode="global"):
+        plan.execute(*ptrs, O.INT32)
+    model = M.Model(fixture(name), CL8, n, commop, 0, default_chunks=8)
+    for rep in range(4):
+        rng = np.random.default_rng(500 + rep)
+        hosts = [rng.integers(-2**27, 2**27, n, dtype=np.int32) for _ in range(nr)]
+        for r in range(nr):
+            send[r].copy_(to_dev(hosts[r]))
+            recv[r].fill_(0x55550000 + rep)
+            if scr:
+                scr[r].fill_(0x33330000 + rep)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        mrecv = [np.full(n, 0x55550000 + rep, dtype=np.int32) for _ in range(nr)]
+        mscr = [np.full(n, 0x33330000 + rep, dtype=np.int32) for _ in range(nr)] if scratch else None
+        model.execute([h.copy() for h in hosts], mrecv, mscr, algorithm=2)
+        for r in range(nr):
+            assert same(from_dev(recv[r], np.int32), mrecv[r]), (rep, r)
+            assert same(from_dev(send[r], np.int32), hosts[r]), (rep, r)
