@@ -829,7 +829,7 @@ def table_plan(L, args):
         extra = "  ".join("%s=%s" % (k, v) for k, v in r.items() if k not in ("bytes", "ms", "gbps", "frac", "note"))
         print("%-32s %14d B  %9.4f ms  %8.1f GB/s  %5.1f %%  %s" % (name, r["bytes"], r["ms"], r["gbps"],
                                                                       100 * r["frac"], extra), flush=True)
-    if args.plan_name in (None, "allreduce8") and args.plan_mode in ("fused", "both"):
+    if args.plan_name in (None, "allreduce8") and args.plan_mode == "both":   # one-mode runs are the profiled ones
         for name, r in plan_replay_small(L).items():
             print("%-32s %s" % (name, "  ".join("%s=%s" % kv for kv in r.items() if kv[0] != "note")), flush=True)
 

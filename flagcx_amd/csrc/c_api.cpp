@@ -1002,6 +1002,82 @@ flagcxResult_t flagcxLocalUnpackList(void *const *dsts, const void *src, int n, 
   return copy2d(c, stream, who);
 }
 
+// One source to several destinations, several such copies at once.  Destinations that agree
+// with their source modulo 16 bytes share one read of it (up to kFanMaxDst per read); the
+// others are plain copies.  Everything is checked before the first launch.
+flagcxResult_t flagcxLocalCopyFanout(const flagcxLocalFanoutDesc *descs, int ndescs, flagcxStream_t stream) {
+  const char *who = "flagcxLocalCopyFanout";
+  if (ndescs < 0) return fail(flagcxInvalidArgument, "%s: ndescs %d is negative", who, ndescs);
+  if (ndescs == 0) return flagcxSuccess;
+  if (!descs) return fail(flagcxInvalidArgument, "%s: descs is NULL", who);
+  if (ndescs > FLAGCX_LOCAL_FANOUT_MAX)
+    return fail(flagcxInvalidArgument, "%s: %d copies, at most %d at once", who, ndescs, FLAGCX_LOCAL_FANOUT_MAX);
+  // every byte range of the call: the copies run concurrently, so nothing may be written
+  // that another copy reads or writes
+  struct Range {
+    uintptr_t b, e;
+    int desc;
+    bool write;
+  };
+  Range ranges[FLAGCX_LOCAL_FANOUT_MAX_DSTS + FLAGCX_LOCAL_FANOUT_MAX];
+  int nranges = 0, ndsts = 0;
+  for (int i = 0; i < ndescs; i++) {
+    const flagcxLocalFanoutDesc &d = descs[i];
+    if (d.ndsts < 0) return fail(flagcxInvalidArgument, "%s: descs[%d].ndsts %d is negative", who, i, d.ndsts);
+    if (d.bytes == 0 || d.ndsts == 0) continue;
+    if (!d.src || !d.dsts) return fail(flagcxInvalidArgument, "%s: descs[%d]: NULL pointer", who, i);
+    if (d.ndsts > FLAGCX_LOCAL_FANOUT_MAX_DSTS - ndsts)
+      return fail(flagcxInvalidArgument, "%s: more than %d destinations in one call", who, FLAGCX_LOCAL_FANOUT_MAX_DSTS);
+    ndsts += d.ndsts;
+    ranges[nranges++] = {(uintptr_t)d.src, (uintptr_t)d.src + d.bytes, i, false};
+    for (int j = 0; j < d.ndsts; j++) {
+      if (!d.dsts[j]) return fail(flagcxInvalidArgument, "%s: descs[%d].dsts[%d] is NULL", who, i, j);
+      if (d.dsts[j] == d.src) continue; // a copy onto itself is nothing (the root of a broadcast in place)
+      ranges[nranges++] = {(uintptr_t)d.dsts[j], (uintptr_t)d.dsts[j] + d.bytes, i, true};
+    }
+  }
+  for (int x = 0; x < nranges; x++)
+    for (int y = 0; y < x; y++)
+      if ((ranges[x].write || ranges[y].write) && ranges[x].b < ranges[y].e && ranges[y].b < ranges[x].e)
+        return fail(flagcxInvalidArgument, "%s: a destination of descs[%d] overlaps a buffer of descs[%d]", who,
+                    ranges[x].write ? ranges[x].desc : ranges[y].desc, ranges[x].write ? ranges[y].desc : ranges[x].desc);
+  bool work = false;
+  for (int x = 0; x < nranges; x++) work = work || ranges[x].write;
+  if (!work) return flagcxSuccess;
+  (void)deviceInfo();
+  hipStream_t hs = hipStreamOf(stream);
+  FanoutCall calls[kFanMaxSeg];
+  int ncalls = 0;
+  int err = 0;
+  for (int i = 0; i < ndescs && !err; i++) {
+    const flagcxLocalFanoutDesc &d = descs[i];
+    if (d.bytes == 0 || d.ndsts == 0) continue;
+    FanoutCall *cur = nullptr;
+    for (int j = 0; j < d.ndsts && !err; j++) {
+      if (d.dsts[j] == d.src) continue;
+      if ((((uintptr_t)d.dsts[j] ^ (uintptr_t)d.src) & 15u) != 0) {
+        Copy2D c{d.dsts[j], d.src, 1, d.bytes, d.bytes, d.bytes, nullptr, nullptr, hs};
+        err = launchCopy2D(c);
+        continue;
+      }
+      if (!cur || cur->ndst == kFanMaxDst) {
+        if (ncalls == kFanMaxSeg) {
+          err = launchFanout(calls, ncalls, hs);
+          ncalls = 0;
+          if (err) break;
+        }
+        cur = &calls[ncalls++];
+        cur->src = d.src;
+        cur->ndst = 0;
+        cur->bytes = d.bytes;
+      }
+      cur->dst[cur->ndst++] = d.dsts[j];
+    }
+  }
+  if (!err && ncalls) err = launchFanout(calls, ncalls, hs);
+  return finish(stream, err, who);
+}
+
 // ---------------------------------------------------- launcher convention
 
 void flagcxLocalReduceFunc(flagcxStream_t stream, void *args) {

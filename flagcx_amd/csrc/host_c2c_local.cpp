@@ -375,14 +375,48 @@ struct Exec {
       launches++;
       r = flagcxLocalMemcpy(pending[0].dst, pending[0].src, pending[0].n, stream);
     } else {
-      std::vector<const void *> src(pending.size());
-      std::vector<flagcxLocalReduceDesc> descs(pending.size());
-      for (size_t i = 0; i < pending.size(); i++) {
-        src[i] = pending[i].src;
-        descs[i] = {&src[i], pending[i].dst, pending[i].n};
+      // copies of one source and one length (the sends of a broadcast, a member's block in an
+      // all-gather) share one read of it: flagcxLocalCopyFanout; the rest go as one batch
+      const size_t np = pending.size();
+      std::vector<int> groupOf(np, -1);
+      std::vector<std::vector<void *>> dsts;
+      std::vector<size_t> first;
+      for (size_t i = 0; i < np; i++) {
+        for (size_t g = 0; g < first.size() && groupOf[i] < 0; g++)
+          if (pending[first[g]].src == pending[i].src && pending[first[g]].n == pending[i].n) groupOf[i] = (int)g;
+        if (groupOf[i] < 0) {
+          groupOf[i] = (int)first.size();
+          first.push_back(i);
+          dsts.emplace_back();
+        }
+        dsts[groupOf[i]].push_back(pending[i].dst);
       }
-      launches += (pending.size() + 31) / 32;
-      r = flagcxLocalReduceBatch(descs.data(), (int)descs.size(), 1, flagcxUint8, flagcxSum, stream);
+      std::vector<flagcxLocalFanoutDesc> fans;
+      std::vector<const void *> src;
+      std::vector<flagcxLocalReduceDesc> descs;
+      src.reserve(np);
+      for (size_t g = 0; g < first.size(); g++) {
+        const Pending &c = pending[first[g]];
+        if (dsts[g].size() >= 2) {
+          fans.push_back({c.src, dsts[g].data(), (int)dsts[g].size(), c.n});
+          bytes -= (uint64_t)(dsts[g].size() - 1) * c.n; // the source is read once
+        } else {
+          src.push_back(c.src);
+          descs.push_back({&src.back(), c.dst, c.n});
+        }
+      }
+      r = flagcxSuccess;
+      if (!fans.empty()) {
+        launches += (fans.size() + 15) / 16;
+        r = flagcxLocalCopyFanout(fans.data(), (int)fans.size(), stream);
+      }
+      if (r == flagcxSuccess && descs.size() == 1) {
+        launches++;
+        r = flagcxLocalMemcpy(descs[0].recvbuff, src[0], descs[0].count, stream);
+      } else if (r == flagcxSuccess && !descs.empty()) {
+        launches += (descs.size() + 31) / 32;
+        r = flagcxLocalReduceBatch(descs.data(), (int)descs.size(), 1, flagcxUint8, flagcxSum, stream);
+      }
     }
     pending.clear();
     return r;

@@ -138,6 +138,17 @@ struct Copy2D {
 };
 int launchCopy2D(const Copy2D &c);
 int launchFill(void *p0, uint64_t n0, void *p1, uint64_t n1, int value, hipStream_t stream);
+// One source copied to several destinations, up to kFanMaxSeg such copies in one launch: the
+// source is read once.  Every destination agrees with its source modulo 16 bytes.
+constexpr int kFanMaxDst = 8;
+constexpr int kFanMaxSeg = 16;
+struct FanoutCall {
+  const void *src;
+  void *dst[kFanMaxDst];
+  int ndst;
+  uint64_t bytes;
+};
+int launchFanout(const FanoutCall *calls, int n, hipStream_t stream);
 
 // Text that flagcxLocalGetLastError returns to the calling thread (c_api.cpp).
 void setLastError(const char *text);

@@ -71,6 +71,10 @@ class ReduceDesc(C.Structure):       # flagcxLocalReduceDesc
     _fields_ = [("sendbuffs", C.POINTER(C.c_void_p)), ("recvbuff", C.c_void_p), ("count", C.c_size_t)]
 
 
+class FanoutDesc(C.Structure):       # flagcxLocalFanoutDesc
+    _fields_ = [("src", C.c_void_p), ("dsts", C.POINTER(C.c_void_p)), ("ndsts", C.c_int), ("bytes", C.c_size_t)]
+
+
 class ReduceTrigger(C.Structure):    # flagcxLocalReduceTrigger, 16-byte aligned
     _fields_ = [("value", C.c_uint64 * 4)]
     _pack_ = 16
@@ -118,7 +122,7 @@ EXPORTS = [
     "flagcxLocalTune", "flagcxLocalGetTune", "flagcxLocalTuneLoads", "flagcxLocalGetTuneLoads", "flagcxLocalPlaceBuffers", "flagcxLocalReduce", "flagcxLocalReduceScatter", "flagcxLocalReduceScatterChunked",
     "flagcxLocalAllReduce", "flagcxLocalRingChunkTable", "flagcxLocalMemcpy", "flagcxLocalMemset",
     "flagcxLocalRefresh", "flagcxLocalPack", "flagcxLocalUnpack", "flagcxLocalPackList",
-    "flagcxLocalUnpackList", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
+    "flagcxLocalUnpackList", "flagcxLocalCopyFanout", "flagcxLocalReduceFunc", "flagcxLocalCopyFunc",
     "flagcxLocalSetMaxSpinCount", "deviceAsyncStore", "deviceAsyncLoad",
     "flagcxLocalReduceBatch", "flagcxLocalReduceBatchSparse", "flagcxLocalReduceTriggers",
     "flagcxLocalGateCreate", "flagcxLocalGateDestroy", "flagcxLocalReduceBatchGated", "flagcxLocalGateOpen",
@@ -183,6 +187,7 @@ def lib():
         L.flagcxLocalUnpack.argtypes = [vp, vp, sz, sz, sz, sp]
         L.flagcxLocalPackList.argtypes = [vp, pp, i, sz, sp]
         L.flagcxLocalUnpackList.argtypes = [pp, vp, i, sz, sp]
+        L.flagcxLocalCopyFanout.argtypes = [C.POINTER(FanoutDesc), i, sp]
         L.flagcxLocalReduceFunc.restype = None
         L.flagcxLocalReduceFunc.argtypes = [sp, C.POINTER(ReduceArgs)]
         L.flagcxLocalCopyFunc.restype = None
@@ -405,6 +410,14 @@ def pack_list(dst_ptr, src_ptrs, nbytes, stream="current"):
 def unpack_list(dst_ptrs, src_ptr, nbytes, stream="current"):
     st = current_stream() if stream == "current" else stream
     check(lib().flagcxLocalUnpackList(_ptr_array(dst_ptrs), src_ptr, len(dst_ptrs), nbytes, _sref(st)))
+
+
+def copy_fanout(copies, stream="current"):
+    """copies: list of (src_ptr, list_of_dst_ptrs, nbytes).  One flagcxLocalCopyFanout call."""
+    st = current_stream() if stream == "current" else stream
+    keep = [_ptr_array(list(c[1])) for c in copies]
+    arr = (FanoutDesc * len(copies))(*[FanoutDesc(c[0], keep[i], len(c[1]), c[2]) for i, c in enumerate(copies)])
+    check(lib().flagcxLocalCopyFanout(arr, len(copies), _sref(st)))
 
 
 class Plan:

@@ -409,6 +409,27 @@ flagcxResult_t flagcxLocalPackList(void *dst, const void *const *srcs, int n,
 flagcxResult_t flagcxLocalUnpackList(void *const *dsts, const void *src, int n,
                                      size_t bytes, flagcxStream_t stream);
 
+/* One source copied to several destinations, and several such copies in one call: what a
+ * broadcast (flagcxC2cHomoFunc::run, flagcx/core/c2c_algo.cc:464-472 ->
+ * flagcx/adaptor/ccl/rccl_adaptor.cc:161-168) or an all-gather (c2c_algo.cc:337-345 ->
+ * rccl_adaptor.cc:188-195) moves when the ranks of a cluster are buffers on one GPU.
+ * Destinations that agree with their source modulo 16 bytes share one read of it: the
+ * launch moves (1 + ndsts) * bytes instead of 2 * ndsts * bytes; the others are plain
+ * copies.  A destination equal to its source is skipped (the root of an in-place
+ * broadcast).  The copies of one call run concurrently: a destination that overlaps any
+ * other buffer of the call -> flagcxInvalidArgument, before anything is launched.
+ * dsts is a host array. */
+#define FLAGCX_LOCAL_FANOUT_MAX 64       /* copies per call */
+#define FLAGCX_LOCAL_FANOUT_MAX_DSTS 256 /* destinations per call, all copies together */
+typedef struct {
+  const void *src;
+  void *const *dsts;
+  int ndsts;
+  size_t bytes;
+} flagcxLocalFanoutDesc;
+flagcxResult_t flagcxLocalCopyFanout(const flagcxLocalFanoutDesc *descs, int ndescs,
+                                     flagcxStream_t stream);
+
 /* ------------------------------------------------------------------------- */
 /* Device-producer / host-consumer trigger FIFO                                */
 /* ------------------------------------------------------------------------- */

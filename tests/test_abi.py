@@ -277,6 +277,36 @@ def test_build_refuses_a_kernel_with_a_scratch_segment():
         B._no_spills("k.hip", ["-DFLAGCX_DT=0"], spilled)
 
 
+def test_copy_fanout_validates_without_a_device():
+    """Every check of flagcxLocalCopyFanout comes before its first launch: counts, NULL pointers,
+    and any destination that overlaps another buffer of the call (its own source, a sibling,
+    a buffer of another copy), since the copies of one call run concurrently."""
+    lib = local.lib()
+    base = 0x7f0000000000                     # never dereferenced: every call below is refused
+
+    def call(copies):
+        keep = [(C.c_void_p * max(1, len(c[1])))(*c[1]) for c in copies]
+        arr = (local.FanoutDesc * max(1, len(copies)))(*[local.FanoutDesc(c[0], keep[i], c[3] if len(c) > 3 else len(c[1]), c[2])
+                                                          for i, c in enumerate(copies)])
+        return lib.flagcxLocalCopyFanout(arr, len(copies), None)
+
+    bad = int(local.Result.InvalidArgument)
+    assert lib.flagcxLocalCopyFanout(None, 0, None) == 0
+    assert lib.flagcxLocalCopyFanout(None, 1, None) == bad
+    assert lib.flagcxLocalCopyFanout(None, -1, None) == bad
+    assert call([(base, [base + 4096], 100, -1)]) == bad                                  # negative ndsts
+    assert call([(None, [base + 4096], 100)]) == bad                                      # NULL source
+    assert call([(base, [None], 100)]) == bad                                             # NULL destination
+    assert call([(base, [base + 50], 100)]) == bad                                        # destination overlaps its source
+    assert call([(base, [base + 4096, base + 4096 + 99], 100)]) == bad                    # two destinations overlap
+    assert call([(base, [base + 4096], 100), (base + 8192, [base + 4096 + 10], 100)]) == bad   # across copies
+    assert call([(base, [base + 4096], 100), (base + 4096 + 64, [base + 8192], 100)]) == bad   # written here, read there
+    assert b"overlaps" in lib.flagcxLocalGetLastError()
+    assert call([(base + 65536 * i, [base + 65536 * i + 4096], 16) for i in range(65)]) == bad  # more than 64 copies
+    assert call([(base, [base + 4096 * (j + 1) for j in range(64)], 16)] * 5) == bad           # more than 256 destinations
+    assert call([(base, [base + 4096], 0), (base, [], 100)]) == 0                         # nothing to do
+
+
 def test_bench_refuses_more_than_one_gpu():
     """The build runs on one GPU (the k ranks are k HBM buffers on it): bench.py says so and
     exits instead of printing a figure for several, under a launcher that sets WORLD_SIZE too."""

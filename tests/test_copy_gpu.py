@@ -188,6 +188,78 @@ def test_pack_list_and_unpack_list(L, nbytes):
             assert (g[:off] == 0x22).all() and (g[off + nbytes:] == 0x22).all()
 
 
+@pytest.mark.parametrize("size", [1, 15, 16, 17, 1000, 4096, 65536 + 5, (3 << 20) + 77])
+def test_copy_fanout_sizes_offsets_and_destination_counts(L, size):
+    """One source to 1..11 destinations (more than eight share the source in two reads), at
+    offsets that agree with the source modulo 16 (inside and on 128-byte lines) and at
+    offsets that do not (those go as plain copies); bytes and guard bytes of every
+    destination against numpy."""
+    import torch
+    rng = np.random.default_rng(size)
+    src_h = rand_bytes(size + 256, size)
+    src = to_dev(src_h)
+    for so, ndst in ((0, 1), (0, 4), (3, 3), (16, 8), (5, 11), (64, 2), (130, 5)):
+        dos = [so + 16 * int(rng.integers(0, 8)) if j % 3 != 2 else int(rng.integers(0, 200)) for j in range(ndst)]
+        dsts = [torch.full((size + 512,), 0xAB, dtype=torch.uint8, device="cuda") for _ in range(ndst)]
+        L.copy_fanout([(src.data_ptr() + so, [d.data_ptr() + o for d, o in zip(dsts, dos)], size)])
+        torch.cuda.synchronize()
+        for j in range(ndst):
+            got = from_dev(dsts[j], np.uint8)
+            assert same(got[dos[j]:dos[j] + size], src_h[so:so + size]), (so, ndst, j, dos[j])
+            assert (got[:dos[j]] == 0xAB).all() and (got[dos[j] + size:] == 0xAB).all(), (so, ndst, j, dos[j])
+
+
+def test_copy_fanout_several_sources_in_one_call(L):
+    """The copies of an all-gather inside a cluster of four: every member's block goes to all
+    four receive buffers, the member's own included; 4 sources x 4 destinations in one call,
+    then 20 sources x 3 (more than one launch's worth).  A destination equal to its source is
+    skipped; empty copies are nothing."""
+    import torch
+    m, blk = 4, 70001
+    hs = [rand_bytes(blk, 900 + r) for r in range(m)]
+    recv = [torch.full((m * blk + 32,), 0x5A, dtype=torch.uint8, device="cuda") for _ in range(m)]
+    for r in range(m):                                          # in place: member r's block already sits at r * blk
+        recv[r][r * blk:(r + 1) * blk] = to_dev(hs[r])
+    torch.cuda.synchronize()
+    L.copy_fanout([(recv[r].data_ptr() + r * blk, [recv[h].data_ptr() + r * blk for h in range(m)], blk) for r in range(m)]
+                  + [(recv[0].data_ptr(), [], blk), (recv[0].data_ptr(), [recv[1].data_ptr()], 0)])
+    torch.cuda.synchronize()
+    want = np.concatenate(hs)
+    for h in range(m):
+        got = from_dev(recv[h], np.uint8)
+        assert same(got[:m * blk], want), h
+        assert (got[m * blk:] == 0x5A).all(), h
+    ns, nd, size = 20, 3, 5000
+    srcs_h = [rand_bytes(size, 1000 + i) for i in range(ns)]
+    srcs = [to_dev(h) for h in srcs_h]
+    outs = [[torch.full((size + 16,), 0x77, dtype=torch.uint8, device="cuda") for _ in range(nd)] for _ in range(ns)]
+    L.copy_fanout([(srcs[i].data_ptr(), [o.data_ptr() for o in outs[i]], size) for i in range(ns)])
+    torch.cuda.synchronize()
+    for i in range(ns):
+        for o in outs[i]:
+            got = from_dev(o, np.uint8)
+            assert same(got[:size], srcs_h[i]) and (got[size:] == 0x77).all(), i
+
+
+def test_copy_fanout_beyond_4GiB_offsets(L):
+    """A block that straddles the 4 GiB mark of its buffers (descriptors are per tile, offsets 64-bit)."""
+    import torch
+    big = (1 << 32) + (1 << 20)
+    src = torch.empty(big, dtype=torch.uint8, device="cuda")
+    dsts = [torch.empty(big, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    at, n = (1 << 32) - 300_000, 600_000
+    h = rand_bytes(n, 4)
+    src[at:at + n] = to_dev(h)
+    for d in dsts:
+        d[at - 16:at + n + 16] = 0x3C
+    torch.cuda.synchronize()
+    L.copy_fanout([(src.data_ptr() + at, [d.data_ptr() + at for d in dsts], n)])
+    torch.cuda.synchronize()
+    for d in dsts:
+        got = from_dev(d[at - 16:at + n + 16], np.uint8)
+        assert same(got[16:16 + n], h) and (got[:16] == 0x3C).all() and (got[16 + n:] == 0x3C).all()
+
+
 def test_device_async_store_and_bounded_load(L):
     """deviceAsyncStore sets the flag, deviceAsyncLoad returns once it is set; with
     the flag never set the load gives up after its spin bound and exits normally."""
