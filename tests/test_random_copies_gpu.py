@@ -91,3 +91,35 @@ def test_random_copies_match_numpy(L, large):
                     torch.cuda.synchronize()
                     for i, d in enumerate(dsts):
                         check(d.cpu().numpy(), chunks[i * cb:(i + 1) * cb], offs[i], cb, (kind, offs, so, nch, cb, i))
+
+
+@pytest.mark.parametrize("large", [False, True], ids=["small", "large"])
+def test_random_fanout_copies_match_numpy(L, large):
+    """flagcxLocalCopyFanout: 1..5 copies per call, each one source to 1..12 destinations, random sizes and
+    random positions inside the cache lines (mostly at the source's offset modulo 16, which shares one read
+    of the source; the rest go as plain copies), now and then a destination that is the source itself."""
+    import torch
+    rnd = random.Random(41 if large else 42)
+    g = np.random.default_rng(6)
+    for case in range(10 if large else 120):
+        copies, keep = [], []
+        for _ in range(rnd.randint(1, 5)):
+            n = size_of(rnd, large)
+            so = rnd.randrange(0, 128)
+            h = g.integers(0, 256, n + 256, dtype=np.uint8)
+            src = torch.from_numpy(h).cuda()
+            outs = []
+            for j in range(rnd.randint(1, 12)):
+                do = (so % 16) + 16 * rnd.randrange(0, 8) if rnd.random() < 0.8 else rnd.randrange(0, 128)
+                outs.append((torch.full((n + 384,), 0x5A, dtype=torch.uint8, device="cuda"), do))
+            ptrs = [o.data_ptr() + do for o, do in outs]
+            if rnd.random() < 0.2:
+                ptrs.insert(rnd.randrange(0, len(ptrs) + 1), src.data_ptr() + so)      # in place: skipped
+            copies.append((src.data_ptr() + so, ptrs, n))
+            keep.append((h, so, n, outs, src))
+        L.copy_fanout(copies)
+        torch.cuda.synchronize()
+        for h, so, n, outs, src in keep:
+            assert np.array_equal(src.cpu().numpy(), h), (case, "source changed")
+            for o, do in outs:
+                check(o.cpu().numpy(), h[so:so + n], do, n, (case, so, do, n, len(outs)))
