@@ -525,6 +525,14 @@ struct Exec {
   // a -0.0 result into +0.0 and change nothing else).
   flagcxResult_t reduce(const std::vector<Red> &reds) {
     if (reds.empty()) return flagcxSuccess;
+    for (auto &r : reds)
+      if (r.src.size() != reds[0].src.size()) {
+        // clusters of different sizes in one slot: one call per member count
+        std::map<size_t, std::vector<Red>> byCount;
+        for (auto &q : reds) byCount[q.src.size()].push_back(q);
+        for (auto &g : byCount) LCHECK(reduce(g.second));
+        return flagcxSuccess;
+      }
     bool plain = !fused || zeros.empty();
     if (!plain) {
       plain = true;
@@ -572,6 +580,23 @@ struct Exec {
     return flagcxSuccess;
   }
 
+  // No reduction of one group writes what a reduction of another group reads or writes (the
+  // groups are collectives of different clusters, or folds local to different ranks).
+  bool independent(const std::vector<std::vector<Red>> &groups) const {
+    for (size_t a = 0; a < groups.size(); a++)
+      for (size_t b = 0; b < groups.size(); b++) {
+        if (a == b) continue;
+        for (auto &w : groups[a])
+          for (auto &r : groups[b]) {
+            const size_t wn = w.count * ts, rn = r.count * ts;
+            if (hit(w.dst, wn, r.dst, rn)) return false;
+            for (auto s : r.src)
+              if (hit(w.dst, wn, s, rn)) return false;
+          }
+      }
+    return true;
+  }
+
   flagcxResult_t refresh(const std::vector<char> *only);
   flagcxResult_t homoSlot(const std::vector<const HomoFunc *> &fn);
   flagcxResult_t sendRecv(int cl, const std::vector<const HomoFunc *> &fn);
@@ -588,6 +613,16 @@ struct Exec {
 flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
   const int ncl = (int)p->clusterRanks.size();
   const int root = homoRoot;
+  // The clusters run a slot side by side, each on its own ranks' buffers: their reductions go
+  // out together (one batch launch per member count instead of one per cluster), and the copies
+  // that hand an all-reduce's result to the other members follow them.
+  std::vector<std::vector<Red>> groups; // one per collective (or per rank-local fold)
+  struct After {
+    char *dst;
+    const char *src;
+    size_t n;
+  };
+  std::vector<After> after;
   for (int cl = 0; cl < ncl; cl++) {
     // members that hold a function in this slot; homoType 1 runs on inter-ranks only
     std::vector<int> mem;
@@ -613,7 +648,7 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
         if (op == kLocCpy) {
           LCHECK(copy(d, s, f->count_ * ts));
         } else {
-          LCHECK(reduce({Red{d, {d, s}, f->count_}})); // acc = recv slice; acc = OP(send slice, acc)
+          groups.push_back({Red{d, {d, s}, f->count_}}); // acc = recv slice; acc = OP(send slice, acc)
         }
       }
       continue;
@@ -693,13 +728,13 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
       case flagcxCommOpReduce: {
         const int rt = homoRootOf(first);
         if (rt < 0 || rt >= n) return badRoot(rt);
-        LCHECK(reduce({Red{D[rt], members, count}}));
+        groups.push_back({Red{D[rt], members, count}});
         break;
       }
       case flagcxCommOpAllReduce: {
         // every member ends with the same bytes: reduce once, then copy
-        LCHECK(reduce({Red{D[0], members, count}}));
-        for (int h = 1; h < n; h++) LCHECK(copy(D[h], D[0], count * ts));
+        groups.push_back({Red{D[0], members, count}});
+        for (int h = 1; h < n; h++) after.push_back({D[h], D[0], count * ts});
         break;
       }
       case flagcxCommOpReduceScatter: {
@@ -710,7 +745,7 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
           reds[h].count = count;
           for (int j = 0; j < n; j++) reds[h].src.push_back(S[j] + (size_t)h * count * ts);
         }
-        LCHECK(reduce(reds));
+        groups.push_back(std::move(reds));
         break;
       }
       case flagcxCommOpAllGather: {
@@ -750,6 +785,15 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
         return planFail(p, flagcxNotSupported, "homo function commOp %s%lld is not replayed", "", op);
     }
   }
+  if (groups.size() > 1 && independent(groups)) {
+    std::vector<Red> all;
+    for (auto &g : groups)
+      for (auto &r : g) all.push_back(std::move(r));
+    LCHECK(reduce(all));
+  } else {
+    for (auto &g : groups) LCHECK(reduce(g));
+  }
+  for (auto &c : after) LCHECK(copy(c.dst, c.src, c.n));
   return flagcxSuccess;
 }
 
