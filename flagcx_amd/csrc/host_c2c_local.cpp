@@ -468,28 +468,13 @@ struct Exec {
     return flagcxSuccess;
   }
 
-  // n blocks of `n` bytes from the pointers in `src` into dst, back to back: one launch
-  // unless a block already lies inside the destination (in-place all-gather,
-  // flagcx/include/flagcx.h:373), which the list copy refuses; then block by block,
-  // where a copy onto itself is nothing.
+  // m blocks of `n` bytes from the pointers in `src` into dst, back to back.  The blocks join
+  // the waiting copies: an all-gather hands every block to every member, and copies of one
+  // source go out with one read of it (flushCopies); a block that already lies at its place
+  // (in-place all-gather, flagcx/include/flagcx.h:373) is a copy onto itself, i.e. nothing.
   flagcxResult_t gather(char *dst, const std::vector<const void *> &src, size_t n) {
-    const int m = (int)src.size();
-    if (!n || !m) return flagcxSuccess;
-    bool single = m <= 64;
-    for (int j = 0; j < m && single; j++) {
-      const char *s = (const char *)src[j];
-      single = !(s < dst + (size_t)m * n && dst < s + n);
-      if (fused && zeros.touches((uintptr_t)s, (uintptr_t)s + n)) single = false;
-    }
-    if (!single) {
-      for (int j = 0; j < m; j++) LCHECK(copy(dst + (size_t)j * n, (const char *)src[j], n));
-      return flagcxSuccess;
-    }
-    if (fused) zeros.remove((uintptr_t)dst, (uintptr_t)dst + (size_t)m * n);
-    LCHECK(flushCopies());
-    bytes += 2 * (uint64_t)m * n;
-    launches++;
-    return flagcxLocalPackList(dst, src.data(), m, n, stream);
+    for (size_t j = 0; j < src.size(); j++) LCHECK(copy(dst + j * n, (const char *)src[j], n));
+    return flagcxSuccess;
   }
 
   // Zeros that are due in [b, e) are written now.
