@@ -648,7 +648,9 @@ flagcxResult_t flagcxLocalStagedReduceScatterNoAlloc(const void *const *sendbuff
  * commOp 12 (LocCpy) and 13 (LocRed), reserved by the reference's plan DSL
  * (flagcx/tools/utils.py:43-44), are rank-local copy and
  * recv = OP(send, recv).  Host-side errors of a plan are reported through
- * flagcxLocalPlanGetLastError. */
+ * flagcxLocalPlanGetLastError.  A plan object belongs to one thread at a time (its
+ * error text and traffic figures are per object); different plans may be used from
+ * different threads at once. */
 typedef struct flagcxLocalPlan *flagcxLocalPlan_t;
 
 /* clusterIds[r]: cluster of global rank r (0-based, dense).  isInterRank[r] != 0:
