@@ -624,6 +624,39 @@ def config_plan_replay(L, mib=128, iters=10, only=None, modes=(False, True)):
     return rows
 
 
+def config_fanout(L, mib=256, ndst=4):
+    """One source to `ndst` destinations (a broadcast inside a simulated cluster): flagcxLocalCopyFanout reads
+    the source once, (1 + n) bytes per payload byte; beside it the same copies as one batch launch, 2 n."""
+    import torch
+    rows = {}
+    try:
+        n = mib * MiB
+        sets = []
+        for _ in range(2):
+            src = torch.empty(n, dtype=torch.uint8, device="cuda")
+            src.random_(0, 255)
+            sets.append((src, [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(ndst)]))
+
+        def fan(i):
+            s, d = sets[i]
+            L.copy_fanout([(s.data_ptr(), [x.data_ptr() for x in d], n)])
+
+        def one_by_one(i):
+            s, d = sets[i]
+            L.reduce_batch([([s.data_ptr()], x.data_ptr(), n) for x in d], L.RedOp.Sum, L.DataType.Uint8, 1)
+        ms_f = timed_sets_ms(fan, 2, warmup=4, iters=20)
+        ok = all(torch.equal(sets[0][0], x) for x in sets[0][1])
+        ms_c = timed_sets_ms(one_by_one, 2, warmup=4, iters=20)
+        rows["fanout_1_to_%d_%dMiB" % (ndst, mib)] = row((1 + ndst) * n, ms_f, destinations_equal_source=bool(ok),
+                                                        speedup_over_separate_copies=round(ms_c / ms_f, 3))
+        rows["copies_%dx_%dMiB_one_batch" % (ndst, mib)] = row(2 * ndst * n, ms_c)
+        del sets
+        torch.cuda.empty_cache()
+    except Exception as e:
+        rows["fanout_error"] = repr(e)
+    return rows
+
+
 def plan_replay_small(L, sizes_kib=(64, 1024, 8192), iters=50):
     """Small collectives are bound by the launches of a replay, not by bytes.  flagcxLocalPlanExecute
     only launches kernels, so one Execute captured into a HIP graph stands for every later one with
@@ -807,6 +840,7 @@ def table_configs(L, args):
     rows.update(config_c1(L, args.allocator_layout)[0])
     rows.update(config_c3(L, full=True, separate=args.allocator_layout))
     rows.update(config_c4(L, args.allocator_layout))
+    rows.update(config_fanout(L))
     rows.update(config_plan_replay(L))
     for name, r in rows.items():
         if not isinstance(r, dict) or "bytes" not in r:
@@ -1211,7 +1245,7 @@ def main():
         cfg.update(variants or {})
         for name, fn in (("C3", lambda: config_c3(L, full=False, separate=args.allocator_layout)),
                          ("C4", lambda: config_c4(L, args.allocator_layout)), ("C5", lambda: config_c5(L)),
-                         ("plan", lambda: config_plan_replay(L))):
+                         ("fanout", lambda: config_fanout(L)), ("plan", lambda: config_plan_replay(L))):
             try:
                 cfg.update(fn())
             except Exception as e:
