@@ -1,0 +1,139 @@
+"""The plan executor's host logic on the CPU.  flagcx_amd/csrc/host_c2c_local.cpp is plain C++ over eight
+C-ABI entry points; here it is compiled with AddressSanitizer and UBSan against a test double of those
+entry points that works on host memory (tests/plan_host_harness/device_double.cpp) and replays
+  - the DSL-written fixtures under tests/golden/plans, and
+  - the seeded random two-cluster plans of tests/test_plan_random_gpu.py,
+fused and literally, against the numpy model of flagcxC2cPlanner::execute.  Every buffer is a heap block of
+exactly its size, so an access of the executor past an end aborts the run, and the double aborts when
+operations it is told to run concurrently are not independent.  The double is test infrastructure: the
+library never links it."""
+import os
+import random
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import c2c_plan_model as M
+from tests import test_plan_random_gpu as R
+from tests.test_plan_fixtures import CL4, CL8, fixture
+from tests.test_plan_fused_gpu import special_values
+from oracle import cpu_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HARNESS_DIR = os.path.join(ROOT, "tests", "plan_host_harness")
+SOURCES = [os.path.join(HARNESS_DIR, "harness.cpp"), os.path.join(HARNESS_DIR, "device_double.cpp"),
+           os.path.join(ROOT, "flagcx_amd", "csrc", "host_c2c_local.cpp")]
+
+
+@pytest.fixture(scope="module")
+def harness(tmp_path_factory):
+    gxx = shutil.which("g++")
+    if not gxx:
+        pytest.skip("no g++")
+    exe = str(tmp_path_factory.mktemp("plan_harness") / "harness")
+    cmd = [gxx, "-O0", "-g", "-std=c++17", "-w", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+           "-fno-omit-frame-pointer"] + SOURCES + ["-o", exe]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return exe
+
+
+def run_cases(harness, tmp_path, cases):
+    """cases: dicts with prefix, clusters, n, chunks, commop, redop, algo, fused, dt, root, scratch, hosts.
+    Returns per case (status, message, recv arrays, send arrays)."""
+    lines = []
+    for i, c in enumerate(cases):
+        d = tmp_path / ("case%d" % i)
+        d.mkdir()
+        for r, h in enumerate(c["hosts"]):
+            h.tofile(str(d / ("in_%d.bin" % r)))
+        lines.append(" ".join(str(x) for x in [c["prefix"], len(c["clusters"])] + list(c["clusters"]) +
+                              [c["n"], c["chunks"], c["commop"], c["redop"], c["algo"], int(c["fused"]), c["dt"], c["root"],
+                               int(c["scratch"]), d, d]))
+    man = tmp_path / "manifest.txt"
+    man.write_text("\n".join(lines) + "\n")
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=1", UBSAN_OPTIONS="print_stacktrace=1")
+    r = subprocess.run([harness, str(man)], capture_output=True, text=True, timeout=900, env=env)
+    assert r.returncode == 0, (r.returncode, r.stdout[-500:], r.stderr[-3000:])
+    out = []
+    for i, c in enumerate(cases):
+        d = tmp_path / ("case%d" % i)
+        status, _, msg = (d / "status.txt").read_text().strip().partition(" ")
+        npdt = c["hosts"][0].dtype
+        out.append((int(status), msg, [np.fromfile(str(d / ("out_%d.bin" % r)), dtype=npdt) for r in range(len(c["clusters"]))],
+                    [np.fromfile(str(d / ("send_%d.bin" % r)), dtype=npdt) for r in range(len(c["clusters"]))]))
+    return out
+
+
+def model_recv(c):
+    nr, n, npdt = len(c["clusters"]), c["n"], c["hosts"][0].dtype
+    m = M.Model(c["prefix"], c["clusters"], n, c["commop"], c["redop"], default_chunks=c["chunks"] or None)
+    recv = [np.frombuffer(bytes([0x55]) * (n * npdt.itemsize), dtype=npdt).copy() for _ in range(nr)]
+    scr = [np.frombuffer(bytes([0x33]) * (n * npdt.itemsize), dtype=npdt).copy() for _ in range(nr)] if c["scratch"] else None
+    with np.errstate(over="ignore"):
+        m.execute([h.copy() for h in c["hosts"]], recv, scr, root=c["root"], algorithm=c["algo"])
+    return recv
+
+
+def same_bits(a, b):
+    return a.shape == b.shape and a.tobytes() == b.tobytes()
+
+
+def test_fixtures_replay_like_the_model_on_the_cpu(harness, tmp_path):
+    cases = []
+    for name, clusters, commop, chunks, scratch, root in (("allreduce8", CL8, 6, 8, False, -1), ("reducescatter8", CL8, 8, 8, True, -1),
+                                                           ("reduce8", CL8, 5, 8, False, 6), ("gather4", CL4, 3, 4, True, 3),
+                                                           ("uneven4", CL4, 6, 4, False, -1), ("allgather4", CL4, 7, 4, False, -1)):
+        for algo in (0, 1, 2):
+            for fused in (True, False):
+                n = chunks * 613
+                rng = np.random.default_rng(len(cases))
+                hosts = [rng.integers(-2**27, 2**27, n, dtype=np.int32) for _ in clusters]
+                cases.append(dict(prefix=fixture(name), clusters=clusters, n=n, chunks=chunks, commop=commop, redop=0, algo=algo,
+                                  fused=fused, dt=int(O.INT32), root=root, scratch=scratch, hosts=hosts, name=name))
+    for c, (status, msg, recv, send) in zip(cases, run_cases(harness, tmp_path, cases)):
+        what = (c["name"], c["algo"], c["fused"])
+        assert status == 0, (what, msg)
+        want = model_recv(c)
+        for r in range(len(c["clusters"])):
+            assert same_bits(recv[r], want[r]), (what, r)
+            assert same_bits(send[r], c["hosts"][r]), (what, r)
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_plans_on_the_cpu_fused_literal_and_model_agree(harness, tmp_path, block):
+    """100 seeded random plans per block (other seeds than the GPU test's): int32 fused == literal == model,
+    fp32 full of signed zeros, NaNs and infinities fused == literal (NaNs by bits too: the double folds both
+    replays with the same host arithmetic)."""
+    rnd = random.Random(31000 + block)
+    cases = []
+    for k in range(100):
+        nr = rnd.choice([4, 8])
+        clusters = [0] * (nr // 2) + [1] * (nr // 2)
+        commop = rnd.choice([6, 8])
+        redop = rnd.choice([0, 0, 0, 2, 3])
+        algo = rnd.choice([0, 1, 2])
+        n = R.NCH * rnd.choice([1, 3, 64, 257])
+        prefix = str(tmp_path / ("p%d" % k))
+        R.make_plan(prefix, rnd, nr, commop)
+        rng = np.random.default_rng(1000 * block + k)
+        ints = [rng.integers(-2**20, 2**20, n).astype(np.int32) for _ in range(nr)]
+        flts = [special_values(O.FP32, n, 7000 * block + 10 * k + r) for r in range(nr)]
+        for hosts, dt in ((ints, int(O.INT32)), (flts, int(O.FP32))):
+            for fused in (True, False):
+                cases.append(dict(prefix=prefix, clusters=clusters, n=n, chunks=0, commop=commop, redop=redop, algo=algo,
+                                  fused=fused, dt=dt, root=-1, scratch=True, hosts=hosts, k=k))
+    res = run_cases(harness, tmp_path, cases)
+    for i in range(0, len(cases), 4):
+        c = cases[i]
+        what = (block, c["k"], len(c["clusters"]), c["commop"], c["redop"], c["algo"], c["n"])
+        (s0, m0, fi, si), (s1, m1, li, _), (s2, m2, ff, _), (s3, m3, lf, _) = res[i:i + 4]
+        assert (s0, s1, s2, s3) == (0, 0, 0, 0), (what, m0, m1, m2, m3)
+        want = model_recv(c)
+        for r in range(len(c["clusters"])):
+            assert same_bits(fi[r], li[r]), ("int32 fused != literal", what, r)
+            assert same_bits(li[r], want[r]), ("int32 literal != model", what, r)
+            assert same_bits(si[r], c["hosts"][r]), ("send buffer changed", what, r)
+            assert same_bits(ff[r], lf[r]), ("fp32 fused != literal", what, r)
