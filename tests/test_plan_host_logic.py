@@ -102,22 +102,28 @@ def test_fixtures_replay_like_the_model_on_the_cpu(harness, tmp_path):
             assert same_bits(send[r], c["hosts"][r]), (what, r)
 
 
-@pytest.mark.parametrize("block", range(4))
+# more blocks and other seeds for a longer run: FLAGCX_PLAN_FUZZ_BLOCKS=40 FLAGCX_PLAN_FUZZ_SEED=90000 pytest tests/test_plan_host_logic.py
+FUZZ_BLOCKS = int(os.environ.get("FLAGCX_PLAN_FUZZ_BLOCKS", "4"))
+FUZZ_SEED = int(os.environ.get("FLAGCX_PLAN_FUZZ_SEED", "31000"))
+
+
+@pytest.mark.parametrize("block", range(FUZZ_BLOCKS))
 def test_random_plans_on_the_cpu_fused_literal_and_model_agree(harness, tmp_path, block):
     """100 seeded random plans per block (other seeds than the GPU test's): int32 fused == literal == model,
     fp32 full of signed zeros, NaNs and infinities fused == literal (NaNs by bits too: the double folds both
     replays with the same host arithmetic)."""
-    rnd = random.Random(31000 + block)
+    rnd = random.Random(FUZZ_SEED + block)
     cases = []
     for k in range(100):
-        nr = rnd.choice([4, 8])
-        clusters = [0] * (nr // 2) + [1] * (nr // 2)
+        sizes = rnd.choice([(2, 2), (4, 4), (1, 3), (3, 1), (2, 6), (5, 3), (1, 1), (3, 4)])   # clusters of unequal sizes too
+        nr = sum(sizes)
+        clusters = [0] * sizes[0] + [1] * sizes[1]
         commop = rnd.choice([6, 8])
         redop = rnd.choice([0, 0, 0, 2, 3])
         algo = rnd.choice([0, 1, 2])
-        n = R.NCH * rnd.choice([1, 3, 64, 257])
+        n = R.NCH * nr * rnd.choice([1, 3, 40])
         prefix = str(tmp_path / ("p%d" % k))
-        R.make_plan(prefix, rnd, nr, commop)
+        R.make_plan(prefix, rnd, nr, commop, sizes)
         rng = np.random.default_rng(1000 * block + k)
         ints = [rng.integers(-2**20, 2**20, n).astype(np.int32) for _ in range(nr)]
         flts = [special_values(O.FP32, n, 7000 * block + 10 * k + r) for r in range(nr)]

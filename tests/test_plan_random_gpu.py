@@ -89,13 +89,13 @@ def homo_for_cluster(rnd, m, allow_scratch):
     return None
 
 
-def hetero_step(rnd, nr, m):
+def hetero_step(rnd, nr, cluster_of):
     """One hetero function per rank: a few transfers between the clusters; on every rank the
     ranges it receives into are disjoint from each other and from the ranges it sends."""
     ops = [[] for _ in range(nr)]
     for _ in range(rnd.randint(0, nr)):
         a = rnd.randrange(nr)
-        b = rnd.choice([r for r in range(nr) if r // m != a // m])
+        b = rnd.choice([r for r in range(nr) if cluster_of[r] != cluster_of[a]])
         cnt = rnd.randint(1, 4)
         so, ro = rnd.randint(0, NCH - cnt), rnd.randint(0, NCH - cnt)
         # nothing may be received into a range that the same rank receives into or sends from in this function
@@ -113,9 +113,12 @@ def hetero_step(rnd, nr, m):
 recv_ranges, send_ranges = {}, {}
 
 
-def make_plan(prefix, rnd, nr, commop):
+def make_plan(prefix, rnd, nr, commop, sizes=None):
+    """Writes <prefix>_<rank>.xml for nr ranks in two clusters of sizes[0] and sizes[1] ranks (halves by default)."""
     global recv_ranges, send_ranges
-    m = nr // 2
+    sizes = sizes or (nr // 2, nr // 2)
+    first = (0, sizes[0])
+    cluster_of = [0] * sizes[0] + [1] * sizes[1]
     shape = rnd.choice([(1, 0, 1, 0, 1), (1, 0, 1, 1, 1), (0, 1, 1, 0, 1), (1, 0, 2, 0, 1)])
     n_pre, n_het, n_post = shape[0] + shape[1], shape[1] + shape[2] + shape[3], shape[3] + shape[4]
     allow_scratch = True
@@ -125,11 +128,11 @@ def make_plan(prefix, rnd, nr, commop):
         for s in range(nsteps):
             for cl in range(2):
                 for _ in range(rnd.randint(0, maxfuncs)):
-                    fs = homo_for_cluster(rnd, m, allow_scratch)
+                    fs = homo_for_cluster(rnd, sizes[cl], allow_scratch)
                     if fs is None:
                         continue
-                    for h in range(m):
-                        per_rank[cl * m + h][s].append(fs[h])
+                    for h in range(sizes[cl]):
+                        per_rank[first[cl] + h][s].append(fs[h])
         return per_rank
 
     pre, post = homo_steps(n_pre, 2), homo_steps(n_post, 2)
@@ -137,21 +140,22 @@ def make_plan(prefix, rnd, nr, commop):
     inter = [[[] for _ in range(n_het)] for _ in range(nr)]
     for s in range(n_het):
         recv_ranges, send_ranges = {}, {}
-        ops = hetero_step(rnd, nr, m)
+        ops = hetero_step(rnd, nr, cluster_of)
         for r in range(nr):
             het[r][s] = [ops[r]]                           # one hetero function per rank and step, maybe without ops
         for cl in range(2):
             if rnd.random() < 0.7:
-                fs = homo_for_cluster(rnd, m, allow_scratch)
+                fs = homo_for_cluster(rnd, sizes[cl], allow_scratch)
                 if fs is not None:
-                    for h in range(m):
+                    for h in range(sizes[cl]):
                         fs[h]["homoType"] = 2
-                        inter[cl * m + h][s].append(fs[h])
+                        inter[first[cl] + h][s].append(fs[h])
     for r in range(nr):
         bufftype = rnd.choice([1, 2, -1])
         # buffType -1 under the pipeline algorithm starts at the cluster's part (c2c_algo.cc:2159-2163),
-        # chunk NCH/2 for the second cluster: the window has to fit behind it
-        total = rnd.randint(1, NCH // 2 if bufftype == -1 else NCH)
+        # chunk sizes[0] * NCH / nr for the second cluster: the window has to fit behind it
+        behind = NCH - (sizes[0] * NCH + nr - 1) // nr
+        total = rnd.randint(1, min(NCH // 2, behind) if bufftype == -1 else NCH)
         start = rnd.randint(0, NCH - total)
         off = rnd.randint(0, total)
         cnt = rnd.randint(0, total - off)
