@@ -186,16 +186,17 @@ def replay(prefix, clusters, n, commop, redop, hosts, dt, algo, fused):
 def test_random_plans_fused_literal_and_model_agree(tmp_path, block):
     rnd = random.Random(9000 + block)
     for case in range(25):
-        nr = rnd.choice([4, 8])
-        clusters = [0] * (nr // 2) + [1] * (nr // 2)
+        sizes = rnd.choice([(2, 2), (4, 4), (2, 2), (4, 4), (1, 3), (2, 6), (5, 3), (3, 4)])   # unequal clusters too
+        nr = sum(sizes)
+        clusters = [0] * sizes[0] + [1] * sizes[1]
         commop = rnd.choice([6, 8])                        # all-reduce: staging in recv; reduce-scatter: in scratch
         redop = rnd.choice([local.RedOp.Sum, local.RedOp.Sum, local.RedOp.Sum, local.RedOp.Max, local.RedOp.Min])
         algo = rnd.choice([0, 1, 2])
         c = rnd.choice([1, 3, 64, 1000, 4099])
         n = NCH * c
         prefix = str(tmp_path / ("p%d_%d" % (block, case)))
-        make_plan(prefix, rnd, nr, commop)
-        tag = (block, case, nr, commop, int(redop), algo, c)
+        make_plan(prefix, rnd, nr, commop, sizes)
+        tag = (block, case, sizes, commop, int(redop), algo, c)
         # int32: literal == fused == model
         rng = np.random.default_rng(100 * block + case)
         hosts = [rng.integers(-2**20, 2**20, n).astype(np.int32) for _ in range(nr)]
