@@ -6,7 +6,7 @@
 // the collectives run over `nranks` simulated ranks whose buffers all live on this
 // GPU.  Unlike the reference's strcmp, results are compared in full.
 //
-//   local_coll_test [-n nranks] [-c count_per_rank]      exit code 0 = all passed
+//   local_coll_test [-n nranks (3 or more)] [-c count_per_rank]      exit code 0 = all passed
 #include "../../include/flagcx_amd_adaptor.h"
 
 #include <cstdio>
@@ -37,7 +37,7 @@ int main(int argc, char **argv) {
     if (!strcmp(argv[i], "-n")) nranks = atoi(argv[i + 1]);
     if (!strcmp(argv[i], "-c")) count = strtoull(argv[i + 1], 0, 0);
   }
-  if (nranks < 1 || nranks > FLAGCX_LOCAL_MAX_RANKS || count % (size_t)nranks) return 2;
+  if (nranks < 3 || nranks > FLAGCX_LOCAL_MAX_RANKS || count % (size_t)nranks) return 2; // the checks use ranks 0, 1 and 2
   struct flagcxDeviceAdaptor *dev = flagcxLocalGetDeviceAdaptor();
   const size_t size = count * sizeof(float);
   flagcxStream_t stream;
@@ -102,6 +102,22 @@ int main(int argc, char **argv) {
   OK(dev->deviceMemcpy(hostrecv, recvbuff[nranks - 1], size, flagcxMemcpyDeviceToHost, stream, NULL));
   OK(dev->streamSynchronize(stream));
   EXPECT(memcmp(hostsend, hostrecv, size) == 0, "Broadcast of float(i) to the last rank");
+
+  // ---- Broadcast as one call: the root's buffer read once, stored to every other rank
+  for (int r = 0; r < nranks; r++) OK(dev->deviceMemset(recvbuff[r], 0, size, flagcxMemDevice, stream));
+  {
+    std::vector<void *> others;
+    for (int r = 1; r < nranks; r++) others.push_back(recvbuff[r]);
+    flagcxLocalFanoutDesc f = {sendbuff[0], others.data(), (int)others.size(), size};
+    OK(flagcxLocalCopyFanout(&f, 1, stream));
+    bool all = true;
+    for (int r = 1; r < nranks; r++) {
+      OK(dev->deviceMemcpy(hostrecv, recvbuff[r], size, flagcxMemcpyDeviceToHost, stream, NULL));
+      OK(dev->streamSynchronize(stream));
+      all = all && memcmp(hostsend, hostrecv, size) == 0;
+    }
+    EXPECT(all, "Broadcast of float(i) to every other rank with one read of the root's buffer");
+  }
 
   // ---- Self send/recv byte pattern (test/perf/test_core_sendrecv.cpp:80-94)
   unsigned char *hb = static_cast<unsigned char *>(hostsend);

@@ -170,4 +170,4 @@ def test_cpp_collective_test_program():
     assert os.path.exists(exe), "build it with python -m flagcx_amd.build"
     r = subprocess.run([exe, "-n", "8", "-c", str(1 << 22)], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert "PASSED" in r.stdout and r.stdout.count("ok ") == 6
+    assert "PASSED" in r.stdout and r.stdout.count("ok ") == 7
