@@ -868,6 +868,41 @@ def table_plan(L, args):
             print("%-32s %s" % (name, "  ".join("%s=%s" % kv for kv in r.items() if kv[0] != "note")), flush=True)
 
 
+def table_fanout(L, args):
+    """flagcxLocalCopyFanout, one source of --mib MiB to n destinations, beside the same n copies as one batch
+    launch; rotating buffer sets.  --once: one fan-out launch per n and nothing else (for counter runs)."""
+    import torch
+    n = args.mib * MiB
+    print("one source of %d MiB to n destinations; GB/s of (1 + n) x size (fan-out) and of 2 n x size (batch of copies)" % args.mib,
+          flush=True)
+    for nd in (1, 2, 3, 4, 6, 8):
+        sets = []
+        for _ in range(1 if args.once else 3):
+            src = torch.empty(n, dtype=torch.uint8, device="cuda")
+            src.random_(0, 255)
+            sets.append((src, [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(nd)]))
+
+        def fan(i):
+            s, d = sets[i]
+            L.copy_fanout([(s.data_ptr(), [x.data_ptr() for x in d], n)])
+
+        def one_by_one(i):
+            s, d = sets[i]
+            L.reduce_batch([([s.data_ptr()], x.data_ptr(), n) for x in d], L.RedOp.Sum, L.DataType.Uint8, 1)
+        if args.once:
+            fan(0)
+            torch.cuda.synchronize()
+            print("  1 -> %d launched once" % nd, flush=True)
+        else:
+            ms_f = timed_sets_ms(fan, 3, warmup=6, iters=18)
+            ms_c = timed_sets_ms(one_by_one, 3, warmup=6, iters=18)
+            print("  1 -> %d   fan-out %8.4f ms %7.0f GB/s %5.1f %%    batch of copies %8.4f ms %7.0f GB/s %5.1f %%    %.2f x"
+                  % (nd, ms_f, (1 + nd) * n / ms_f / 1e6, (1 + nd) * n / ms_f / 1e6 / 80, ms_c, 2 * nd * n / ms_c / 1e6,
+                     2 * nd * n / ms_c / 1e6 / 80, ms_c / ms_f), flush=True)
+        del sets
+        torch.cuda.empty_cache()
+
+
 def table_dtypes(L, args):
     import torch
     lib = L.lib()
@@ -1018,7 +1053,7 @@ def main():
     ap.add_argument("--plan-name", default=None, help="plan table: allreduce8 or reducescatter8 (default both)")
     ap.add_argument("--plan-mode", default="both", choices=["literal", "fused", "both"], help="plan table: which replay")
     ap.add_argument("--plan-iters", type=int, default=10, help="plan table: timed replays per row")
-    ap.add_argument("--table", choices=["sweep", "sweep-rotate", "configs", "dtypes", "stride", "positions", "plan"],
+    ap.add_argument("--table", choices=["sweep", "sweep-rotate", "configs", "dtypes", "stride", "positions", "plan", "fanout"],
                     help="print one of the tables instead of the JSON line")
     ap.add_argument("--min", type=int, default=1 << 10, help="sweep tables: smallest size")
     ap.add_argument("--max", type=int, default=1 << 30, help="sweep tables: largest size")
@@ -1044,7 +1079,7 @@ def main():
 
     if args.table:
         {"sweep": table_sweep, "sweep-rotate": table_sweep, "configs": table_configs, "dtypes": table_dtypes,
-         "stride": table_stride, "positions": table_positions, "plan": table_plan}[args.table](L, args)
+         "stride": table_stride, "positions": table_positions, "plan": table_plan, "fanout": table_fanout}[args.table](L, args)
         return
 
     # The 8 input buffers and the output live in one allocation, at the addresses
