@@ -399,8 +399,8 @@ int launchFanout(const FanoutCall *calls, int n, hipStream_t stream) {
     // destinations, TB/s of (1 + n) x 256 MiB: no cap 6.43 / 6.18 / 5.93 / 5.91 / 5.79 / 5.52,
     // 25 per CU 6.43 / 6.19 / 6.17 / 6.09 / 5.97 / 5.58, 21: - / 6.20 / 6.08 / 6.15 / 6.11 / 6.00,
     // 16: 5.88 / 5.95 / 6.03 / 6.05 / 5.99 / 5.99 (workgroups of two wavefronts the same, of
-    // four 0.3-0.5 lower; the same copies one by one: 6.65 of 2 n x 256 MiB, i.e. 1.3-1.5 x
-    // the time).
+    // four 0.3-0.5 lower; 2 or 4 KiB per wavefront 0.1-0.9 lower under every cap; the same
+    // copies one by one: 6.65 of 2 n x 256 MiB, i.e. 1.3-1.55 x the time).
     const int lds = ldsReservation(maxDst >= 3 ? 21 : 0);
     fanoutWaveKernel<<<dim3((unsigned)maxTiles, (unsigned)m), dim3(64), lds, stream>>>(p);
     const int e = (int)hipGetLastError();
