@@ -74,11 +74,21 @@ static Split splitFor(const ReduceCall &c) {
 // the 128-byte cache line, and a KiB tile that does not start on a line shares its first
 // and last line with its neighbours, which run on other XCDs: such a stream costs an
 // extra line fetch (or a partial line write) per KiB.  The first tile is cut short by
-// `lead` bytes so that all later tiles start on a line of as many of the K + 1 streams as
-// possible (the destination counts double: a straddling store stream costs more than a
-// straddling load stream).  Measured, 256 MiB bf16 per input, percent of peak: every
-// buffer 16 or 64 bytes into a line 68 / 74-77 -> 83-85 (as with line-aligned buffers);
-// sources 80 and destination 16 bytes into a line 66-70 -> 78.
+// `lead` bytes so that all later tiles start on a line of the streams that it pays most
+// to have there.  What a stream that straddles costs, fitted to measurements (256 MiB bf16
+// per input, percent of peak, tiles on the sources' lines / on the destination's, sources
+// 16 bytes into their lines and the destination on one: 2 inputs 77.5 / 83.2, 3: 77.5 /
+// 81.5, 4: 78.9 / 82.9, 5: 76.7 / 80.7, 6: 78.2 / 79.2, 7: 78.1 / 79.1, 8: 77.1 / 76.4;
+// at 64 MiB per input 6 and 8 inputs: 82-83 / 77): a straddling load stream 1, a
+// straddling store stream 5.5 - unless it straddles by exactly half a line (sources 80
+// and destination 16 bytes in: 83-85 on the sources' lines for every input count, 80-83
+// on the destination's), where whole 64-byte halves are still written: 0.5.  So up to
+// five sources follow the destination and six or more outvote it.  Under 96 MiB per input
+// it is the other way round (64 MiB, 3 / 5 inputs: 83-84 on the sources' lines, 80-81 on
+// the destination's; 128 MiB: 78 / 78-79 against 80 / 80-81) and the destination counts
+// as two sources, so two or more sources that agree outvote it.  Every buffer 16 or 64
+// bytes into a line: 68 / 74-77 without the short first tile, 83-85 with it (as with
+// line-aligned buffers).
 // Sources that still straddle get runs of kLineRun consecutive tiles per XCD, so that a
 // shared line is fetched into one L2 once (+1 to +3 points; with only the destination
 // straddling the runs cost 2 to 6 points and are not used, as they cost 4 with every
@@ -91,12 +101,17 @@ static void setTiling(ReduceParams<K> &p, const ReduceCall &c, const Split &s) {
   for (int j = 0; j < K; j++) off[j] = (uint32_t)(((uintptr_t)c.src[j] + headBytes) & 127u);
   off[K] = (uint32_t)(((uintptr_t)c.dst + headBytes) & 127u);
   uint32_t best = off[K];
-  int bestScore = -1;
-  for (int i = 0; i <= K; i++) {
-    int score = 0;
-    for (int j = 0; j <= K; j++) score += off[j] == off[i] ? (j == K ? 2 : 1) : 0;
-    if (score > bestScore) {
-      bestScore = score;
+  int bestCost = 1 << 30;
+  // launches of under 96 MiB per input run few rounds of wavefronts and do better on the sources'
+  // lines: there the destination counts as two sources
+  const int storeCost = s.nvec >= (96ull << 20) / 16 ? 11 : 4;
+  for (int i = K; i >= 0; i--) { // the destination's own offset first: it wins ties
+    int cost = 0; // in halves of a straddling load stream
+    for (int j = 0; j < K; j++) cost += off[j] != off[i] ? 2 : 0;
+    const uint32_t apart = (off[K] - off[i]) & 127u;
+    cost += apart == 0 ? 0 : apart == 64 && storeCost > 4 ? 1 : storeCost;
+    if (cost < bestCost) {
+      bestCost = cost;
       best = off[i];
     }
   }
