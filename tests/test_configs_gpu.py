@@ -333,3 +333,29 @@ def test_more_tiles_than_the_largest_grid(L):
     wrong = sum(int((out[i:min(i + (1 << 30), 16 + n)] != 0x5A).sum()) for i in range(16, 16 + n, 1 << 30))
     before, after = int(out[:16].sum()), int(out[16 + n:].sum())
     assert (wrong, before, after) == (0, 0, 0)
+
+
+@pytest.mark.parametrize("k,src_in,dst_in", [(2, 16, 0), (5, 0, 48), (5, 80, 16), (6, 16, 0), (3, 112, 64)])
+def test_large_inputs_at_other_places_inside_their_cache_lines_than_the_output(L, k, src_in, dst_in):
+    """Inputs of 96 MiB and more whose buffers agree modulo 16 bytes but sit at other places inside their
+    128-byte cache lines than the output: from that size on the tiles follow the output's lines for up to five
+    inputs (a straddling store stream costs more than five straddling load streams) and the inputs' lines for
+    more, and the first tile is cut short accordingly.  int32 sums against torch (both wrap), bit for bit,
+    with a ragged tail and guard elements on both sides of the output."""
+    import torch
+    n = (100 << 20) // 4 + 1237                       # a little over 100 MiB of int32, ragged
+    pad = 64
+    g = torch.Generator(device="cuda").manual_seed(100 * k + src_in + dst_in)
+    raws = [torch.randint(-2**31, 2**31 - 1, (n + pad,), generator=g, device="cuda", dtype=torch.int32) for _ in range(k)]
+    out = torch.full((n + pad,), 0x5A5A5A5A, dtype=torch.int32, device="cuda")
+    so, do = src_in // 4, dst_in // 4
+    srcs = [r[so:so + n] for r in raws]
+    assert all(s.data_ptr() % 128 == src_in for s in srcs) and (out.data_ptr() + dst_in) % 128 == dst_in
+    L.reduce(srcs, out[do:do + n], L.RedOp.Sum)
+    torch.cuda.synchronize()
+    want = srcs[0].clone()
+    for s in srcs[1:]:
+        want += s                                      # int32 addition wraps in torch as in the kernel
+    ok = torch.equal(out[do:do + n], want)
+    guards = bool((out[:do] == 0x5A5A5A5A).all()) and bool((out[do + n:] == 0x5A5A5A5A).all())
+    assert ok and guards, (k, src_in, dst_in)
