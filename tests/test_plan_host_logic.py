@@ -146,3 +146,48 @@ def test_random_plans_on_the_cpu_fused_literal_and_model_agree(harness, tmp_path
             assert same_bits(li[r], want[r]), ("int32 literal != model", what, r)
             assert same_bits(si[r], c["hosts"][r]), ("send buffer changed", what, r)
             assert same_bits(ff[r], lf[r]), ("fp32 fused != literal", what, r)
+
+
+def test_hand_written_plans_on_the_cpu(harness, tmp_path):
+    """The hand-written plans of the GPU tests through the same harness: the 2 x 2 all-reduces (local fold and
+    copy, refresh of scratch, the reference's own operations only), every one-cluster block mover for 1..8 ranks
+    and every root, the broadcast from a root in the second cluster, and the Send / Recv homo functions of all
+    three types; each fused and literally, against the model."""
+    from tests import plan_xml as PX
+    from tests.test_plan_fixtures import broadcast_two_clusters, send_recv_plan
+    cases = []
+
+    def add(name, prefix, clusters, n, commop, root=-1, scratch=False, algo=2, chunks=0):
+        rng = np.random.default_rng(len(cases))
+        hosts = [rng.integers(-2**27, 2**27, n, dtype=np.int32) for _ in clusters]
+        for fused in (True, False):
+            cases.append(dict(prefix=prefix, clusters=clusters, n=n, chunks=chunks, commop=commop, redop=0, algo=algo, fused=fused,
+                              dt=int(O.INT32), root=root, scratch=scratch, hosts=hosts, name=name))
+
+    for maker, scratch in ((PX.allreduce_2x2_locred, False), (PX.allreduce_2x2_refresh_scratch, True),
+                           (PX.allreduce_2x2_reference_ops_only, False)):
+        prefix = str(tmp_path / maker.__name__)
+        maker(prefix)
+        for algo in (0, 1, 2):
+            add(maker.__name__, prefix, CL4, 4 * 501, 8 if scratch else 6, scratch=scratch, algo=algo)
+    for commop in (PX.ALLGATHER, PX.GATHER, PX.ALLTOALL, PX.SCATTER, PX.BROADCAST, PX.REDUCE, PX.REDUCESCATTER):
+        for nranks in (1, 2, 3, 5, 8):
+            for root in {0, nranks - 1, nranks // 2}:
+                prefix = str(tmp_path / ("one_%d_%d_%d" % (commop, nranks, root)))
+                PX.one_cluster_collective(prefix, commop, nranks, root)
+                add("one_cluster_%d" % commop, prefix, [0] * nranks, nranks * 77, commop, root=root)
+    for root in (4, 5, 7):
+        prefix = str(tmp_path / ("bc%d" % root))
+        broadcast_two_clusters(prefix, root)
+        add("broadcast_root_%d" % root, prefix, CL8, 4 * 333, 2, root=root)
+    prefix = str(tmp_path / "sr")
+    send_recv_plan(prefix)
+    add("send_recv", prefix, CL4, 6 * 211, 3, root=1, scratch=True)
+
+    for c, (status, msg, recv, send) in zip(cases, run_cases(harness, tmp_path, cases)):
+        what = (c["name"], len(c["clusters"]), c["root"], c["algo"], c["fused"])
+        assert status == 0, (what, msg)
+        want = model_recv(c)
+        for r in range(len(c["clusters"])):
+            assert same_bits(recv[r], want[r]), (what, r)
+            assert same_bits(send[r], c["hosts"][r]), (what, r)
