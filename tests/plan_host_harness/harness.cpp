@@ -2,7 +2,9 @@
 // through device_double.cpp.  Every buffer is a heap block of exactly its size, so a build with
 // AddressSanitizer reports any access past an end.
 // usage: harness <manifest>; one case per line:
-//   prefix nranks c0 .. c{n-1} totalCount chunks commOp redOp algorithm fused dtype root scratch inDir outDir
+//   prefix nranks c0 .. c{n-1} totalCount chunks commOp redOp algorithm fused dtype root scratch inDir outDir [v]
+// with v: 4 * nranks * nranks more numbers follow, the counts and displacements of an AlltoAllv
+// (sendCounts, sDispls, recvCounts, rDispls, row r = rank r's arrays)
 #include "../../include/flagcx_amd.h"
 
 #include <cstdio>
@@ -37,6 +39,12 @@ int main(int argc, char **argv) {
     size_t total, chunks;
     int commOp, redOp, algo, fused, dt, root, useScratch;
     in >> total >> chunks >> commOp >> redOp >> algo >> fused >> dt >> root >> useScratch >> inDir >> outDir;
+    std::string tag;
+    std::vector<size_t> v;
+    if (in >> tag && tag == "v") {
+      v.resize(4 * (size_t)nr * nr);
+      for (auto &x : v) in >> x;
+    }
     const size_t ts = flagcxLocalGetDataTypeSize((flagcxDataType_t)dt), nbytes = total * ts;
     flagcxLocalPlan_t plan = nullptr;
     if (flagcxLocalPlanCreate(&plan, nr, cl.data(), nullptr, total, (flagcxCommOp_t)commOp, (flagcxRedOp_t)redOp) != flagcxSuccess) return 4;
@@ -44,6 +52,10 @@ int main(int argc, char **argv) {
     flagcxResult_t r = flagcxLocalPlanImportXml(plan, prefix.c_str());
     if (r == flagcxSuccess) r = flagcxLocalPlanSetAlgorithm(plan, algo);
     if (r == flagcxSuccess) r = flagcxLocalPlanSetFused(plan, fused);
+    if (r == flagcxSuccess && !v.empty()) {
+      const size_t m = (size_t)nr * nr;
+      r = flagcxLocalPlanSetAlltoAllv(plan, v.data(), v.data() + m, v.data() + 2 * m, v.data() + 3 * m);
+    }
     std::vector<void *> send(nr), recv(nr), scr(nr, nullptr);
     for (int k = 0; k < nr; k++) {
       std::vector<char> h = slurp(inDir + "/in_" + std::to_string(k) + ".bin", nbytes);

@@ -53,7 +53,8 @@ def run_cases(harness, tmp_path, cases):
             h.tofile(str(d / ("in_%d.bin" % r)))
         lines.append(" ".join(str(x) for x in [c["prefix"], len(c["clusters"])] + list(c["clusters"]) +
                               [c["n"], c["chunks"], c["commop"], c["redop"], c["algo"], int(c["fused"]), c["dt"], c["root"],
-                               int(c["scratch"]), d, d]))
+                               int(c["scratch"]), d, d] +
+                              (["v"] + [x for mat in c["v_args"] for row in mat for x in row] if c.get("v_args") else [])))
     man = tmp_path / "manifest.txt"
     man.write_text("\n".join(lines) + "\n")
     # leak detection needs ptrace rights that a sandboxed runner may lack; it was run once by hand (no leak)
@@ -76,7 +77,7 @@ def model_recv(c):
     recv = [np.frombuffer(bytes([0x55]) * (n * npdt.itemsize), dtype=npdt).copy() for _ in range(nr)]
     scr = [np.frombuffer(bytes([0x33]) * (n * npdt.itemsize), dtype=npdt).copy() for _ in range(nr)] if c["scratch"] else None
     with np.errstate(over="ignore"):
-        m.execute([h.copy() for h in c["hosts"]], recv, scr, root=c["root"], algorithm=c["algo"])
+        m.execute([h.copy() for h in c["hosts"]], recv, scr, root=c["root"], algorithm=c["algo"], v_args=c.get("v_args"))
     return recv
 
 
@@ -183,6 +184,12 @@ def test_hand_written_plans_on_the_cpu(harness, tmp_path):
     prefix = str(tmp_path / "sr")
     send_recv_plan(prefix)
     add("send_recv", prefix, CL4, 6 * 211, 3, root=1, scratch=True)
+    # the all-to-all-v fixture: ragged counts and displacements handed over beside the plan
+    from tests.test_plan_fixtures import alltoallv_case
+    n, v, hosts, want = alltoallv_case(37, np.int32, 9)
+    for fused in (True, False):
+        cases.append(dict(prefix=fixture("alltoallv4"), clusters=CL4, n=n, chunks=8, commop=10, redop=0, algo=2, fused=fused,
+                          dt=int(O.INT32), root=-1, scratch=False, hosts=hosts, name="alltoallv4", v_args=v, closed=want))
 
     for c, (status, msg, recv, send) in zip(cases, run_cases(harness, tmp_path, cases)):
         what = (c["name"], len(c["clusters"]), c["root"], c["algo"], c["fused"])
@@ -191,3 +198,5 @@ def test_hand_written_plans_on_the_cpu(harness, tmp_path):
         for r in range(len(c["clusters"])):
             assert same_bits(recv[r], want[r]), (what, r)
             assert same_bits(send[r], c["hosts"][r]), (what, r)
+            if "closed" in c:
+                assert same_bits(recv[r], c["closed"][r]), (what, r, "closed form")
