@@ -212,6 +212,31 @@ static void writeHomoSteps(FILE *f, const char *tag, const std::vector<std::vect
 
 } // namespace
 
+// Temporaries of one Execute (member lists, pending copies, the record of cleared ranges) come
+// from a block that the plan keeps between calls: an allocation is a pointer bump, a release is
+// nothing, and everything goes at once when the call ends.  A replay of a small collective is
+// bound by the host, and some three hundred heap allocations per call were half of its time.
+struct Arena {
+  std::vector<char> block;
+  size_t used = 0;
+  std::vector<void *> overflow; // requests that did not fit: plain heap, freed at reset
+  void *alloc(size_t n, size_t align) {
+    size_t at = (used + align - 1) & ~(align - 1);
+    if (at + n <= block.size()) {
+      used = at + n;
+      return block.data() + at;
+    }
+    void *q = ::operator new(n);
+    overflow.push_back(q);
+    return q;
+  }
+  void reset() {
+    used = 0;
+    for (void *q : overflow) ::operator delete(q);
+    overflow.clear();
+  }
+};
+
 struct flagcxLocalPlan {
   int nranks = 0;
   std::vector<int> clusterOf, isInter;
@@ -228,6 +253,7 @@ struct flagcxLocalPlan {
   bool loaded = false;
   bool fused = true; // flagcxLocalPlanSetFused
   uint64_t lastBytes = 0, lastLaunches = 0; // flagcxLocalPlanGetTraffic
+  Arena arena;                              // temporaries of the Execute in progress
   char err[256] = "";
 };
 
@@ -245,6 +271,33 @@ static flagcxResult_t planFail(flagcxLocalPlan *p, flagcxResult_t code, const ch
     if (r_ != flagcxSuccess) return r_;                                        \
   } while (0)
 
+static thread_local Arena *tlsArena = nullptr; // set for the duration of one flagcxLocalPlanExecute
+
+template <typename T>
+struct ArenaAlloc {
+  typedef T value_type;
+  ArenaAlloc() = default;
+  template <typename U>
+  ArenaAlloc(const ArenaAlloc<U> &) {}
+  T *allocate(size_t n) {
+    if (!tlsArena) return static_cast<T *>(::operator new(n * sizeof(T)));
+    return static_cast<T *>(tlsArena->alloc(n * sizeof(T), alignof(T) < 8 ? 8 : alignof(T)));
+  }
+  void deallocate(T *q, size_t) {
+    if (!tlsArena) ::operator delete(q);
+  }
+  template <typename U>
+  bool operator==(const ArenaAlloc<U> &) const { return true; }
+  template <typename U>
+  bool operator!=(const ArenaAlloc<U> &) const { return false; }
+};
+namespace ex {
+template <typename T>
+using vector = std::vector<T, ArenaAlloc<T>>;
+template <typename K, typename V>
+using map = std::map<K, V, std::less<K>, ArenaAlloc<std::pair<const K, V>>>;
+} // namespace ex
+
 // Byte ranges of device memory that hold zeros by definition but have not been written.
 // The reference assembles a sum across a cluster by clearing, in every member's buffer,
 // all but the member's own slice (flagcxC2cRefreshFunc::run, c2c_algo.cc:586-608) and
@@ -253,7 +306,7 @@ static flagcxResult_t planFail(flagcxLocalPlan *p, flagcxResult_t code, const ch
 // a refresh adds ranges, a write removes them, a copy out of them moves them, a sum leaves
 // out the members that lie in them, and what is left when the plan ends is written then.
 class ZeroSet {
-  std::map<uintptr_t, uintptr_t> r_; // begin -> end: disjoint, never adjacent
+  ex::map<uintptr_t, uintptr_t> r_; // begin -> end: disjoint, never adjacent
  public:
   bool empty() const { return r_.empty(); }
   void add(uintptr_t b, uintptr_t e) {
@@ -301,7 +354,7 @@ class ZeroSet {
     return it->second >= e;
   }
   // where zero ranges begin or end strictly inside (b, e), as offsets from b, ascending
-  void cuts(uintptr_t b, uintptr_t e, std::vector<size_t> &out) const {
+  void cuts(uintptr_t b, uintptr_t e, ex::vector<size_t> &out) const {
     auto it = r_.upper_bound(b);
     if (it != r_.begin()) --it;
     for (; it != r_.end() && it->first < e; ++it) {
@@ -309,15 +362,15 @@ class ZeroSet {
       if (it->second > b && it->second < e) out.push_back(it->second - b);
     }
   }
-  std::vector<std::pair<uintptr_t, uintptr_t>> ranges() const {
-    return std::vector<std::pair<uintptr_t, uintptr_t>>(r_.begin(), r_.end());
+  ex::vector<std::pair<uintptr_t, uintptr_t>> ranges() const {
+    return ex::vector<std::pair<uintptr_t, uintptr_t>>(r_.begin(), r_.end());
   }
 };
 
 // One reduction of a collective: dst = fold of src[0..n) over `count` elements.
 struct Red {
   char *dst;
-  std::vector<const char *> src;
+  ex::vector<const char *> src;
   size_t count;
 };
 
@@ -333,8 +386,8 @@ struct Exec {
   flagcxStream_t stream;
   bool fused;
   ZeroSet zeros;
-  std::vector<char> ownsScratch; // per rank: the reference allocates a scratch buffer for this call (c2c_algo.cc:2122-2129)
-  std::vector<char *> recvTmp, sendTmp;
+  ex::vector<char> ownsScratch; // per rank: the reference allocates a scratch buffer for this call (c2c_algo.cc:2122-2129)
+  ex::vector<char *> recvTmp, sendTmp;
   uint64_t bytes = 0, launches = 0; // algorithmic traffic handed to the kernels
 
   char *pick(int rank, int type) const {
@@ -365,7 +418,7 @@ struct Exec {
     const char *src;
     size_t n;
   };
-  std::vector<Pending> pending;
+  ex::vector<Pending> pending;
   static bool hit(const char *a, size_t an, const char *b, size_t bn) { return a < b + bn && b < a + an; }
 
   flagcxResult_t flushCopies() {
@@ -378,9 +431,9 @@ struct Exec {
       // copies of one source and one length (the sends of a broadcast, a member's block in an
       // all-gather) share one read of it: flagcxLocalCopyFanout; the rest go as one batch
       const size_t np = pending.size();
-      std::vector<int> groupOf(np, -1);
-      std::vector<std::vector<void *>> dsts;
-      std::vector<size_t> first;
+      ex::vector<int> groupOf(np, -1);
+      ex::vector<ex::vector<void *>> dsts;
+      ex::vector<size_t> first;
       for (size_t i = 0; i < np; i++) {
         for (size_t g = 0; g < first.size() && groupOf[i] < 0; g++)
           if (pending[first[g]].src == pending[i].src && pending[first[g]].n == pending[i].n) groupOf[i] = (int)g;
@@ -391,9 +444,9 @@ struct Exec {
         }
         dsts[groupOf[i]].push_back(pending[i].dst);
       }
-      std::vector<flagcxLocalFanoutDesc> fans;
-      std::vector<const void *> src;
-      std::vector<flagcxLocalReduceDesc> descs;
+      ex::vector<flagcxLocalFanoutDesc> fans;
+      ex::vector<const void *> src;
+      ex::vector<flagcxLocalReduceDesc> descs;
       src.reserve(np);
       for (size_t g = 0; g < first.size(); g++) {
         const Pending &c = pending[first[g]];
@@ -451,10 +504,10 @@ struct Exec {
       return memcpyNow(dst, src, n);
     }
     if (d < s + n && s < d + n) return planFail(p, flagcxInvalidArgument, "a copy's buffers overlap%s", "");
-    std::vector<size_t> cut{0};
+    ex::vector<size_t> cut{0};
     zeros.cuts(s, s + n, cut);
     cut.push_back(n);
-    std::vector<char> isZero(cut.size() - 1);
+    ex::vector<char> isZero(cut.size() - 1);
     for (size_t i = 0; i + 1 < cut.size(); i++) isZero[i] = zeros.covers(s + cut[i], s + cut[i + 1]);
     for (size_t i = 0; i + 1 < cut.size(); i++) {
       const size_t at = cut[i], len = cut[i + 1] - cut[i];
@@ -472,7 +525,7 @@ struct Exec {
   // the waiting copies: an all-gather hands every block to every member, and copies of one
   // source go out with one read of it (flushCopies); a block that already lies at its place
   // (in-place all-gather, flagcx/include/flagcx.h:373) is a copy onto itself, i.e. nothing.
-  flagcxResult_t gather(char *dst, const std::vector<const void *> &src, size_t n) {
+  flagcxResult_t gather(char *dst, const ex::vector<const void *> &src, size_t n) {
     for (size_t j = 0; j < src.size(); j++) LCHECK(copy(dst + j * n, (const char *)src[j], n));
     return flagcxSuccess;
   }
@@ -480,7 +533,7 @@ struct Exec {
   // Zeros that are due in [b, e) are written now.
   flagcxResult_t materialize(uintptr_t b, uintptr_t e) {
     if (!fused || !zeros.touches(b, e)) return flagcxSuccess;
-    std::vector<size_t> cut{0};
+    ex::vector<size_t> cut{0};
     zeros.cuts(b, e, cut);
     cut.push_back(e - b);
     for (size_t i = 0; i + 1 < cut.size(); i++)
@@ -489,11 +542,11 @@ struct Exec {
     return flagcxSuccess;
   }
 
-  flagcxResult_t reduceNow(const std::vector<Red> &reds, int nzero) {
+  flagcxResult_t reduceNow(const ex::vector<Red> &reds, int nzero) {
     LCHECK(flushCopies());
     const int nlive = (int)reds[0].src.size();
     const flagcxRedOp_t rop = (flagcxRedOp_t)p->redOp;
-    std::vector<flagcxLocalReduceDesc> descs(reds.size());
+    ex::vector<flagcxLocalReduceDesc> descs(reds.size());
     for (size_t i = 0; i < reds.size(); i++) {
       descs[i] = {(const void *const *)reds[i].src.data(), reds[i].dst, reds[i].count};
       bytes += (uint64_t)(nlive + 1) * reds[i].count * ts;
@@ -508,12 +561,12 @@ struct Exec {
   // whose slice lies in zeros that were never written are not read: a sum over the rest,
   // with +0.0 added once, has the bytes of the sum over all of them (the zero members turn
   // a -0.0 result into +0.0 and change nothing else).
-  flagcxResult_t reduce(const std::vector<Red> &reds) {
+  flagcxResult_t reduce(const ex::vector<Red> &reds) {
     if (reds.empty()) return flagcxSuccess;
     for (auto &r : reds)
       if (r.src.size() != reds[0].src.size()) {
         // clusters of different sizes in one slot: one call per member count
-        std::map<size_t, std::vector<Red>> byCount;
+        ex::map<size_t, ex::vector<Red>> byCount;
         for (auto &q : reds) byCount[q.src.size()].push_back(q);
         for (auto &g : byCount) LCHECK(reduce(g.second));
         return flagcxSuccess;
@@ -537,11 +590,11 @@ struct Exec {
       return reduceNow(reds, 0);
     }
     const int n = (int)reds[0].src.size();
-    std::map<int, std::vector<Red>> byLive; // members read -> pieces (n: no member left out)
-    std::vector<std::pair<uintptr_t, uintptr_t>> written, cleared;
+    ex::map<int, ex::vector<Red>> byLive; // members read -> pieces (n: no member left out)
+    ex::vector<std::pair<uintptr_t, uintptr_t>> written, cleared;
     for (auto &r : reds) {
       const size_t len = r.count * ts;
-      std::vector<size_t> cut{0, len};
+      ex::vector<size_t> cut{0, len};
       for (auto s : r.src) zeros.cuts((uintptr_t)s, (uintptr_t)s + len, cut);
       std::sort(cut.begin(), cut.end());
       cut.erase(std::unique(cut.begin(), cut.end()), cut.end());
@@ -567,7 +620,7 @@ struct Exec {
 
   // No reduction of one group writes what a reduction of another group reads or writes (the
   // groups are collectives of different clusters, or folds local to different ranks).
-  bool independent(const std::vector<std::vector<Red>> &groups) const {
+  bool independent(const ex::vector<ex::vector<Red>> &groups) const {
     for (size_t a = 0; a < groups.size(); a++)
       for (size_t b = 0; b < groups.size(); b++) {
         if (a == b) continue;
@@ -582,11 +635,11 @@ struct Exec {
     return true;
   }
 
-  flagcxResult_t refresh(const std::vector<char> *only);
-  flagcxResult_t homoSlot(const std::vector<const HomoFunc *> &fn);
-  flagcxResult_t sendRecv(int cl, const std::vector<const HomoFunc *> &fn);
+  flagcxResult_t refresh(const ex::vector<char> *only);
+  flagcxResult_t homoSlot(const ex::vector<const HomoFunc *> &fn);
+  flagcxResult_t sendRecv(int cl, const ex::vector<const HomoFunc *> &fn);
   flagcxResult_t homoStep(std::vector<std::vector<HomoFunc>> RankPlan::*table, int s, int onlyIndex = -1,
-                          const std::vector<char> *only = nullptr, bool refreshBeforeEach = false);
+                          const ex::vector<char> *only = nullptr, bool refreshBeforeEach = false);
   flagcxResult_t heteroSlot(int s, int i);
   flagcxResult_t run();
   flagcxResult_t finish();
@@ -595,22 +648,22 @@ struct Exec {
 // One homo function slot (step s, index i of one table) across all ranks; fn[r] is rank
 // r's function or NULL.  The collective's root reaches the functions as a rank of its
 // cluster, globalrank2homorank[root] (c2c_algo.cc:2147,2170).
-flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
+flagcxResult_t Exec::homoSlot(const ex::vector<const HomoFunc *> &fn) {
   const int ncl = (int)p->clusterRanks.size();
   const int root = homoRoot;
   // The clusters run a slot side by side, each on its own ranks' buffers: their reductions go
   // out together (one batch launch per member count instead of one per cluster), and the copies
   // that hand an all-reduce's result to the other members follow them.
-  std::vector<std::vector<Red>> groups; // one per collective (or per rank-local fold)
+  ex::vector<ex::vector<Red>> groups; // one per collective (or per rank-local fold)
   struct After {
     char *dst;
     const char *src;
     size_t n;
   };
-  std::vector<After> after;
+  ex::vector<After> after;
   for (int cl = 0; cl < ncl; cl++) {
     // members that hold a function in this slot; homoType 1 runs on inter-ranks only
-    std::vector<int> mem;
+    ex::vector<int> mem;
     const HomoFunc *first = nullptr;
     for (int r : p->clusterRanks[cl]) {
       const HomoFunc *f = fn[r];
@@ -676,8 +729,8 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
     // the communicator the reference would use: homoInterComm for homoType 1, else homo_comm
     const std::vector<int> &comm = first->homoType_ == 1 ? p->clusterInterRanks[cl] : p->clusterRanks[cl];
     const int n = (int)comm.size();
-    std::vector<char *> S(n, nullptr), D(n, nullptr);
-    std::vector<size_t> cnt(n, 0);
+    ex::vector<char *> S(n, nullptr), D(n, nullptr);
+    ex::vector<size_t> cnt(n, 0);
     for (int h = 0; h < n; h++) {
       const int r = comm[h];
       const HomoFunc *f = fn[r];
@@ -708,7 +761,7 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
           if (!(dRootOnly && h != rt) && !fits(f->recvOffset_, count, dBlocks ? (size_t)n : 1)) return outside(comm[h]);
         }
     }
-    const std::vector<const char *> members(S.begin(), S.end());
+    const ex::vector<const char *> members(S.begin(), S.end());
     switch (op) {
       case flagcxCommOpReduce: {
         const int rt = homoRootOf(first);
@@ -724,7 +777,7 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
       }
       case flagcxCommOpReduceScatter: {
         // member h receives the fold of everybody's h-th block; one batch launch
-        std::vector<Red> reds(n);
+        ex::vector<Red> reds(n);
         for (int h = 0; h < n; h++) {
           reds[h].dst = D[h];
           reds[h].count = count;
@@ -734,14 +787,14 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
         break;
       }
       case flagcxCommOpAllGather: {
-        const std::vector<const void *> blocks(S.begin(), S.end());
+        const ex::vector<const void *> blocks(S.begin(), S.end());
         for (int h = 0; h < n; h++) LCHECK(gather(D[h], blocks, count * ts));
         break;
       }
       case flagcxCommOpGather: {
         const int rt = homoRootOf(first);
         if (rt < 0 || rt >= n) return badRoot(rt);
-        LCHECK(gather(D[rt], std::vector<const void *>(S.begin(), S.end()), count * ts));
+        LCHECK(gather(D[rt], ex::vector<const void *>(S.begin(), S.end()), count * ts));
         break;
       }
       case flagcxCommOpScatter: {
@@ -757,7 +810,7 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
         break;
       }
       case flagcxCommOpAlltoAll: {
-        std::vector<const void *> blocks(n);
+        ex::vector<const void *> blocks(n);
         for (int h = 0; h < n; h++) {
           for (int j = 0; j < n; j++) blocks[j] = S[j] + (size_t)h * count * ts;
           LCHECK(gather(D[h], blocks, count * ts));
@@ -771,7 +824,7 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
     }
   }
   if (groups.size() > 1 && independent(groups)) {
-    std::vector<Red> all;
+    ex::vector<Red> all;
     for (auto &g : groups)
       for (auto &r : g) all.push_back(std::move(r));
     LCHECK(reduce(all));
@@ -786,16 +839,16 @@ flagcxResult_t Exec::homoSlot(const std::vector<const HomoFunc *> &fn) {
 // take part (a rank leaves a loop of the reference when ITS table runs out); with
 // refreshBeforeEach every rank that runs function i refreshes first (c2c_algo.cc:2276-2282).
 flagcxResult_t Exec::homoStep(std::vector<std::vector<HomoFunc>> RankPlan::*table, int s, int onlyIndex,
-                              const std::vector<char> *only, bool refreshBeforeEach) {
+                              const ex::vector<char> *only, bool refreshBeforeEach) {
   size_t width = 0;
   for (auto &rp : p->ranks) {
     auto &t = rp.*table;
     if (s < (int)t.size() && t[s].size() > width) width = t[s].size();
   }
-  std::vector<char> has(p->nranks);
+  ex::vector<char> has(p->nranks);
   for (size_t i = 0; i < width; i++) {
     if (onlyIndex >= 0 && (int)i != onlyIndex) continue;
-    std::vector<const HomoFunc *> fn(p->nranks, nullptr);
+    ex::vector<const HomoFunc *> fn(p->nranks, nullptr);
     bool any = false;
     for (int r = 0; r < p->nranks; r++) {
       auto &t = p->ranks[r].*table;
@@ -813,14 +866,14 @@ flagcxResult_t Exec::homoStep(std::vector<std::vector<HomoFunc>> RankPlan::*tabl
 // Hetero function i of step s on every rank: match each send with the peer's
 // next unmatched receive from that sender (order of appearance).
 flagcxResult_t Exec::heteroSlot(int s, int i) {
-  std::map<std::pair<int, int>, std::vector<const P2pOp *>> recvs; // (receiver, sender) -> ops
+  ex::map<std::pair<int, int>, ex::vector<const P2pOp *>> recvs; // (receiver, sender) -> ops
   for (int r = 0; r < p->nranks; r++) {
     auto &t = p->ranks[r].heteroFuncSteps_;
     if (s >= (int)t.size() || i >= (int)t[s].size()) continue;
     for (auto &op : t[s][i].p2pOps_)
       if (op.isRecv_) recvs[{r, op.peerRank_}].push_back(&op);
   }
-  std::map<std::pair<int, int>, size_t> used;
+  ex::map<std::pair<int, int>, size_t> used;
   for (int r = 0; r < p->nranks; r++) {
     auto &t = p->ranks[r].heteroFuncSteps_;
     if (s >= (int)t.size() || i >= (int)t[s].size()) continue;
@@ -851,7 +904,7 @@ flagcxResult_t Exec::heteroSlot(int s, int i) {
 }
 
 // The refresh function of every rank (only: of the ranks marked).
-flagcxResult_t Exec::refresh(const std::vector<char> *only) {
+flagcxResult_t Exec::refresh(const ex::vector<char> *only) {
   for (int r = 0; r < p->nranks; r++) {
     if (only && !(*only)[r]) continue;
     const RefreshFunc &f = p->ranks[r].refreshFunc_;
@@ -899,7 +952,7 @@ flagcxResult_t Exec::refresh(const std::vector<char> *only) {
 //               clusters, piece by piece at the pieces' own offsets;
 //   homoType 2: inter-rank 0 sends to the root unless it is the root itself.
 // Roots are ranks inside the cluster.
-flagcxResult_t Exec::sendRecv(int cl, const std::vector<const HomoFunc *> &fn) {
+flagcxResult_t Exec::sendRecv(int cl, const ex::vector<const HomoFunc *> &fn) {
   const std::vector<int> &members = p->clusterRanks[cl], &inters = p->clusterInterRanks[cl];
   const int root = homoRoot;
   auto recvOf = [&](int r) -> const HomoFunc * {
@@ -932,7 +985,7 @@ flagcxResult_t Exec::sendRecv(int cl, const std::vector<const HomoFunc *> &fn) {
       char *dst = pick(inters[0], g->recvType_ == 1 ? 1 : 2);
       if (!dst) return needScratch();
       // what rank r received from other clusters: every receive of its hetero functions
-      std::vector<std::pair<size_t, size_t>> pieces;
+      ex::vector<std::pair<size_t, size_t>> pieces;
       for (auto &step : p->ranks[r].heteroFuncSteps_)
         for (auto &h : step)
           for (auto &o : h.p2pOps_) {
@@ -971,7 +1024,7 @@ flagcxResult_t Exec::run() {
   // Every rank walks ITS OWN tables: it runs hetero function i of a step while
   // i < heteroFuncSteps_[s].size() for itself, and behind it homoInter function i if its own
   // homoInterFuncSteps_[s] holds one (c2c_algo.cc:2177-2194,2204-2231,2247-2267).
-  std::vector<char> in(nr), has(nr);
+  ex::vector<char> in(nr), has(nr);
   auto heteroAt = [&](int hs, size_t i) {
     bool any = false;
     for (int r = 0; r < nr; r++) {
@@ -1332,6 +1385,18 @@ flagcxResult_t flagcxLocalPlanExecute(flagcxLocalPlan *p, const void *const *sen
     if (!flagcxLocalGetDataTypeSize(datatype)) return planFail(p, flagcxInvalidArgument, "unsupported data type%s", "");
     for (int r = 0; r < p->nranks; r++)
       if (!sendbuffs[r] || !recvbuffs[r]) return planFail(p, flagcxInvalidArgument, "rank %s%lld has a NULL buffer", "", r);
+    // the call's temporaries: one block, kept by the plan, released as a whole when the call ends
+    // (declared before the executor, so that the executor's containers go first)
+    if (p->arena.block.empty()) p->arena.block.resize(1 << 20);
+    struct Scope {
+      Arena *a;
+      explicit Scope(Arena *arena) : a(arena) { tlsArena = a; }
+      ~Scope() {
+        tlsArena = nullptr;
+        a->reset();
+      }
+    };
+    Scope scope(&p->arena);
     Exec x;
     x.p = p;
     x.send = sendbuffs;
