@@ -11,6 +11,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
 #include <atomic>
 #include <map>
 #include <mutex>
@@ -1036,11 +1037,19 @@ flagcxResult_t flagcxLocalCopyFanout(const flagcxLocalFanoutDesc *descs, int nde
       ranges[nranges++] = {(uintptr_t)d.dsts[j], (uintptr_t)d.dsts[j] + d.bytes, i, true};
     }
   }
-  for (int x = 0; x < nranges; x++)
-    for (int y = 0; y < x; y++)
-      if ((ranges[x].write || ranges[y].write) && ranges[x].b < ranges[y].e && ranges[y].b < ranges[x].e)
-        return fail(flagcxInvalidArgument, "%s: a destination of descs[%d] overlaps a buffer of descs[%d]", who,
-                    ranges[x].write ? ranges[x].desc : ranges[y].desc, ranges[x].write ? ranges[y].desc : ranges[x].desc);
+  // sorted by begin, a range overlaps an earlier one exactly when it begins before the furthest end seen so far:
+  // kept once over all earlier ranges (a destination may overlap nothing) and once over the earlier destinations
+  // (a source may overlap other sources)
+  std::sort(ranges, ranges + nranges, [](const Range &x, const Range &y) { return x.b < y.b; });
+  int furthest = -1, furthestWrite = -1;
+  for (int x = 0; x < nranges; x++) {
+    const int other = ranges[x].write ? furthest : furthestWrite;
+    if (other >= 0 && ranges[x].b < ranges[other].e)
+      return fail(flagcxInvalidArgument, "%s: a destination of descs[%d] overlaps a buffer of descs[%d]", who,
+                  ranges[x].write ? ranges[x].desc : ranges[other].desc, ranges[x].write ? ranges[other].desc : ranges[x].desc);
+    if (furthest < 0 || ranges[x].e > ranges[furthest].e) furthest = x;
+    if (ranges[x].write && (furthestWrite < 0 || ranges[x].e > ranges[furthestWrite].e)) furthestWrite = x;
+  }
   bool work = false;
   for (int x = 0; x < nranges; x++) work = work || ranges[x].write;
   if (!work) return flagcxSuccess;

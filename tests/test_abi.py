@@ -307,6 +307,42 @@ def test_copy_fanout_validates_without_a_device():
     assert call([(base, [base + 4096], 0), (base, [], 100)]) == 0                         # nothing to do
 
 
+def test_copy_fanout_overlap_check_agrees_with_brute_force():
+    """Random sets of copies over made-up addresses: the call is refused exactly when some destination overlaps
+    another buffer of the call (pairwise check here; the library sorts the ranges and sweeps them once).  Accepted
+    sets would go on to launch, so this runs only where there is no GPU to launch on."""
+    import random
+    import torch
+    if torch.cuda.device_count() > 0:
+        pytest.skip("accepted calls would launch on made-up addresses")
+    lib = local.lib()
+    rnd = random.Random(5)
+    base = 0x7e0000000000
+    bad = int(local.Result.InvalidArgument)
+    refused = accepted = 0
+    for case in range(3000):
+        ncopies = rnd.randint(1, 6)
+        copies, ranges = [], []
+        for i in range(ncopies):
+            nbytes = rnd.choice([1, 16, 100, 4096])
+            src = base + rnd.randrange(0, 40) * 1024 + rnd.choice([0, 0, 7])
+            dsts = []
+            for j in range(rnd.randint(1, 4)):
+                d = src if rnd.random() < 0.05 else base + rnd.randrange(0, 40) * 1024 + rnd.choice([0, 0, 50, 1000])
+                dsts.append(d)
+            copies.append((src, dsts, nbytes))
+            ranges.append((src, src + nbytes, False, i))
+            ranges += [(d, d + nbytes, True, i) for d in dsts if d != src]
+        clash = any((a[2] or b[2]) and a[0] < b[1] and b[0] < a[1] for x, a in enumerate(ranges) for b in ranges[:x])
+        keep = [(C.c_void_p * len(c[1]))(*c[1]) for c in copies]
+        arr = (local.FanoutDesc * ncopies)(*[local.FanoutDesc(c[0], keep[i], len(c[1]), c[2]) for i, c in enumerate(copies)])
+        rc = lib.flagcxLocalCopyFanout(arr, ncopies, None)
+        assert (rc == bad) == clash, (case, copies, rc)
+        refused += clash
+        accepted += not clash
+    assert refused > 300 and accepted > 300
+
+
 def test_bench_refuses_more_than_one_gpu():
     """The build runs on one GPU (the k ranks are k HBM buffers on it): bench.py says so and
     exits instead of printing a figure for several, under a launcher that sets WORLD_SIZE too."""
