@@ -44,6 +44,7 @@
 #include <cstring>
 #include <iterator>
 #include <map>
+#include <new>
 #include <string>
 #include <utility>
 #include <vector>
@@ -279,13 +280,12 @@ struct ArenaAlloc {
   ArenaAlloc() = default;
   template <typename U>
   ArenaAlloc(const ArenaAlloc<U> &) {}
+  // containers with this allocator live inside one flagcxLocalPlanExecute and nowhere else
   T *allocate(size_t n) {
-    if (!tlsArena) return static_cast<T *>(::operator new(n * sizeof(T)));
+    if (!tlsArena) throw std::bad_alloc();
     return static_cast<T *>(tlsArena->alloc(n * sizeof(T), alignof(T) < 8 ? 8 : alignof(T)));
   }
-  void deallocate(T *q, size_t) {
-    if (!tlsArena) ::operator delete(q);
-  }
+  void deallocate(T *, size_t) {}
   template <typename U>
   bool operator==(const ArenaAlloc<U> &) const { return true; }
   template <typename U>
